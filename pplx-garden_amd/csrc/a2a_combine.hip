@@ -1,0 +1,270 @@
+// Combine: for every token, gather the K expert-output rows of its routes,
+// weight them, accumulate in float and write one output row in token order.
+//
+// What it replaces: the reference's combine-send kernel (copy of every
+// expert_y row back to the sender's staging buffer, a2a_combine_send.cu:
+// 119-138,182-207) fused with its combine-recv kernel (weighted gather,
+// a2a_combine_recv.cu:94-148).  Here the rows are read in place from the
+// receivers' expert_y buffers, which live in the same HBM: one read per row,
+// no staging write.
+//
+// Design for CDNA4: one workgroup per token; a lane owns 16 bytes of every
+// source row, so K independent 16-byte loads are in flight per lane before the
+// first multiply-add.  Row pointers and weights are resolved once by the
+// first K lanes and read back as wave-uniform scalars (SGPR base + VGPR
+// offset addressing).  Accumulation is an explicit float fused multiply-add
+// chain, k ascending, then one round-to-nearest-even to the output type
+// (combine_utils.cuh:108-114,14-23).
+#include "a2a_internal.h"
+
+namespace a2a {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct Bf16 {};
+struct F16 {};
+struct F32 {};
+
+template <typename T> struct Elem;
+template <> struct Elem<Bf16> { static constexpr int kSize = 2; };
+template <> struct Elem<F16> { static constexpr int kSize = 2; };
+template <> struct Elem<F32> { static constexpr int kSize = 4; };
+
+// Elements per 16-byte source chunk (vector.cuh:14-27: 8 for the 16-bit
+// types, 4 for float).
+template <typename T> constexpr int vec_elems() { return 16 / Elem<T>::kSize; }
+
+template <typename T, int V>
+__device__ __forceinline__ void load_elems(const uint8_t *p, float (&f)[V], bool streaming) {
+    if constexpr (Elem<T>::kSize == 4) {
+        static_assert(V == 4 || V == 8, "");
+#pragma unroll
+        for (int h = 0; h < V / 4; ++h) {
+            const u32x4 *q = reinterpret_cast<const u32x4 *>(p) + h;
+            const u32x4 v = streaming ? __builtin_nontemporal_load(q) : *q;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) f[4 * h + j] = __uint_as_float(v[j]);
+        }
+    } else if constexpr (V == 8) {
+        const u32x4 *q = reinterpret_cast<const u32x4 *>(p);
+        const u32x4 v = streaming ? __builtin_nontemporal_load(q) : *q;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if constexpr (__is_same(T, Bf16)) {
+                f[2 * j] = __uint_as_float(v[j] << 16);
+                f[2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+            } else {
+                f[2 * j] = (float)__builtin_bit_cast(_Float16, (uint16_t)(v[j] & 0xFFFF));
+                f[2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(v[j] >> 16));
+            }
+        }
+    } else {  // V == 4, 16-bit type: 8 bytes
+        const u32x2 *q = reinterpret_cast<const u32x2 *>(p);
+        const u32x2 v = streaming ? __builtin_nontemporal_load(q) : *q;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            if constexpr (__is_same(T, Bf16)) {
+                f[2 * j] = __uint_as_float(v[j] << 16);
+                f[2 * j + 1] = __uint_as_float(v[j] & 0xFFFF0000u);
+            } else {
+                f[2 * j] = (float)__builtin_bit_cast(_Float16, (uint16_t)(v[j] & 0xFFFF));
+                f[2 * j + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(v[j] >> 16));
+            }
+        }
+    }
+}
+
+template <typename U>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+    if constexpr (__is_same(U, Bf16)) {
+        const uint16_t lo = __builtin_bit_cast(uint16_t, (__bf16)a);
+        const uint16_t hi = __builtin_bit_cast(uint16_t, (__bf16)b);
+        return (uint32_t)lo | ((uint32_t)hi << 16);
+    } else {
+        const uint16_t lo = __builtin_bit_cast(uint16_t, (_Float16)a);
+        const uint16_t hi = __builtin_bit_cast(uint16_t, (_Float16)b);
+        return (uint32_t)lo | ((uint32_t)hi << 16);
+    }
+}
+
+template <typename U, int V>
+__device__ __forceinline__ void store_elems(uint8_t *p, const float (&f)[V]) {
+    if constexpr (Elem<U>::kSize == 4) {
+#pragma unroll
+        for (int h = 0; h < V / 4; ++h) {
+            u32x4 v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = __float_as_uint(f[4 * h + j]);
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p) + h);
+        }
+    } else if constexpr (V == 8) {
+        u32x4 v;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) v[j] = pack2<U>(f[2 * j], f[2 * j + 1]);
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(p));
+    } else {
+        u32x2 v;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) v[j] = pack2<U>(f[2 * j], f[2 * j + 1]);
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x2 *>(p));
+    }
+}
+
+__device__ __forceinline__ uint64_t read_lane64c(uint64_t v, uint32_t lane) {
+    const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)v, (int)lane);
+    const uint32_t hi = __builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), (int)lane);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// T: type of the expert_y rows, U: type of out_tokens.  KFIX > 0 unrolls the
+// route loop (all K loads issued before the first use).
+template <typename T, typename U, int KFIX>
+__global__ __launch_bounds__(1024) void combine_gather_kernel(const CombArgs args,
+                                                              const Workspace ws) {
+    constexpr int V = vec_elems<T>();
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const uint32_t E = ws.num_experts;
+    const uint32_t K = KFIX > 0 ? (uint32_t)KFIX : ws.topk;
+
+    uint32_t g = 0;
+    while (g + 1 < ws.world && blockIdx.x >= args.token_start[g + 1]) ++g;
+    const uint32_t token = blockIdx.x - args.token_start[g];
+    const CombDst &dst = args.dst[g];
+    if (token >= effective_tokens(dst.bound_m, dst.num_tokens)) return;
+
+    uint64_t row_ptr = 0;
+    float weight = 0.0f;
+    if (lane < K) {
+        const uint32_t expert = (uint32_t)dst.indices[(size_t)token * dst.indices_stride + lane];
+        weight = dst.weights[(size_t)token * dst.weights_stride + lane];
+        bool ok = false;
+        if (args.staged_base != nullptr) {
+            // a2a_combine_recv.cu:67-73: position = exclusive offset of the expert + token offset.
+            if (expert < E) {
+                const uint32_t excl = expert > 0 ? ws.expert_offsets[g * E + expert - 1] : 0;
+                const uint32_t pos = excl + ws.token_offset[(size_t)g * ws.max_tk + token * K + lane];
+                if (pos < ws.max_tk) {
+                    row_ptr = (uint64_t)(args.staged_base +
+                                         ((size_t)g * ws.max_tk + pos) * args.staged_stride);
+                    ok = true;
+                }
+            }
+        } else if (expert < E) {
+            const uint32_t slot = ws.route_slot[(size_t)g * ws.max_tk + token * K + lane];
+            const CombSrc &src = args.src[expert / ws.experts_per_rank];
+            if (src.y != nullptr && slot < src.y_rows) {
+                row_ptr = (uint64_t)(src.y + (size_t)slot * src.y_stride);
+                ok = true;
+            }
+        }
+        if (!ok && wave == 0) atomicOr(ws.err, A2A_DEV_BAD_SLOT);
+    }
+
+    uint8_t *out_row = dst.out + (size_t)token * dst.out_stride;
+    const uint32_t num_chunks = args.hidden_dim / V;
+
+    if constexpr (KFIX > 0) {
+        uint64_t rows[KFIX];
+        float w[KFIX];
+#pragma unroll
+        for (int k = 0; k < KFIX; ++k) {
+            rows[k] = read_lane64c(row_ptr, k);
+            w[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(weight), k));
+        }
+        for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
+            float y[KFIX][V];
+#pragma unroll
+            for (int k = 0; k < KFIX; ++k) {
+                if (rows[k] != 0) {
+                    load_elems<T, V>(reinterpret_cast<const uint8_t *>(rows[k]) + (size_t)c * 16, y[k],
+                                     true);
+                } else {
+#pragma unroll
+                    for (int j = 0; j < V; ++j) y[k][j] = 0.0f;
+                }
+            }
+            float acc[V];
+            if (args.accumulate) {
+                load_elems<U, V>(out_row + (size_t)c * V * Elem<U>::kSize, acc, false);
+            } else {
+#pragma unroll
+                for (int j = 0; j < V; ++j) acc[j] = 0.0f;
+            }
+#pragma unroll
+            for (int k = 0; k < KFIX; ++k) {
+                if (rows[k] != 0) {
+#pragma unroll
+                    for (int j = 0; j < V; ++j) acc[j] = __builtin_fmaf(w[k], y[k][j], acc[j]);
+                }
+            }
+            store_elems<U, V>(out_row + (size_t)c * V * Elem<U>::kSize, acc);
+        }
+    } else {
+        for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
+            float acc[V];
+            if (args.accumulate) {
+                load_elems<U, V>(out_row + (size_t)c * V * Elem<U>::kSize, acc, false);
+            } else {
+#pragma unroll
+                for (int j = 0; j < V; ++j) acc[j] = 0.0f;
+            }
+            for (uint32_t k = 0; k < K; ++k) {
+                const uint64_t row = read_lane64c(row_ptr, k);
+                const float wk =
+                    __int_as_float(__builtin_amdgcn_readlane(__float_as_int(weight), (int)k));
+                if (row != 0) {
+                    float y[V];
+                    load_elems<T, V>(reinterpret_cast<const uint8_t *>(row) + (size_t)c * 16, y, true);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) acc[j] = __builtin_fmaf(wk, y[j], acc[j]);
+                }
+            }
+            store_elems<U, V>(out_row + (size_t)c * V * Elem<U>::kSize, acc);
+        }
+    }
+}
+
+template <typename T, typename U>
+static hipError_t launch_typed(const CombArgs &args, const Workspace &ws, uint32_t total_tokens,
+                               hipStream_t stream) {
+    constexpr int V = vec_elems<T>();
+    const uint32_t chunks = args.hidden_dim / V;
+    uint32_t threads = (chunks + kWave - 1) / kWave * kWave;
+    // Two chunks per lane once a row is wide enough: more bytes in flight per
+    // wavefront, fewer workgroups to schedule.
+    if (threads > 512) threads = ((chunks + 1) / 2 + kWave - 1) / kWave * kWave;
+    if (threads > 1024) threads = 1024;
+    if (threads < (uint32_t)kWave) threads = kWave;
+    if (ws.topk == 8) {
+        hipLaunchKernelGGL((combine_gather_kernel<T, U, 8>), dim3(total_tokens), dim3(threads), 0,
+                           stream, args, ws);
+    } else {
+        hipLaunchKernelGGL((combine_gather_kernel<T, U, 0>), dim3(total_tokens), dim3(threads), 0,
+                           stream, args, ws);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_combine_gather(const CombArgs &args, const Workspace &ws, uint32_t in_dtype,
+                                 uint32_t out_dtype, uint32_t total_tokens, hipStream_t stream) {
+    if (total_tokens == 0) return hipSuccess;
+#define A2A_COMBINE_CASE(IN_TAG, IN_T, OUT_TAG, OUT_T) \
+    if (in_dtype == IN_TAG && out_dtype == OUT_TAG)    \
+        return launch_typed<IN_T, OUT_T>(args, ws, total_tokens, stream);
+    A2A_COMBINE_CASE(A2A_BF16, Bf16, A2A_BF16, Bf16)
+    A2A_COMBINE_CASE(A2A_BF16, Bf16, A2A_F32, F32)
+    A2A_COMBINE_CASE(A2A_BF16, Bf16, A2A_F16, F16)
+    A2A_COMBINE_CASE(A2A_F16, F16, A2A_F16, F16)
+    A2A_COMBINE_CASE(A2A_F16, F16, A2A_F32, F32)
+    A2A_COMBINE_CASE(A2A_F16, F16, A2A_BF16, Bf16)
+    A2A_COMBINE_CASE(A2A_F32, F32, A2A_F32, F32)
+    A2A_COMBINE_CASE(A2A_F32, F32, A2A_BF16, Bf16)
+    A2A_COMBINE_CASE(A2A_F32, F32, A2A_F16, F16)
+#undef A2A_COMBINE_CASE
+    return hipErrorInvalidValue;
+}
+
+}  // namespace a2a

@@ -1,0 +1,716 @@
+// Host side of the library: the context object and the C ABI.
+//
+// Stands in for the reference's Rust crate `p2p-all-to-all`
+// (p2p-all-to-all/src/a2a_context.rs): it owns the device workspace
+// (DeviceWorkspace, a2a_context.rs:15-97), checks arguments, and turns each
+// call into kernel launches on the caller's stream.  The reference's host
+// worker thread, its GDRCopy flags and RDMA submissions have no counterpart:
+// with every logical rank on one GPU, stream order is the only synchronisation.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "a2a_internal.h"
+#include "a2a_staged.h"
+
+using namespace a2a;
+
+struct a2a_ctx {
+    a2a_config cfg;
+    Workspace ws;
+    void *arena = nullptr;
+    size_t arena_bytes = 0;
+    std::string error;
+
+    // State of the current step.
+    uint32_t sent_mask = 0;        // split calls: ranks whose dispatch_send ran in this step
+    bool step_open = false;        // split calls: a send has run and no recv yet closed the step
+    bool recv_seen = false;        // split calls: a recv has run in this step
+    bool group_routing = false;    // the last dispatch was a group call (route_slot is valid)
+    uint32_t num_tokens[kMaxWorld] = {};  // tokens of each rank in the last dispatch
+    uint32_t quantized = 0;        // mode of the last dispatch
+
+    Staging staging;               // buffers and tables of the split calls
+};
+
+namespace {
+
+thread_local std::string g_create_error;
+
+int fail(a2a_ctx *ctx, int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    if (ctx != nullptr) {
+        ctx->error = buf;
+    } else {
+        g_create_error = buf;
+    }
+    return code;
+}
+
+int hip_fail(a2a_ctx *ctx, hipError_t e, const char *what) {
+    return fail(ctx, (int)e, "%s: %s", what, hipGetErrorString(e));
+}
+
+size_t align_up(size_t n, size_t a) { return (n + a - 1) / a * a; }
+
+uint32_t ceil_div_u32(uint64_t n, uint64_t m) { return (uint32_t)((n + m - 1) / m); }
+
+bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+struct DeviceGuard {
+    int prev = -1;
+    bool ok = false;
+    explicit DeviceGuard(int dev) {
+        if (hipGetDevice(&prev) == hipSuccess) {
+            ok = prev == dev || hipSetDevice(dev) == hipSuccess;
+        }
+    }
+    ~DeviceGuard() {
+        if (ok && prev >= 0) (void)hipSetDevice(prev);
+    }
+};
+
+size_t row_bytes_of(const a2a_config &c) { return (size_t)c.hidden_dim * c.in_elemsize; }
+
+int check_config(const a2a_config &c) {
+    if (c.struct_size != sizeof(a2a_config))
+        return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "a2a_config.struct_size is %u, expected %zu",
+                    c.struct_size, sizeof(a2a_config));
+    if (c.world_size == 0 || c.world_size > A2A_MAX_WORLD_SIZE)
+        return fail(nullptr, A2A_ERR_UNSUPPORTED, "world_size %u not in [1, %d]", c.world_size,
+                    A2A_MAX_WORLD_SIZE);
+    if (c.dp_size != 1)
+        return fail(nullptr, A2A_ERR_UNSUPPORTED, "dp_size %u: only 1 is supported", c.dp_size);
+    if (c.node_size == 0 || c.world_size % c.node_size != 0)
+        return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "node_size %u does not divide world_size %u",
+                    c.node_size, c.world_size);
+    if (c.num_experts == 0 || c.num_experts > A2A_MAX_EXPERTS)
+        return fail(nullptr, A2A_ERR_UNSUPPORTED, "num_experts %u not in [1, %d]", c.num_experts,
+                    A2A_MAX_EXPERTS);
+    if (c.num_experts_per_token == 0 || c.num_experts_per_token > A2A_MAX_EXPERTS_PER_TOKEN)
+        return fail(nullptr, A2A_ERR_UNSUPPORTED, "num_experts_per_token %u not in [1, %d]",
+                    c.num_experts_per_token, A2A_MAX_EXPERTS_PER_TOKEN);
+    if (((size_t)c.world_size + 1) * c.num_experts + 32 > 16384)
+        return fail(nullptr, A2A_ERR_UNSUPPORTED,
+                    "world_size * num_experts = %u is too large for the layout kernel",
+                    c.world_size * c.num_experts);
+    if (c.expert_padding == 0)
+        return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "expert_padding must be at least 1");
+    if (c.hidden_dim == 0 || (c.in_elemsize != 1 && c.in_elemsize != 2 && c.in_elemsize != 4))
+        return fail(nullptr, A2A_ERR_UNSUPPORTED, "hidden_dim %u / in_elemsize %u", c.hidden_dim,
+                    c.in_elemsize);
+    if (row_bytes_of(c) % 16 != 0)
+        return fail(nullptr, A2A_ERR_UNSUPPORTED,
+                    "a dispatched row of %zu bytes is not a multiple of 16 "
+                    "(the reference copies 16-byte chunks too, a2a_dispatch_send.cu:341)",
+                    row_bytes_of(c));
+    const uint32_t od = c.out_dtype;
+    if (!((od == A2A_BF16 && c.out_elemsize == 2) || (od == A2A_F16 && c.out_elemsize == 2) ||
+          (od == A2A_F32 && c.out_elemsize == 4)))
+        return fail(nullptr, A2A_ERR_UNSUPPORTED, "out_dtype %u with out_elemsize %u", od,
+                    c.out_elemsize);
+    if (c.hidden_dim % (c.out_elemsize == 4 ? 4 : 8) != 0)
+        return fail(nullptr, A2A_ERR_UNSUPPORTED,
+                    "hidden_dim %u is not a multiple of the combine vector width", c.hidden_dim);
+    if (c.hidden_dim_scale != 0 && c.scale_elemsize != 4)
+        return fail(nullptr, A2A_ERR_UNSUPPORTED, "scale_elemsize %u: scales must be float",
+                    c.scale_elemsize);
+    if (c.max_num_tokens == 0)
+        return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "max_num_tokens must be at least 1");
+    if ((uint64_t)c.max_num_tokens * c.num_experts_per_token > 0x7FFFFFFFull)
+        return fail(nullptr, A2A_ERR_UNSUPPORTED, "max_num_tokens * num_experts_per_token too large");
+    return A2A_OK;
+}
+
+int check_rank(a2a_ctx *ctx, uint32_t rank) {
+    if (rank >= ctx->cfg.world_size)
+        return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "rank %u out of range [0, %u)", rank,
+                    ctx->cfg.world_size);
+    return A2A_OK;
+}
+
+// Arguments of the send half that do not depend on who receives.
+int check_send(a2a_ctx *ctx, uint32_t rank, uint64_t num_tokens, const void *x, uint64_t x_stride,
+               uint32_t quantize, const float *xs, const int32_t *indices) {
+    const a2a_config &c = ctx->cfg;
+    if (num_tokens > c.max_num_tokens)
+        return fail(ctx, A2A_ERR_TOO_MANY_TOKENS, "Number of tokens exceeds maximum allowed (rank %u: %llu > %u)",
+                    rank, (unsigned long long)num_tokens, c.max_num_tokens);
+    if (quantize > 1) return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "quantize must be 0 or 1");
+    if (quantize) {
+        if (c.in_elemsize != 1 || c.hidden_dim % 128 != 0 || c.hidden_dim_scale != c.hidden_dim / 128 ||
+            c.scale_elemsize != 4)
+            return fail(ctx, A2A_ERR_UNSUPPORTED,
+                        "quantise mode needs in_elemsize 1, hidden_dim %% 128 == 0 and "
+                        "hidden_dim_scale == hidden_dim / 128 (got %u, %u, %u)",
+                        c.in_elemsize, c.hidden_dim, c.hidden_dim_scale);
+        if (xs != nullptr)
+            return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "quantise mode computes the scales: x_scale must be null");
+    }
+    if (num_tokens == 0) return A2A_OK;
+    if (x == nullptr || indices == nullptr)
+        return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "rank %u: null x or indices with %llu tokens", rank,
+                    (unsigned long long)num_tokens);
+    if (!aligned16(x) || x_stride % 16 != 0)
+        return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: x rows must be 16-byte aligned", rank);
+    const uint64_t need = quantize ? (uint64_t)c.hidden_dim * 2 : row_bytes_of(c);
+    if (x_stride < need && num_tokens > 1)
+        return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "rank %u: x_stride %llu smaller than a row (%llu bytes)",
+                    rank, (unsigned long long)x_stride, (unsigned long long)need);
+    if (!quantize && c.hidden_dim_scale != 0 && xs == nullptr)
+        return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "rank %u: hidden_dim_scale is %u but x_scale is null",
+                    rank, c.hidden_dim_scale);
+    return A2A_OK;
+}
+
+int check_recv(a2a_ctx *ctx, uint32_t rank, const void *out_x, uint64_t out_stride,
+               const float *out_scale) {
+    const a2a_config &c = ctx->cfg;
+    if (out_x == nullptr) return A2A_OK;  // a rank may decline to receive
+    if (!aligned16(out_x) || out_stride % 16 != 0)
+        return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: out_x rows must be 16-byte aligned", rank);
+    if (out_stride < row_bytes_of(c))
+        return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "rank %u: out_x_stride %llu smaller than a row", rank,
+                    (unsigned long long)out_stride);
+    if (c.hidden_dim_scale != 0 && out_scale == nullptr)
+        return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "rank %u: hidden_dim_scale is %u but out_x_scale is null",
+                    rank, c.hidden_dim_scale);
+    return A2A_OK;
+}
+
+uint32_t elem_size_of(uint32_t dtype) {
+    switch (dtype) {
+        case A2A_F16:
+        case A2A_BF16:
+            return 2;
+        case A2A_F32:
+            return 4;
+        default:
+            return 0;
+    }
+}
+
+// Upper bound, known to the host, of the rows any receiver got in this step.
+uint32_t rows_upper_bound(const a2a_ctx *ctx) {
+    uint64_t rows = 0;
+    for (uint32_t g = 0; g < ctx->cfg.world_size; ++g) {
+        if (ctx->sent_mask >> g & 1) rows += (uint64_t)ctx->num_tokens[g] * ctx->cfg.num_experts_per_token;
+    }
+    const uint64_t cap = ctx->staging.max_recv;
+    return (uint32_t)(rows < cap ? rows : cap);
+}
+
+uint32_t all_ranks(const a2a_ctx *ctx) {
+    return ctx->cfg.world_size >= 32 ? 0xFFFFFFFFu : ((1u << ctx->cfg.world_size) - 1);
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *a2a_version(void) { return "0.1"; }
+
+size_t a2a_dispatch_token_stride(const a2a_config *c) {
+    // a2a_worker.rs:317-321
+    return align_up((size_t)c->hidden_dim * c->in_elemsize, 16) +
+           align_up((size_t)c->hidden_dim_scale * c->scale_elemsize, 16) + 16;
+}
+
+size_t a2a_combine_token_stride(const a2a_config *c) {
+    // a2a_worker.rs:323-325
+    return align_up((size_t)c->hidden_dim * c->out_elemsize, 16);
+}
+
+const char *a2a_last_error(const a2a_ctx *ctx) {
+    return ctx != nullptr ? ctx->error.c_str() : g_create_error.c_str();
+}
+
+int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
+    if (config == nullptr || out_ctx == nullptr)
+        return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "null argument");
+    *out_ctx = nullptr;
+    if (int rc = check_config(*config)) return rc;
+
+    int ndev = 0;
+    hipError_t e = hipGetDeviceCount(&ndev);
+    if (e != hipSuccess) return hip_fail(nullptr, e, "hipGetDeviceCount");
+    if (config->device < 0 || config->device >= ndev)
+        return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "device %d not in [0, %d)", config->device, ndev);
+    DeviceGuard guard(config->device);
+    if (!guard.ok) return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "cannot select device %d", config->device);
+
+    a2a_ctx *ctx = new (std::nothrow) a2a_ctx();
+    if (ctx == nullptr) return fail(nullptr, A2A_ERR_OUT_OF_MEMORY, "out of host memory");
+    ctx->cfg = *config;
+
+    const uint32_t N = config->world_size, E = config->num_experts, K = config->num_experts_per_token;
+    Workspace &ws = ctx->ws;
+    ws.max_tk = config->max_num_tokens * K;
+    ws.nb_max = ceil_div_u32(ws.max_tk, kRouteBlock);
+    ws.world = N;
+    ws.num_experts = E;
+    ws.topk = K;
+    ws.experts_per_rank = ceil_div_u32(E, N);
+    ws.node_size = config->node_size;
+    ws.expert_padding = config->expert_padding;
+
+    // One allocation, carved into 256-byte aligned tables.
+    size_t off = 0;
+    auto carve = [&off](size_t bytes) {
+        const size_t at = off;
+        off = align_up(off + bytes, 256);
+        return at;
+    };
+    const size_t o_local = carve((size_t)N * ws.max_tk * sizeof(uint16_t));
+    const size_t o_block = carve((size_t)N * ws.nb_max * E * sizeof(uint32_t));
+    const size_t o_routed = carve((size_t)N * E * sizeof(uint32_t));
+    const size_t o_offsets = carve((size_t)N * E * sizeof(uint32_t));
+    const size_t o_base = carve((size_t)N * E * sizeof(uint32_t));
+    const size_t o_tpe = carve((size_t)E * sizeof(uint32_t));
+    const size_t o_poff = carve((size_t)E * sizeof(uint32_t));
+    const size_t o_slot = carve((size_t)N * ws.max_tk * sizeof(uint32_t));
+    const size_t o_toff = carve((size_t)N * ws.max_tk * sizeof(uint32_t));
+    const size_t o_err = carve(sizeof(uint32_t));
+    ctx->arena_bytes = off;
+    e = hipMalloc(&ctx->arena, ctx->arena_bytes);
+    if (e != hipSuccess) {
+        delete ctx;
+        return hip_fail(nullptr, e, "hipMalloc(workspace)");
+    }
+    e = hipMemset(ctx->arena, 0, ctx->arena_bytes);
+    if (e == hipSuccess) e = hipDeviceSynchronize();
+    if (e != hipSuccess) {
+        (void)hipFree(ctx->arena);
+        delete ctx;
+        return hip_fail(nullptr, e, "hipMemset(workspace)");
+    }
+    uint8_t *base = static_cast<uint8_t *>(ctx->arena);
+    ws.local_rank = reinterpret_cast<uint16_t *>(base + o_local);
+    ws.block_prefix = reinterpret_cast<uint32_t *>(base + o_block);
+    ws.num_routed = reinterpret_cast<uint32_t *>(base + o_routed);
+    ws.expert_offsets = reinterpret_cast<uint32_t *>(base + o_offsets);
+    ws.slot_base = reinterpret_cast<uint32_t *>(base + o_base);
+    ws.tokens_per_expert = reinterpret_cast<uint32_t *>(base + o_tpe);
+    ws.padded_offset = reinterpret_cast<uint32_t *>(base + o_poff);
+    ws.route_slot = reinterpret_cast<uint32_t *>(base + o_slot);
+    ws.token_offset = reinterpret_cast<uint32_t *>(base + o_toff);
+    ws.err = reinterpret_cast<uint32_t *>(base + o_err);
+
+    if (config->flags & A2A_FLAG_PREALLOC_STAGING) {
+        std::string msg;
+        const int rc = staging_allocate(ctx->staging, *config, &msg);
+        if (rc != 0) {
+            (void)hipFree(ctx->arena);
+            delete ctx;
+            return fail(nullptr, rc, "%s", msg.c_str());
+        }
+    }
+    *out_ctx = ctx;
+    return A2A_OK;
+}
+
+int a2a_ctx_destroy(a2a_ctx *ctx) {
+    if (ctx == nullptr) return A2A_OK;
+    DeviceGuard guard(ctx->cfg.device);
+    (void)hipDeviceSynchronize();
+    staging_free(ctx->staging);
+    hipError_t e = hipFree(ctx->arena);
+    delete ctx;
+    return e == hipSuccess ? A2A_OK : (int)e;
+}
+
+int a2a_ctx_status(a2a_ctx *ctx, void *stream, uint32_t *flags) {
+    if (ctx == nullptr || flags == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    DeviceGuard guard(ctx->cfg.device);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e = hipStreamSynchronize(s);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamSynchronize");
+    e = hipMemcpy(flags, ctx->ws.err, sizeof(uint32_t), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipMemcpy(err)");
+    if (*flags != 0) {
+        e = hipMemset(ctx->ws.err, 0, sizeof(uint32_t));
+        if (e != hipSuccess) return hip_fail(ctx, e, "hipMemset(err)");
+    }
+    return A2A_OK;
+}
+
+int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize, void *stream) {
+    if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (args == nullptr) return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "null args");
+    const a2a_config &c = ctx->cfg;
+    const uint32_t N = c.world_size, K = c.num_experts_per_token;
+    for (uint32_t r = 0; r < N; ++r) {
+        const a2a_dispatch_args &a = args[r];
+        if (int rc = check_send(ctx, r, a.num_tokens, a.x_ptr, a.x_stride, quantize, a.x_scale_ptr, a.indices))
+            return rc;
+        if (int rc = check_recv(ctx, r, a.out_x, a.out_x_stride, a.out_x_scale)) return rc;
+    }
+    DeviceGuard guard(c.device);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+
+    RouteArgs ra;
+    FinalizeArgs fa;
+    PushArgs pa;
+    memset(&ra, 0, sizeof ra);
+    memset(&fa, 0, sizeof fa);
+    memset(&pa, 0, sizeof pa);
+    uint32_t blocks = 0, tokens = 0;
+    for (uint32_t r = 0; r < N; ++r) {
+        const a2a_dispatch_args &a = args[r];
+        const uint32_t T = (uint32_t)a.num_tokens;
+        ra.src[r] = RouteSrc{a.indices, a.bound_m, (uint32_t)a.indices_stride, T};
+        ra.block_start[r] = blocks;
+        fa.num_blocks[r] = ceil_div_u32((uint64_t)T * K, kRouteBlock);
+        blocks += fa.num_blocks[r];
+        fa.out_num_tokens[r] = a.out_num_tokens;
+        fa.out_rows[r] = a.out_x != nullptr ? (uint32_t)(a.out_x_rows > 0xFFFFFFFFull ? 0xFFFFFFFFull : a.out_x_rows)
+                                            : 0xFFFFFFFFu;
+        PushSrc &ps = pa.src[r];
+        ps.x = static_cast<const uint8_t *>(a.x_ptr);
+        ps.x_scale = a.x_scale_ptr;
+        ps.indices = a.indices;
+        ps.bound_m = a.bound_m;
+        ps.x_stride = a.x_stride;
+        ps.xs_stride_elem = (uint32_t)a.x_scale_stride_elem;
+        ps.xs_stride_token = (uint32_t)a.x_scale_stride_token;
+        ps.indices_stride = (uint32_t)a.indices_stride;
+        ps.num_tokens = T;
+        PushDst &pd = pa.dst[r];
+        pd.out_x = static_cast<uint8_t *>(a.out_x);
+        pd.out_scale = a.out_x_scale;
+        pd.out_stride = a.out_x_stride;
+        pd.os_stride_elem = (uint32_t)a.out_x_scale_stride_elem;
+        pd.os_stride_token = (uint32_t)a.out_x_scale_stride_token;
+        pd.out_rows = fa.out_rows[r];
+        pa.token_start[r] = tokens;
+        tokens += T;
+        ctx->num_tokens[r] = T;
+    }
+    for (uint32_t r = N; r <= (uint32_t)kMaxWorld; ++r) {
+        ra.block_start[r] = blocks;
+        pa.token_start[r] = tokens;
+    }
+    ra.rank_mask = fa.fold_mask = fa.valid_mask = fa.recv_mask = all_ranks(ctx);
+    pa.row_bytes = (uint32_t)row_bytes_of(c);
+    pa.hidden_dim = c.hidden_dim;
+    pa.hidden_dim_scale = c.hidden_dim_scale;
+
+    hipError_t e = launch_route(ra, ctx->ws, blocks, s);
+    if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
+    e = launch_finalize(fa, ctx->ws, s);
+    if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+    e = launch_dispatch_push(pa, ctx->ws, quantize != 0, tokens, s);
+    if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_push");
+
+    ctx->group_routing = true;
+    ctx->step_open = false;
+    ctx->sent_mask = 0;
+    ctx->quantized = quantize;
+    return A2A_OK;
+}
+
+int a2a_combine(a2a_ctx *ctx, const a2a_combine_args *args, uint32_t expert_y_dtype,
+                uint32_t accumulate, void *stream) {
+    if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (args == nullptr) return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "null args");
+    const a2a_config &c = ctx->cfg;
+    const uint32_t N = c.world_size;
+    if (!ctx->group_routing)
+        return fail(ctx, A2A_ERR_BAD_ORDER, "a2a_combine needs the routing of a preceding a2a_dispatch");
+    const uint32_t in_size = elem_size_of(expert_y_dtype);
+    if (in_size == 0)
+        return fail(ctx, A2A_ERR_UNSUPPORTED, "expert_y dtype %u: only F16, BF16 and F32 are supported",
+                    expert_y_dtype);
+    const uint32_t vec = 16 / in_size;
+    if (c.hidden_dim % vec != 0)
+        return fail(ctx, A2A_ERR_UNSUPPORTED, "hidden_dim %u is not a multiple of %u", c.hidden_dim, vec);
+    CombArgs ca;
+    memset(&ca, 0, sizeof ca);
+    uint32_t tokens = 0;
+    for (uint32_t r = 0; r < N; ++r) {
+        const a2a_combine_args &a = args[r];
+        if (a.num_tokens > c.max_num_tokens)
+            return fail(ctx, A2A_ERR_TOO_MANY_TOKENS, "Number of tokens exceeds maximum allowed (rank %u)", r);
+        if (a.expert_y != nullptr && (!aligned16(a.expert_y) || a.expert_y_stride % 16 != 0))
+            return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: expert_y rows must be 16-byte aligned", r);
+        const uint64_t out_stride_bytes = a.out_tokens_stride * c.out_elemsize;
+        const uint32_t out_chunk = vec * c.out_elemsize;
+        if (a.num_tokens != 0) {
+            if (a.out_tokens == nullptr || a.indices == nullptr || a.weights == nullptr)
+                return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "rank %u: null out_tokens, indices or weights", r);
+            if (((uintptr_t)a.out_tokens % out_chunk) != 0 || out_stride_bytes % out_chunk != 0)
+                return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: out_tokens rows must be %u-byte aligned", r,
+                            out_chunk);
+        }
+        ca.src[r] = CombSrc{static_cast<const uint8_t *>(a.expert_y), a.expert_y_stride,
+                            (uint32_t)(a.expert_y_rows > 0xFFFFFFFFull ? 0xFFFFFFFFull : a.expert_y_rows), 0};
+        CombDst &d = ca.dst[r];
+        d.out = static_cast<uint8_t *>(a.out_tokens);
+        d.indices = a.indices;
+        d.weights = a.weights;
+        d.bound_m = a.bound_m;
+        d.out_stride = out_stride_bytes;
+        d.indices_stride = (uint32_t)a.indices_stride;
+        d.weights_stride = (uint32_t)a.weights_stride;
+        d.num_tokens = (uint32_t)a.num_tokens;
+        ca.token_start[r] = tokens;
+        tokens += (uint32_t)a.num_tokens;
+    }
+    for (uint32_t r = N; r <= (uint32_t)kMaxWorld; ++r) ca.token_start[r] = tokens;
+    ca.hidden_dim = c.hidden_dim;
+    ca.accumulate = accumulate ? 1 : 0;
+    DeviceGuard guard(c.device);
+    hipError_t e = launch_combine_gather(ca, ctx->ws, expert_y_dtype, c.out_dtype, tokens,
+                                         static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(ctx, e, "launch combine_gather");
+    return A2A_OK;
+}
+
+int a2a_ctx_read_table(a2a_ctx *ctx, uint32_t rank, uint32_t which, uint32_t *out, size_t count,
+                       void *stream) {
+    if (ctx == nullptr || out == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (int rc = check_rank(ctx, rank)) return rc;
+    const Workspace &ws = ctx->ws;
+    const uint32_t E = ws.num_experts;
+    const uint32_t *src = nullptr;
+    size_t limit = 0;
+    switch (which) {
+        case A2A_TABLE_NUM_ROUTED:
+            src = ws.num_routed + (size_t)rank * E;
+            limit = E;
+            break;
+        case A2A_TABLE_EXPERT_OFFSETS:
+            src = ws.expert_offsets + (size_t)rank * E;
+            limit = E;
+            break;
+        case A2A_TABLE_TOKEN_OFFSET:
+            src = ws.token_offset + (size_t)rank * ws.max_tk;
+            limit = ws.max_tk;
+            break;
+        case A2A_TABLE_SLOT:
+            if (!ctx->group_routing)
+                return fail(ctx, A2A_ERR_BAD_ORDER, "slots exist only after a2a_dispatch");
+            src = ws.route_slot + (size_t)rank * ws.max_tk;
+            limit = ws.max_tk;
+            break;
+        case A2A_TABLE_PADDED_INDEX:
+        case A2A_TABLE_SOURCE_RANK:
+        case A2A_TABLE_SOURCE_POSITION:
+        case A2A_TABLE_NUM_RECV_TOKENS:
+            src = staging_table(ctx->staging, ctx->cfg, rank, which, &limit);
+            if (src == nullptr)
+                return fail(ctx, A2A_ERR_BAD_ORDER, "receive tables exist only after a2a_dispatch_recv");
+            break;
+        default:
+            return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "unknown table %u", which);
+    }
+    if (count > limit) return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "count %zu exceeds the table (%zu)", count, limit);
+    DeviceGuard guard(ctx->cfg.device);
+    hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamSynchronize");
+    e = hipMemcpy(out, src, count * sizeof(uint32_t), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) return hip_fail(ctx, e, "hipMemcpy(table)");
+    return A2A_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Split calls: one logical rank at a time, rows travel through staging.
+// ---------------------------------------------------------------------------
+
+int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void *x_ptr,
+                      size_t x_stride, uint32_t quantize, const float *x_scale_ptr,
+                      size_t x_scale_stride_elem, size_t x_scale_stride_token,
+                      const int32_t *indices, size_t indices_stride, const float *weights,
+                      size_t weights_stride, const int32_t *bound_m, void *stream) {
+    (void)weights;
+    (void)weights_stride;
+    if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (int rc = check_rank(ctx, rank)) return rc;
+    if (int rc = check_send(ctx, rank, num_tokens, x_ptr, x_stride, quantize, x_scale_ptr, indices)) return rc;
+    const a2a_config &c = ctx->cfg;
+    DeviceGuard guard(c.device);
+    if (!ctx->staging.allocated) {
+        std::string msg;
+        if (int rc = staging_allocate(ctx->staging, c, &msg)) return fail(ctx, rc, "%s", msg.c_str());
+    }
+    // A send after a recv starts a new step.
+    if (!ctx->step_open || ctx->recv_seen) {
+        ctx->sent_mask = 0;
+        ctx->recv_seen = false;
+        ctx->step_open = true;
+        ctx->staging.recv_mask = 0;
+        ctx->staging.combine_sent_mask = 0;
+    }
+    if (ctx->sent_mask != 0 && ctx->quantized != quantize)
+        return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "all sends of a step must use the same mode");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint32_t K = c.num_experts_per_token;
+    const uint32_t T = (uint32_t)num_tokens;
+
+    RouteArgs ra;
+    FinalizeArgs fa;
+    memset(&ra, 0, sizeof ra);
+    memset(&fa, 0, sizeof fa);
+    const uint32_t nb = ceil_div_u32((uint64_t)T * K, kRouteBlock);
+    ra.src[rank] = RouteSrc{indices, bound_m, (uint32_t)indices_stride, T};
+    for (uint32_t r = 0; r <= (uint32_t)kMaxWorld; ++r) ra.block_start[r] = r <= rank ? 0 : nb;
+    ra.rank_mask = 1u << rank;
+    fa.num_blocks[rank] = nb;
+    fa.fold_mask = 1u << rank;
+    fa.valid_mask = ctx->sent_mask | (1u << rank);
+    fa.recv_mask = 0;
+    // Route launches address sources through block_start, so a single source
+    // other than rank 0 needs the grid to start at it.
+    hipError_t e = launch_route(ra, ctx->ws, nb, s);
+    if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
+    e = launch_finalize(fa, ctx->ws, s);
+    if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+
+    StageSendArgs sa;
+    memset(&sa, 0, sizeof sa);
+    sa.rank = rank;
+    sa.src.x = static_cast<const uint8_t *>(x_ptr);
+    sa.src.x_scale = x_scale_ptr;
+    sa.src.indices = indices;
+    sa.src.bound_m = bound_m;
+    sa.src.x_stride = x_stride;
+    sa.src.xs_stride_elem = (uint32_t)x_scale_stride_elem;
+    sa.src.xs_stride_token = (uint32_t)x_scale_stride_token;
+    sa.src.indices_stride = (uint32_t)indices_stride;
+    sa.src.num_tokens = T;
+    sa.row_bytes = (uint32_t)row_bytes_of(c);
+    sa.hidden_dim = c.hidden_dim;
+    sa.hidden_dim_scale = c.hidden_dim_scale;
+    e = launch_stage_send(sa, ctx->ws, ctx->staging, quantize != 0, s);
+    if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send");
+
+    ctx->sent_mask |= 1u << rank;
+    ctx->num_tokens[rank] = T;
+    ctx->quantized = quantize;
+    ctx->group_routing = false;
+    return A2A_OK;
+}
+
+int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void *out_x,
+                      size_t out_x_stride, size_t out_x_rows, float *out_x_scale,
+                      size_t out_x_scale_stride_elem, size_t out_x_scale_stride_token,
+                      void *stream) {
+    if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (int rc = check_rank(ctx, rank)) return rc;
+    if (!ctx->step_open || ctx->sent_mask == 0)
+        return fail(ctx, A2A_ERR_BAD_ORDER, "a2a_dispatch_recv before any a2a_dispatch_send of the step");
+    if (int rc = check_recv(ctx, rank, out_x, out_x_stride, out_x_scale)) return rc;
+    const a2a_config &c = ctx->cfg;
+    DeviceGuard guard(c.device);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+
+    FinalizeArgs fa;
+    memset(&fa, 0, sizeof fa);
+    fa.fold_mask = 0;
+    fa.valid_mask = ctx->sent_mask;
+    fa.recv_mask = 1u << rank;
+    fa.out_num_tokens[rank] = out_num_tokens;
+    fa.out_rows[rank] = out_x != nullptr ? (uint32_t)(out_x_rows > 0xFFFFFFFFull ? 0xFFFFFFFFull : out_x_rows)
+                                         : 0xFFFFFFFFu;
+    hipError_t e = launch_finalize(fa, ctx->ws, s);
+    if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+
+    StageRecvArgs rv;
+    memset(&rv, 0, sizeof rv);
+    rv.rank = rank;
+    rv.valid_mask = ctx->sent_mask;
+    rv.dst.out_x = static_cast<uint8_t *>(out_x);
+    rv.dst.out_scale = out_x_scale;
+    rv.dst.out_stride = out_x_stride;
+    rv.dst.os_stride_elem = (uint32_t)out_x_scale_stride_elem;
+    rv.dst.os_stride_token = (uint32_t)out_x_scale_stride_token;
+    rv.dst.out_rows = fa.out_rows[rank];
+    rv.row_bytes = (uint32_t)row_bytes_of(c);
+    rv.hidden_dim_scale = c.hidden_dim_scale;
+    rv.max_rows = rows_upper_bound(ctx);
+    e = launch_stage_recv(rv, ctx->ws, ctx->staging, s);
+    if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_recv");
+    ctx->recv_seen = true;
+    ctx->staging.recv_mask |= 1u << rank;
+    return A2A_OK;
+}
+
+int a2a_combine_send(a2a_ctx *ctx, uint32_t rank, const void *expert_y, size_t expert_y_stride,
+                     size_t expert_y_rows, void *stream) {
+    if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (int rc = check_rank(ctx, rank)) return rc;
+    if (!ctx->staging.allocated || !(ctx->staging.recv_mask >> rank & 1))
+        return fail(ctx, A2A_ERR_BAD_ORDER, "a2a_combine_send before a2a_dispatch_recv of rank %u", rank);
+    if (expert_y == nullptr || !aligned16(expert_y) || expert_y_stride % 16 != 0)
+        return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: expert_y rows must be non-null and 16-byte aligned", rank);
+    const a2a_config &c = ctx->cfg;
+    DeviceGuard guard(c.device);
+    CombineSendArgs cs;
+    memset(&cs, 0, sizeof cs);
+    cs.rank = rank;
+    cs.y = static_cast<const uint8_t *>(expert_y);
+    cs.y_stride = expert_y_stride;
+    cs.y_rows = (uint32_t)(expert_y_rows > 0xFFFFFFFFull ? 0xFFFFFFFFull : expert_y_rows);
+    cs.row_bytes = (uint32_t)((size_t)c.hidden_dim * c.out_elemsize);
+    cs.max_rows = rows_upper_bound(ctx);
+    hipError_t e = launch_combine_send(cs, ctx->ws, ctx->staging, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(ctx, e, "launch combine_send");
+    ctx->staging.combine_sent_mask |= 1u << rank;
+    return A2A_OK;
+}
+
+int a2a_combine_recv(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, size_t num_recv_tokens,
+                     uint32_t expert_y_dtype, void *out_tokens, size_t out_tokens_stride,
+                     const int32_t *indices, size_t indices_stride, const float *weights,
+                     size_t weights_stride, const int32_t *bound_m, uint32_t accumulate,
+                     void *stream) {
+    (void)num_recv_tokens;
+    if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (int rc = check_rank(ctx, rank)) return rc;
+    const a2a_config &c = ctx->cfg;
+    if (!ctx->staging.allocated || ctx->staging.combine_sent_mask == 0)
+        return fail(ctx, A2A_ERR_BAD_ORDER, "a2a_combine_recv before any a2a_combine_send of the step");
+    if (num_tokens > c.max_num_tokens)
+        return fail(ctx, A2A_ERR_TOO_MANY_TOKENS, "Number of tokens exceeds maximum allowed (rank %u)", rank);
+    if (elem_size_of(expert_y_dtype) != c.out_elemsize)
+        return fail(ctx, A2A_ERR_UNSUPPORTED,
+                    "expert_y dtype %u does not have the %u-byte elements the staging rows were sized for",
+                    expert_y_dtype, c.out_elemsize);
+    const uint32_t vec = 16 / c.out_elemsize;
+    const uint32_t out_chunk = vec * c.out_elemsize;
+    if (num_tokens != 0) {
+        if (out_tokens == nullptr || indices == nullptr || weights == nullptr)
+            return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "rank %u: null out_tokens, indices or weights", rank);
+        if (((uintptr_t)out_tokens % out_chunk) != 0 || (out_tokens_stride * c.out_elemsize) % out_chunk != 0)
+            return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: out_tokens rows must be %u-byte aligned", rank, out_chunk);
+    }
+    DeviceGuard guard(c.device);
+    CombineRecvArgs cr;
+    memset(&cr, 0, sizeof cr);
+    cr.rank = rank;
+    cr.dst.out = static_cast<uint8_t *>(out_tokens);
+    cr.dst.indices = indices;
+    cr.dst.weights = weights;
+    cr.dst.bound_m = bound_m;
+    cr.dst.out_stride = out_tokens_stride * c.out_elemsize;
+    cr.dst.indices_stride = (uint32_t)indices_stride;
+    cr.dst.weights_stride = (uint32_t)weights_stride;
+    cr.dst.num_tokens = (uint32_t)num_tokens;
+    cr.hidden_dim = c.hidden_dim;
+    cr.accumulate = accumulate ? 1 : 0;
+    hipError_t e = launch_combine_recv(cr, ctx->ws, ctx->staging, expert_y_dtype, c.out_dtype,
+                                       static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(ctx, e, "launch combine_recv");
+    return A2A_OK;
+}
+
+}  // extern "C"

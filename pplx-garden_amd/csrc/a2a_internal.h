@@ -1,0 +1,164 @@
+// Shared between the HIP kernels and the host context: argument blocks that
+// are passed to kernels BY VALUE (so a launch records everything it needs and
+// nothing has to be uploaded first), and the layout of the device workspace.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "a2a.h"
+
+namespace a2a {
+
+constexpr int kWave = 64;
+// Entries ((token, k) pairs) handled by one routing workgroup; one entry per
+// thread, so block-local ranks fit in 16 bits.
+constexpr int kRouteBlock = 1024;
+constexpr uint32_t kInvalidSlot = 0xFFFFFFFFu;
+constexpr int kMaxWorld = A2A_MAX_WORLD_SIZE;
+
+// Device workspace, shared by all logical ranks of a context.  Per-rank arrays
+// are laid out [world][...] with the strides below.
+struct Workspace {
+    uint16_t *local_rank;      // [N][max_tk]    rank of an entry among equal experts inside its routing block
+    uint32_t *block_prefix;    // [N][nb_max][E] per-block histogram, turned into an exclusive prefix over blocks
+    uint32_t *num_routed;      // [N][E]         routes per (source, expert)
+    uint32_t *expert_offsets;  // [N][E]         inclusive scan of num_routed over experts
+    uint32_t *slot_base;       // [N][E]         first receiver row of (source, expert)
+    uint32_t *tokens_per_expert;  // [E]         per receiver-local expert, summed over sources
+    uint32_t *padded_offset;   // [E]            first row of an expert inside its receiver
+    uint32_t *route_slot;      // [N][max_tk]    receiver row of every copy (kInvalidSlot if dropped)
+    uint32_t *token_offset;    // [N][max_tk]    rank of every copy inside its (source, expert)
+    uint32_t *err;             // [1]            A2A_DEV_* bits, sticky
+    uint32_t max_tk;           // max_num_tokens * K
+    uint32_t nb_max;           // ceil(max_tk / kRouteBlock)
+    uint32_t world;            // N
+    uint32_t num_experts;      // E
+    uint32_t topk;             // K
+    uint32_t experts_per_rank; // Le = ceil(E / N)
+    uint32_t node_size;
+    uint32_t expert_padding;
+};
+
+struct RouteSrc {
+    const int32_t *indices;
+    const int32_t *bound_m;
+    uint32_t indices_stride;
+    uint32_t num_tokens;
+};
+
+struct RouteArgs {
+    RouteSrc src[kMaxWorld];
+    uint32_t block_start[kMaxWorld + 1];  // first routing block of each source in the grid
+    uint32_t rank_mask;                   // sources routed by this launch
+};
+
+struct FinalizeArgs {
+    int32_t *out_num_tokens[kMaxWorld];   // per receiver, may be null
+    uint32_t out_rows[kMaxWorld];         // rows of the receiver's buffer (overflow check)
+    uint32_t num_blocks[kMaxWorld];       // routing blocks written per source by the route launch
+    uint32_t fold_mask;                   // sources whose block histograms are folded by this launch
+    uint32_t valid_mask;                  // sources that count for the layout (others count as empty)
+    uint32_t recv_mask;                   // receivers whose layout is computed by this launch
+};
+
+struct PushSrc {
+    const uint8_t *x;
+    const float *x_scale;
+    const int32_t *indices;
+    const int32_t *bound_m;
+    uint64_t x_stride;        // bytes
+    uint32_t xs_stride_elem;  // elements
+    uint32_t xs_stride_token;
+    uint32_t indices_stride;
+    uint32_t num_tokens;
+};
+
+struct PushDst {
+    uint8_t *out_x;
+    float *out_scale;
+    uint64_t out_stride;      // bytes
+    uint32_t os_stride_elem;  // elements
+    uint32_t os_stride_token;
+    uint32_t out_rows;
+    uint32_t pad_;
+};
+
+struct PushArgs {
+    PushSrc src[kMaxWorld];
+    PushDst dst[kMaxWorld];
+    uint32_t token_start[kMaxWorld + 1];  // first workgroup (token) of each source in the grid
+    uint32_t row_bytes;                   // bytes of a dispatched row
+    uint32_t hidden_dim;
+    uint32_t hidden_dim_scale;
+};
+
+struct CombSrc {  // one per receiver rank: the expert outputs it holds
+    const uint8_t *y;
+    uint64_t y_stride;        // bytes
+    uint32_t y_rows;
+    uint32_t pad_;
+};
+
+struct CombDst {  // one per source rank: where its combined tokens go
+    uint8_t *out;
+    const int32_t *indices;
+    const float *weights;
+    const int32_t *bound_m;
+    uint64_t out_stride;      // bytes
+    uint32_t indices_stride;
+    uint32_t weights_stride;
+    uint32_t num_tokens;
+    uint32_t pad_;
+};
+
+struct CombArgs {
+    CombSrc src[kMaxWorld];
+    CombDst dst[kMaxWorld];
+    uint32_t token_start[kMaxWorld + 1];
+    uint32_t hidden_dim;
+    uint32_t accumulate;
+    // Split calls: rows are read from a staging buffer at the sender's own
+    // positions (exclusive expert offset + token offset) instead of from the
+    // receivers' expert_y at route_slot.  Null for the group call.
+    const uint8_t *staged_base;
+    uint64_t staged_stride;
+};
+
+// Launchers (defined next to their kernels); all return the hipError_t of the
+// launch.
+hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
+                        hipStream_t stream);
+hipError_t launch_finalize(const FinalizeArgs &args, const Workspace &ws, hipStream_t stream);
+hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool quantize,
+                                uint32_t total_tokens, hipStream_t stream);
+hipError_t launch_combine_gather(const CombArgs &args, const Workspace &ws, uint32_t in_dtype,
+                                 uint32_t out_dtype, uint32_t total_tokens, hipStream_t stream);
+
+// Device-side: effective token count of a source (bound_m clamps num_tokens,
+// a2a_dispatch_send.cu:172).
+__device__ __forceinline__ uint32_t effective_tokens(const int32_t *bound_m, uint32_t num_tokens) {
+    if (bound_m == nullptr) return num_tokens;
+    int32_t b = *bound_m;
+    if (b < 0) b = 0;
+    return (uint32_t)b < num_tokens ? (uint32_t)b : num_tokens;
+}
+
+// i-th source that receiver `rank` lays out (a2a_worker.rs:681-694, dp_size 1):
+// ranks of the other nodes starting at the next node, then the rest of the own
+// node starting after `rank`, then `rank`.
+__host__ __device__ __forceinline__ uint32_t source_order(uint32_t rank, uint32_t i, uint32_t world,
+                                                          uint32_t node_size) {
+    const uint32_t num_nodes = world / node_size;
+    const uint32_t rank_node = rank / node_size;
+    const uint32_t remote = (num_nodes - 1) * node_size;
+    if (i < remote) {
+        const uint32_t node = (rank_node + 1 + i / node_size) % num_nodes;
+        return node * node_size + i % node_size;
+    }
+    const uint32_t local = i - remote + 1;  // 1 .. node_size
+    if (local < node_size) return rank_node * node_size + (rank + local) % node_size;
+    return rank;
+}
+
+}  // namespace a2a

@@ -1,0 +1,90 @@
+// Staging buffers and kernels of the split calls (one logical rank per call).
+//
+// They keep the reference's structure: a send stages the rows of its tokens
+// (a2a_dispatch_send.cu:341-367), a recv lays out what it received and copies
+// it into the caller's buffers (a2a_worker.rs:526-703 on the CPU there, then
+// a2a_dispatch_recv.cu:122-156), combine-send copies expert rows back to the
+// staging row of the copy they answer (a2a_combine_send.cu:119-138,182-207)
+// and combine-recv gathers them (a2a_combine_recv.cu:94-148).
+//
+// Differences that follow from every rank living in one HBM: a token is staged
+// ONCE (quantised), not once per route, and the receiver finds it through a
+// position -> token table; the private / overflow split of the receive buffer
+// (max_private_tokens) does not exist.
+#pragma once
+
+#include <string>
+
+#include "a2a_internal.h"
+
+namespace a2a {
+
+struct Staging {
+    bool allocated = false;
+    void *arena = nullptr;
+    uint8_t *send_buf = nullptr;         // [N][max_num_tokens][disp_stride]: payload, scales, 16 spare bytes
+    uint32_t *pos_token = nullptr;       // [N][max_tk]: token behind each row of a sender's expert-sorted order
+    uint8_t *comb_buf = nullptr;         // [N][max_tk][comb_stride]: combine rows at the sender's positions
+    uint32_t *seg_start = nullptr;       // [N][N*Le + 1]: first received row of each (source, local expert) run
+    uint32_t *padded_index = nullptr;    // [N][max_recv]
+    uint32_t *source_rank = nullptr;     // [N][max_recv]
+    uint32_t *source_position = nullptr; // [N][max_recv]
+    uint32_t *num_recv = nullptr;        // [N][2]: received rows, rows from other nodes
+    size_t disp_stride = 0;
+    size_t comb_stride = 0;
+    uint32_t payload_bytes = 0;          // offset of the scales inside a staged dispatch row
+    uint32_t max_recv = 0;               // rows per receiver in the tables above
+    uint32_t max_tokens = 0;
+    uint32_t recv_mask = 0;              // receivers whose tables are valid in this step
+    uint32_t combine_sent_mask = 0;
+};
+
+struct StageSendArgs {
+    PushSrc src;
+    uint32_t rank;
+    uint32_t row_bytes;
+    uint32_t hidden_dim;
+    uint32_t hidden_dim_scale;
+};
+
+struct StageRecvArgs {
+    PushDst dst;
+    uint32_t rank;
+    uint32_t valid_mask;
+    uint32_t row_bytes;
+    uint32_t hidden_dim_scale;
+    uint32_t max_rows;        // upper bound of received rows known to the host
+};
+
+struct CombineSendArgs {
+    const uint8_t *y;
+    uint64_t y_stride;
+    uint32_t y_rows;
+    uint32_t rank;
+    uint32_t row_bytes;
+    uint32_t max_rows;
+};
+
+struct CombineRecvArgs {
+    CombDst dst;
+    uint32_t rank;
+    uint32_t hidden_dim;
+    uint32_t accumulate;
+};
+
+int staging_allocate(Staging &st, const a2a_config &cfg, std::string *error);
+void staging_free(Staging &st);
+// Device pointer of a receive-side table of `rank`, or null when none exists.
+const uint32_t *staging_table(const Staging &st, const a2a_config &cfg, uint32_t rank, uint32_t which,
+                              size_t *limit);
+
+hipError_t launch_stage_send(const StageSendArgs &args, const Workspace &ws, const Staging &st,
+                             bool quantize, hipStream_t stream);
+hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st,
+                             hipStream_t stream);
+hipError_t launch_combine_send(const CombineSendArgs &args, const Workspace &ws, const Staging &st,
+                               hipStream_t stream);
+hipError_t launch_combine_recv(const CombineRecvArgs &args, const Workspace &ws, const Staging &st,
+                               uint32_t in_dtype, uint32_t out_dtype, hipStream_t stream);
+
+}  // namespace a2a
