@@ -8,11 +8,11 @@
 // receivers' expert_y buffers, which live in the same HBM: one read per row,
 // no staging write.
 //
-// Design for CDNA4: one workgroup per token; a lane owns 16 bytes of every
-// source row, so K independent 16-byte loads are in flight per lane before the
-// first multiply-add.  Row pointers and weights are resolved once by the
-// first K lanes and read back as wave-uniform scalars (SGPR base + VGPR
-// offset addressing).  Accumulation is an explicit float fused multiply-add
+// Design for CDNA4: one wavefront per (token, slab of 64 sixteen-byte chunks);
+// a lane owns 16 bytes of every source row, so K independent 16-byte loads are
+// in flight per lane before the first multiply-add.  Row pointers and weights
+// are resolved once by the first K lanes and read back as wave-uniform scalars
+// (SGPR base + VGPR offset addressing).  Accumulation is an explicit float fused multiply-add
 // chain, k ascending, then one round-to-nearest-even to the output type
 // (combine_utils.cuh:108-114,14-23).
 #include "a2a_internal.h"
@@ -117,114 +117,139 @@ __device__ __forceinline__ uint64_t read_lane64c(uint64_t v, uint32_t lane) {
     return ((uint64_t)hi << 32) | lo;
 }
 
-// T: type of the expert_y rows, U: type of out_tokens.  KFIX > 0 unrolls the
-// route loop (all K loads issued before the first use).
+// Convert one 16-byte source chunk (raw) and fuse it into the accumulators.
+template <typename T, int V>
+__device__ __forceinline__ void fma_chunk(const u32x4 raw, float w, float (&acc)[V]) {
+    if constexpr (Elem<T>::kSize == 4) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_fmaf(w, __uint_as_float(raw[j]), acc[j]);
+    } else if constexpr (__is_same(T, Bf16)) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            acc[2 * j] = __builtin_fmaf(w, __uint_as_float(raw[j] << 16), acc[2 * j]);
+            acc[2 * j + 1] = __builtin_fmaf(w, __uint_as_float(raw[j] & 0xFFFF0000u), acc[2 * j + 1]);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            acc[2 * j] = __builtin_fmaf(
+                w, (float)__builtin_bit_cast(_Float16, (uint16_t)(raw[j] & 0xFFFF)), acc[2 * j]);
+            acc[2 * j + 1] = __builtin_fmaf(
+                w, (float)__builtin_bit_cast(_Float16, (uint16_t)(raw[j] >> 16)), acc[2 * j + 1]);
+        }
+    }
+}
+
+constexpr int kCombineWaves = 4;  // wavefronts per workgroup; each works on its own
+
+// T: type of the expert_y rows, U: type of out_tokens.  One WAVEFRONT handles
+// one slab of 64 sixteen-byte chunks of one token; wavefronts share nothing, so
+// a compute unit keeps many of them in flight and the latency of resolving a
+// token's routes is hidden by the loads of its neighbours.  KFIX > 0 unrolls
+// the route loop (all K loads issued before the first use).
 template <typename T, typename U, int KFIX>
-__global__ __launch_bounds__(1024) void combine_gather_kernel(const CombArgs args,
-                                                              const Workspace ws) {
+__global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(const CombArgs args,
+                                                                              const Workspace ws) {
     constexpr int V = vec_elems<T>();
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & (kWave - 1);
-    const uint32_t wave = tid / kWave;
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const uint32_t E = ws.num_experts;
     const uint32_t K = KFIX > 0 ? (uint32_t)KFIX : ws.topk;
+    const uint32_t num_chunks = args.hidden_dim / V;
+    const uint32_t slabs = (num_chunks + kWave - 1) / kWave;
 
+    const uint32_t unit = blockIdx.x * kCombineWaves + wave;
+    const uint32_t token_global = unit / slabs;
+    const uint32_t slab = unit - token_global * slabs;
+    if (token_global >= args.token_start[ws.world]) return;
     uint32_t g = 0;
-    while (g + 1 < ws.world && blockIdx.x >= args.token_start[g + 1]) ++g;
-    const uint32_t token = blockIdx.x - args.token_start[g];
+    while (g + 1 < ws.world && token_global >= args.token_start[g + 1]) ++g;
+    const uint32_t token = token_global - args.token_start[g];
     const CombDst &dst = args.dst[g];
     if (token >= effective_tokens(dst.bound_m, dst.num_tokens)) return;
 
-    uint64_t row_ptr = 0;
+    // Lane r holds the descriptor of receiver r; lanes 0..K-1 resolve a route
+    // each and pick their receiver's descriptor with a lane shuffle.
+    uint64_t y_base = 0, y_stride = 0;
+    uint32_t y_rows = 0;
+    if (lane < ws.world && args.staged_base == nullptr) {
+        y_base = (uint64_t)args.src[lane].y;
+        y_stride = args.src[lane].y_stride;
+        y_rows = args.src[lane].y_rows;
+    }
+    uint32_t expert = 0, slot = 0;
     float weight = 0.0f;
     if (lane < K) {
-        const uint32_t expert = (uint32_t)dst.indices[(size_t)token * dst.indices_stride + lane];
+        expert = (uint32_t)dst.indices[(size_t)token * dst.indices_stride + lane];
         weight = dst.weights[(size_t)token * dst.weights_stride + lane];
+        slot = args.staged_base != nullptr
+                   ? ws.token_offset[(size_t)g * ws.max_tk + token * K + lane]
+                   : ws.route_slot[(size_t)g * ws.max_tk + token * K + lane];
+    }
+    const bool expert_ok = expert < E;
+    const uint32_t r = expert_ok ? expert / ws.experts_per_rank : 0;
+    const uint64_t r_base = __shfl(y_base, (int)r);
+    const uint64_t r_stride = __shfl(y_stride, (int)r);
+    const uint32_t r_rows = __shfl(y_rows, (int)r);
+    uint64_t row_ptr = 0;
+    if (lane < K) {
         bool ok = false;
         if (args.staged_base != nullptr) {
             // a2a_combine_recv.cu:67-73: position = exclusive offset of the expert + token offset.
-            if (expert < E) {
+            if (expert_ok) {
                 const uint32_t excl = expert > 0 ? ws.expert_offsets[g * E + expert - 1] : 0;
-                const uint32_t pos = excl + ws.token_offset[(size_t)g * ws.max_tk + token * K + lane];
+                const uint32_t pos = excl + slot;
                 if (pos < ws.max_tk) {
                     row_ptr = (uint64_t)(args.staged_base +
                                          ((size_t)g * ws.max_tk + pos) * args.staged_stride);
                     ok = true;
                 }
             }
-        } else if (expert < E) {
-            const uint32_t slot = ws.route_slot[(size_t)g * ws.max_tk + token * K + lane];
-            const CombSrc &src = args.src[expert / ws.experts_per_rank];
-            if (src.y != nullptr && slot < src.y_rows) {
-                row_ptr = (uint64_t)(src.y + (size_t)slot * src.y_stride);
-                ok = true;
-            }
+        } else if (expert_ok && r_base != 0 && slot < r_rows) {
+            row_ptr = r_base + (uint64_t)slot * r_stride;
+            ok = true;
         }
-        if (!ok && wave == 0) atomicOr(ws.err, A2A_DEV_BAD_SLOT);
+        if (!ok && slab == 0) atomicOr(ws.err, A2A_DEV_BAD_SLOT);
     }
 
-    uint8_t *out_row = dst.out + (size_t)token * dst.out_stride;
-    const uint32_t num_chunks = args.hidden_dim / V;
+    const uint32_t c = slab * kWave + lane;
+    const bool active = c < num_chunks;
+    uint8_t *out_chunk = dst.out + (size_t)token * dst.out_stride + (size_t)c * V * Elem<U>::kSize;
+    float acc[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = 0.0f;
+    if (args.accumulate && active) load_elems<U, V>(out_chunk, acc, false);
 
     if constexpr (KFIX > 0) {
-        uint64_t rows[KFIX];
+        u32x4 raw[KFIX];
         float w[KFIX];
+        bool present[KFIX];
 #pragma unroll
         for (int k = 0; k < KFIX; ++k) {
-            rows[k] = read_lane64c(row_ptr, k);
+            const uint64_t row = read_lane64c(row_ptr, k);
             w[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(weight), k));
+            present[k] = row != 0;
+            raw[k] = u32x4{0, 0, 0, 0};
+            if (present[k] && active) {
+                raw[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row) + c);
+            }
         }
-        for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
-            float y[KFIX][V];
 #pragma unroll
-            for (int k = 0; k < KFIX; ++k) {
-                if (rows[k] != 0) {
-                    load_elems<T, V>(reinterpret_cast<const uint8_t *>(rows[k]) + (size_t)c * 16, y[k],
-                                     true);
-                } else {
-#pragma unroll
-                    for (int j = 0; j < V; ++j) y[k][j] = 0.0f;
-                }
-            }
-            float acc[V];
-            if (args.accumulate) {
-                load_elems<U, V>(out_row + (size_t)c * V * Elem<U>::kSize, acc, false);
-            } else {
-#pragma unroll
-                for (int j = 0; j < V; ++j) acc[j] = 0.0f;
-            }
-#pragma unroll
-            for (int k = 0; k < KFIX; ++k) {
-                if (rows[k] != 0) {
-#pragma unroll
-                    for (int j = 0; j < V; ++j) acc[j] = __builtin_fmaf(w[k], y[k][j], acc[j]);
-                }
-            }
-            store_elems<U, V>(out_row + (size_t)c * V * Elem<U>::kSize, acc);
+        for (int k = 0; k < KFIX; ++k) {
+            if (present[k]) fma_chunk<T, V>(raw[k], w[k], acc);
         }
     } else {
-        for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
-            float acc[V];
-            if (args.accumulate) {
-                load_elems<U, V>(out_row + (size_t)c * V * Elem<U>::kSize, acc, false);
-            } else {
-#pragma unroll
-                for (int j = 0; j < V; ++j) acc[j] = 0.0f;
+        for (uint32_t k = 0; k < K; ++k) {
+            const uint64_t row = read_lane64c(row_ptr, k);
+            const float wk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(weight), (int)k));
+            if (row != 0) {
+                u32x4 raw = {0, 0, 0, 0};
+                if (active) raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row) + c);
+                fma_chunk<T, V>(raw, wk, acc);
             }
-            for (uint32_t k = 0; k < K; ++k) {
-                const uint64_t row = read_lane64c(row_ptr, k);
-                const float wk =
-                    __int_as_float(__builtin_amdgcn_readlane(__float_as_int(weight), (int)k));
-                if (row != 0) {
-                    float y[V];
-                    load_elems<T, V>(reinterpret_cast<const uint8_t *>(row) + (size_t)c * 16, y, true);
-#pragma unroll
-                    for (int j = 0; j < V; ++j) acc[j] = __builtin_fmaf(wk, y[j], acc[j]);
-                }
-            }
-            store_elems<U, V>(out_row + (size_t)c * V * Elem<U>::kSize, acc);
         }
     }
+    if (active) store_elems<U, V>(out_chunk, acc);
 }
 
 template <typename T, typename U>
@@ -232,17 +257,14 @@ static hipError_t launch_typed(const CombArgs &args, const Workspace &ws, uint32
                                hipStream_t stream) {
     constexpr int V = vec_elems<T>();
     const uint32_t chunks = args.hidden_dim / V;
-    uint32_t threads = (chunks + kWave - 1) / kWave * kWave;
-    // Two chunks per lane once a row is wide enough: more bytes in flight per
-    // wavefront, fewer workgroups to schedule.
-    if (threads > 512) threads = ((chunks + 1) / 2 + kWave - 1) / kWave * kWave;
-    if (threads > 1024) threads = 1024;
-    if (threads < (uint32_t)kWave) threads = kWave;
+    const uint32_t slabs = (chunks + kWave - 1) / kWave;
+    const uint64_t units = (uint64_t)total_tokens * slabs;
+    const uint32_t blocks = (uint32_t)((units + kCombineWaves - 1) / kCombineWaves);
     if (ws.topk == 8) {
-        hipLaunchKernelGGL((combine_gather_kernel<T, U, 8>), dim3(total_tokens), dim3(threads), 0,
+        hipLaunchKernelGGL((combine_gather_kernel<T, U, 8>), dim3(blocks), dim3(kCombineWaves * kWave), 0,
                            stream, args, ws);
     } else {
-        hipLaunchKernelGGL((combine_gather_kernel<T, U, 0>), dim3(total_tokens), dim3(threads), 0,
+        hipLaunchKernelGGL((combine_gather_kernel<T, U, 0>), dim3(blocks), dim3(kCombineWaves * kWave), 0,
                            stream, args, ws);
     }
     return hipGetLastError();

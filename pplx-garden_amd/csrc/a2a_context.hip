@@ -271,6 +271,7 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
         return at;
     };
     const size_t o_local = carve((size_t)N * ws.max_tk * sizeof(uint16_t));
+    const size_t o_hist = carve((size_t)N * ws.nb_max * E * sizeof(uint32_t));
     const size_t o_block = carve((size_t)N * ws.nb_max * E * sizeof(uint32_t));
     const size_t o_routed = carve((size_t)N * E * sizeof(uint32_t));
     const size_t o_offsets = carve((size_t)N * E * sizeof(uint32_t));
@@ -295,6 +296,7 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
     }
     uint8_t *base = static_cast<uint8_t *>(ctx->arena);
     ws.local_rank = reinterpret_cast<uint16_t *>(base + o_local);
+    ws.block_hist = reinterpret_cast<uint32_t *>(base + o_hist);
     ws.block_prefix = reinterpret_cast<uint32_t *>(base + o_block);
     ws.num_routed = reinterpret_cast<uint32_t *>(base + o_routed);
     ws.expert_offsets = reinterpret_cast<uint32_t *>(base + o_offsets);
@@ -399,7 +401,8 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
         ra.block_start[r] = blocks;
         pa.token_start[r] = tokens;
     }
-    ra.rank_mask = fa.fold_mask = fa.valid_mask = fa.recv_mask = all_ranks(ctx);
+    fa.fold_mask = fa.valid_mask = fa.recv_mask = all_ranks(ctx);
+
     pa.row_bytes = (uint32_t)row_bytes_of(c);
     pa.hidden_dim = c.hidden_dim;
     pa.hidden_dim_scale = c.hidden_dim_scale;
@@ -563,13 +566,10 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     const uint32_t nb = ceil_div_u32((uint64_t)T * K, kRouteBlock);
     ra.src[rank] = RouteSrc{indices, bound_m, (uint32_t)indices_stride, T};
     for (uint32_t r = 0; r <= (uint32_t)kMaxWorld; ++r) ra.block_start[r] = r <= rank ? 0 : nb;
-    ra.rank_mask = 1u << rank;
     fa.num_blocks[rank] = nb;
     fa.fold_mask = 1u << rank;
     fa.valid_mask = ctx->sent_mask | (1u << rank);
     fa.recv_mask = 0;
-    // Route launches address sources through block_start, so a single source
-    // other than rank 0 needs the grid to start at it.
     hipError_t e = launch_route(ra, ctx->ws, nb, s);
     if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
     e = launch_finalize(fa, ctx->ws, s);

@@ -21,7 +21,8 @@ constexpr int kMaxWorld = A2A_MAX_WORLD_SIZE;
 // are laid out [world][...] with the strides below.
 struct Workspace {
     uint16_t *local_rank;      // [N][max_tk]    rank of an entry among equal experts inside its routing block
-    uint32_t *block_prefix;    // [N][nb_max][E] per-block histogram, turned into an exclusive prefix over blocks
+    uint32_t *block_hist;      // [N][nb_max][E] per-chunk histogram of a source's entries
+    uint32_t *block_prefix;    // [N][nb_max][E] its exclusive prefix over chunks
     uint32_t *num_routed;      // [N][E]         routes per (source, expert)
     uint32_t *expert_offsets;  // [N][E]         inclusive scan of num_routed over experts
     uint32_t *slot_base;       // [N][E]         first receiver row of (source, expert)
@@ -47,12 +48,6 @@ struct RouteSrc {
     uint32_t num_tokens;
 };
 
-struct RouteArgs {
-    RouteSrc src[kMaxWorld];
-    uint32_t block_start[kMaxWorld + 1];  // first routing block of each source in the grid
-    uint32_t rank_mask;                   // sources routed by this launch
-};
-
 struct FinalizeArgs {
     int32_t *out_num_tokens[kMaxWorld];   // per receiver, may be null
     uint32_t out_rows[kMaxWorld];         // rows of the receiver's buffer (overflow check)
@@ -61,6 +56,12 @@ struct FinalizeArgs {
     uint32_t valid_mask;                  // sources that count for the layout (others count as empty)
     uint32_t recv_mask;                   // receivers whose layout is computed by this launch
 };
+
+struct RouteArgs {
+    RouteSrc src[kMaxWorld];
+    uint32_t block_start[kMaxWorld + 1];  // first routing block of each source in the grid
+};
+
 
 struct PushSrc {
     const uint8_t *x;

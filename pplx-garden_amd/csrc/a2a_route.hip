@@ -7,23 +7,197 @@
 // order (a2a_dispatch_send.cu:176-243), and the per-receiver layout the
 // reference computes on a CPU thread (a2a_worker.rs:577-606,621-694).
 //
-// Design for CDNA4: the entries are cut into chunks of 1024, one workgroup of
+// Design for CDNA4, two launches and no device-wide fence or atomic:
+//
+// route_hist_kernel: the entries are cut into chunks of 1024, one workgroup of
 // 16 wavefronts per chunk.  Inside a wavefront, equal expert ids are matched
 // with one 64-bit ballot per id bit (no LDS atomics, so the result does not
 // depend on scheduling); the lane's rank among its matches is a popcount of
 // the match mask below it.  Wavefront totals meet in a [16][E] LDS table whose
-// columns are scanned by E threads.  A second, single-workgroup kernel folds
-// the per-chunk histograms into prefixes and computes all scans.  The rank of
-// an entry is therefore `block_prefix[chunk][e] + local_rank[entry]`, ascending
-// in (token, k): stable, reproducible, and never materialised in a second pass
-// over the entries.
+// columns are scanned by E threads.  The rank of an entry is then
+// `block_prefix[chunk][e] + local_rank[entry]`, ascending in (token, k):
+// stable, reproducible, and never materialised in a second pass over the
+// entries.
+//
+// route_finalize_kernel: one workgroup per logical rank.  Workgroup i turns the
+// chunk histograms of SOURCE i into prefixes over chunks and scans its expert
+// offsets, and lays out RECEIVER i from the chunk histograms of every source.
+// Each workgroup reads what it needs straight from the histograms (one round
+// trip to memory, all loads in flight together), so no workgroup depends on
+// another.
 #include "a2a_internal.h"
 
 namespace a2a {
 
+namespace {
+
+constexpr int kRouteWaves = kRouteBlock / kWave;
+
+// Inclusive scan over the 64 lanes of a wavefront.
+__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, uint32_t lane) {
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        const uint32_t up = __shfl_up(v, d);
+        if (lane >= (uint32_t)d) v += up;
+    }
+    return v;
+}
+
+// Inclusive scan over the first blockDim.x values (one per thread); `scratch`
+// holds one word per wavefront.  Every thread of the workgroup must call.
+__device__ __forceinline__ uint32_t block_inclusive_scan(uint32_t v, uint32_t *scratch) {
+    const uint32_t lane = threadIdx.x & (kWave - 1);
+    const uint32_t wave = threadIdx.x / kWave;
+    const uint32_t incl = wave_inclusive_scan(v, lane);
+    __syncthreads();
+    if (lane == kWave - 1) scratch[wave] = incl;
+    __syncthreads();
+    uint32_t before = 0;
+    for (uint32_t w = 0; w < wave; ++w) before += scratch[w];
+    return before + incl;
+}
+
+// Sum of `n` words spaced `stride` apart, loads batched eight at a time so
+// that they are in flight together.
+__device__ __forceinline__ uint32_t strided_sum(const uint32_t *p, uint32_t n, size_t stride) {
+    uint32_t sum = 0;
+    for (uint32_t b = 0; b < n; b += 8) {
+        uint32_t v[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) v[j] = b + j < n ? p[(size_t)(b + j) * stride] : 0;
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) sum += v[j];
+    }
+    return sum;
+}
+
+// Source part of the finalize: chunk histograms of source `g` -> exclusive
+// prefixes over chunks, per-expert totals, their inclusive scan over experts
+// (a2a_dispatch_send.cu:199-204,209-242).  Whole workgroup.
+__device__ void fold_source(const FinalizeArgs &args, const Workspace &ws, uint32_t g, uint32_t *part_sum,
+                            uint32_t *scratch) {
+    const uint32_t E = ws.num_experts;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t num_blocks = args.num_blocks[g];
+    if (num_blocks == 0) {
+        if (tid < E) {
+            ws.num_routed[g * E + tid] = 0;
+            ws.expert_offsets[g * E + tid] = 0;
+        }
+        return;
+    }
+    const uint32_t parts = blockDim.x / E;   // >= 1: threads that share a column
+    const uint32_t part = tid / E;
+    const uint32_t e0 = tid - part * E;
+    const uint32_t per = (num_blocks + parts - 1) / parts;
+    const bool has_column = part < parts;
+    uint32_t b0 = 0, nb = 0;
+    uint32_t first[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) first[j] = 0;
+    if (has_column) {
+        b0 = part * per < num_blocks ? part * per : num_blocks;
+        const uint32_t b1 = b0 + per < num_blocks ? b0 + per : num_blocks;
+        nb = b1 - b0;
+        const uint32_t *col = ws.block_hist + ((size_t)g * ws.nb_max + b0) * E + e0;
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) first[j] = j < nb ? col[(size_t)j * E] : 0;
+        uint32_t sum = 0;
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) sum += first[j];
+        if (nb > 8) sum += strided_sum(col + (size_t)8 * E, nb - 8, E);
+        part_sum[part * E + e0] = sum;
+    }
+    __syncthreads();
+    uint32_t total = 0;
+    if (has_column) {
+        uint32_t run = 0;
+        for (uint32_t p = 0; p < parts; ++p) {
+            const uint32_t s = part_sum[p * E + e0];
+            if (p < part) run += s;
+            total += s;
+        }
+        const uint32_t *col = ws.block_hist + ((size_t)g * ws.nb_max + b0) * E + e0;
+        uint32_t *out = ws.block_prefix + ((size_t)g * ws.nb_max + b0) * E + e0;
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            if (j < nb) out[(size_t)j * E] = run;
+            run += first[j];
+        }
+        for (uint32_t j = 8; j < nb; ++j) {
+            out[(size_t)j * E] = run;
+            run += col[(size_t)j * E];
+        }
+    }
+    const bool owner = has_column && part == 0;
+    if (owner) ws.num_routed[g * E + e0] = total;
+    const uint32_t incl = block_inclusive_scan(owner ? total : 0, scratch);
+    if (owner) ws.expert_offsets[g * E + e0] = incl;
+}
+
+// Receiver part of the finalize: rows of receiver `r`, from the chunk
+// histograms of the sources folded by this launch and the published counts of
+// the sources that sent earlier in the step.  Whole workgroup; `tot` holds
+// N * Le words.
+__device__ void layout_receiver(const FinalizeArgs &args, const Workspace &ws, uint32_t r, uint32_t *tot,
+                                uint32_t *scratch) {
+    const uint32_t N = ws.world, E = ws.num_experts, Le = ws.experts_per_rank;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t items = N * Le;              // (source, local expert) pairs
+    for (uint32_t i = tid; i < items; i += blockDim.x) tot[i] = 0;
+    __syncthreads();
+    uint32_t parts = blockDim.x / items;
+    if (parts == 0) parts = 1;
+    for (uint32_t w = tid; w < parts * items; w += blockDim.x) {
+        const uint32_t part = w / items;
+        const uint32_t item = w - part * items;
+        const uint32_t g = item / Le;
+        const uint32_t e = r * Le + (item - g * Le);
+        if (e >= E || !(args.valid_mask >> g & 1)) continue;
+        uint32_t sum = 0;
+        if (args.fold_mask >> g & 1) {
+            const uint32_t num_blocks = args.num_blocks[g];
+            const uint32_t per = (num_blocks + parts - 1) / parts;
+            const uint32_t b0 = part * per < num_blocks ? part * per : num_blocks;
+            const uint32_t b1 = b0 + per < num_blocks ? b0 + per : num_blocks;
+            sum = strided_sum(ws.block_hist + ((size_t)g * ws.nb_max + b0) * E + e, b1 - b0, E);
+        } else if (part == 0) {
+            sum = ws.num_routed[g * E + e];
+        }
+        if (sum != 0) atomicAdd(&tot[item], sum);
+    }
+    __syncthreads();
+
+    const uint32_t pad = ws.expert_padding;
+    const uint32_t e = r * Le + tid;
+    const bool mine = tid < Le && e < E;
+    uint32_t tpe = 0;
+    if (mine) {
+        for (uint32_t g = 0; g < N; ++g) tpe += tot[g * Le + tid];
+    }
+    const uint32_t padded = (tpe + pad - 1) / pad * pad;
+    const uint32_t poff = block_inclusive_scan(mine ? padded : 0, scratch) - padded;
+    if (mine) {
+        ws.tokens_per_expert[e] = tpe;
+        ws.padded_offset[e] = poff;
+        if (args.out_num_tokens[r] != nullptr) args.out_num_tokens[r][tid] = (int32_t)tpe;
+        if (poff + tpe > args.out_rows[r]) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+        // Sources in the order the reference's host worker visits them
+        // (a2a_worker.rs:681-694); each gets a contiguous run of rows.
+        uint32_t running = poff;
+        for (uint32_t i = 0; i < N; ++i) {
+            const uint32_t g = source_order(r, i, N, ws.node_size);
+            ws.slot_base[g * E + e] = running;
+            running += tot[g * Le + tid];
+        }
+    }
+}
+
+}  // namespace
+
 __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs args,
                                                                  const Workspace ws) {
-    __shared__ uint16_t wave_hist[kRouteBlock / kWave][A2A_MAX_EXPERTS];
+    __shared__ uint16_t wave_hist[kRouteWaves][A2A_MAX_EXPERTS];
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
@@ -38,9 +212,7 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
     const RouteSrc src = args.src[g];
     const uint32_t num_entries = effective_tokens(src.bound_m, src.num_tokens) * K;
 
-    for (uint32_t i = tid; i < (kRouteBlock / kWave) * E; i += kRouteBlock) {
-        wave_hist[i / E][i % E] = 0;
-    }
+    for (uint32_t i = tid; i < kRouteWaves * E; i += kRouteBlock) wave_hist[i / E][i % E] = 0;
     __syncthreads();
 
     const uint32_t entry = chunk * kRouteBlock + tid;
@@ -49,8 +221,7 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
     if (valid) {
         const uint32_t token = entry / K;
         const uint32_t k = entry - token * K;
-        expert = (uint32_t)__builtin_nontemporal_load(
-            &src.indices[(size_t)token * src.indices_stride + k]);
+        expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + k];
         if (expert >= E) {
             valid = false;
             atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
@@ -66,17 +237,15 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
         peers &= bit ? set : ~set;
     }
     const uint32_t rank_in_wave = __popcll(peers & ((1ull << lane) - 1));
-    if (valid && rank_in_wave == 0) {
-        wave_hist[wave][expert] = (uint16_t)__popcll(peers);
-    }
+    if (valid && rank_in_wave == 0) wave_hist[wave][expert] = (uint16_t)__popcll(peers);
     __syncthreads();
 
     // Exclusive scan of each expert's column over the 16 wavefronts.
-    uint32_t *block_hist = ws.block_prefix + ((size_t)g * ws.nb_max + chunk) * E;
+    uint32_t *block_hist = ws.block_hist + ((size_t)g * ws.nb_max + chunk) * E;
     for (uint32_t e = tid; e < E; e += kRouteBlock) {
         uint32_t run = 0;
 #pragma unroll
-        for (int w = 0; w < kRouteBlock / kWave; ++w) {
+        for (int w = 0; w < kRouteWaves; ++w) {
             const uint32_t c = wave_hist[w][e];
             wave_hist[w][e] = (uint16_t)run;
             run += c;
@@ -91,101 +260,17 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
     }
 }
 
-// Inclusive scan over the 64 lanes of a wavefront.
-__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, uint32_t lane) {
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        const uint32_t up = __shfl_up(v, d);
-        if (lane >= (uint32_t)d) v += up;
-    }
-    return v;
-}
-
-// One workgroup.  Dynamic LDS: counts[N*E] then scratch[E + 32].
-__global__ __launch_bounds__(1024) void route_finalize_kernel(const FinalizeArgs args,
-                                                              const Workspace ws) {
-    extern __shared__ uint32_t lds[];
-    const uint32_t N = ws.world;
-    const uint32_t E = ws.num_experts;
-    const uint32_t Le = ws.experts_per_rank;
-    uint32_t *cnt = lds;               // [N][E]
-    uint32_t *excl = lds + N * E;      // [E] exclusive scan of padded counts
-    uint32_t *wave_tot = excl + E;     // [16]
-
-    const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & (kWave - 1);
-    const uint32_t wave = tid / kWave;
-    const uint32_t nwaves = blockDim.x / kWave;
-
-    // 1. Per (source, expert): exclusive prefix of the chunk histograms, total.
-    for (uint32_t p = tid; p < N * E; p += blockDim.x) {
-        const uint32_t g = p / E;
-        const uint32_t e = p - g * E;
-        uint32_t run = 0;
-        if (args.fold_mask >> g & 1) {
-            uint32_t *col = ws.block_prefix + (size_t)g * ws.nb_max * E + e;
-            for (uint32_t b = 0; b < args.num_blocks[g]; ++b) {
-                const uint32_t c = col[(size_t)b * E];
-                col[(size_t)b * E] = run;
-                run += c;
-            }
-            ws.num_routed[p] = run;
-        } else if (args.valid_mask >> g & 1) {
-            run = ws.num_routed[p];
-        }
-        cnt[p] = run;
-    }
-    __syncthreads();
-
-    // 2. Inclusive scan over experts for every folded source (a2a_dispatch_send.cu:209-242).
-    for (uint32_t g = wave; g < N; g += nwaves) {
-        if (!(args.fold_mask >> g & 1)) continue;
-        uint32_t carry = 0;
-        for (uint32_t base = 0; base < E; base += kWave) {
-            const uint32_t e = base + lane;
-            const uint32_t v = e < E ? cnt[g * E + e] : 0;
-            const uint32_t incl = wave_inclusive_scan(v, lane) + carry;
-            if (e < E) ws.expert_offsets[g * E + e] = incl;
-            carry = __shfl(incl, kWave - 1);
-        }
-    }
-
-    if (args.recv_mask == 0) return;
-
-    // 3. Receiver layout.  Thread e owns expert e (E <= blockDim.x).
-    const uint32_t pad = ws.expert_padding;
-    uint32_t tpe = 0, padded = 0;
-    if (tid < E) {
-        for (uint32_t g = 0; g < N; ++g) tpe += cnt[g * E + tid];
-        padded = (tpe + pad - 1) / pad * pad;
-    }
-    const uint32_t incl = wave_inclusive_scan(padded, lane);
-    if (lane == kWave - 1) wave_tot[wave] = incl;
-    __syncthreads();
-    uint32_t before = 0;
-    for (uint32_t w = 0; w < wave; ++w) before += wave_tot[w];
-    if (tid < E) excl[tid] = before + incl - padded;
-    __syncthreads();
-
-    if (tid < E) {
-        const uint32_t e = tid;
-        const uint32_t r = e / Le;
-        if (args.recv_mask >> r & 1) {
-            const uint32_t le = e - r * Le;
-            const uint32_t poff = excl[e] - excl[r * Le];
-            ws.tokens_per_expert[e] = tpe;
-            ws.padded_offset[e] = poff;
-            if (args.out_num_tokens[r] != nullptr) args.out_num_tokens[r][le] = (int32_t)tpe;
-            if (poff + tpe > args.out_rows[r]) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
-            // Sources in the order the reference's host worker visits them
-            // (a2a_worker.rs:681-694); each gets a contiguous run of rows.
-            uint32_t running = poff;
-            for (uint32_t i = 0; i < N; ++i) {
-                const uint32_t g = source_order(r, i, N, ws.node_size);
-                ws.slot_base[g * E + e] = running;
-                running += cnt[g * E + e];
-            }
-        }
+// One workgroup per logical rank: source part, then receiver part.
+__global__ __launch_bounds__(kRouteBlock) void route_finalize_kernel(const FinalizeArgs args,
+                                                                     const Workspace ws) {
+    __shared__ uint32_t part_sum[kRouteBlock];
+    __shared__ uint32_t tot[A2A_MAX_EXPERTS + kMaxWorld];
+    __shared__ uint32_t scratch[kRouteWaves];
+    const uint32_t rank = blockIdx.x;
+    if (args.fold_mask >> rank & 1) fold_source(args, ws, rank, part_sum, scratch);
+    if (args.recv_mask >> rank & 1) {
+        __syncthreads();
+        layout_receiver(args, ws, rank, tot, scratch);
     }
 }
 
@@ -197,10 +282,7 @@ hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t tot
 }
 
 hipError_t launch_finalize(const FinalizeArgs &args, const Workspace &ws, hipStream_t stream) {
-    const size_t lds = ((size_t)ws.world * ws.num_experts + ws.num_experts + 32) * sizeof(uint32_t);
-    uint32_t threads = (ws.num_experts + kWave - 1) / kWave * kWave;
-    if (threads < 256) threads = 256;
-    hipLaunchKernelGGL(route_finalize_kernel, dim3(1), dim3(threads), lds, stream, args, ws);
+    hipLaunchKernelGGL(route_finalize_kernel, dim3(ws.world), dim3(kRouteBlock), 0, stream, args, ws);
     return hipGetLastError();
 }
 

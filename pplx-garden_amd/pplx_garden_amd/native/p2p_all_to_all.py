@@ -263,21 +263,28 @@ class AllToAllContext:
 
     # -- the two group calls ------------------------------------------------
 
-    def dispatch(self, per_rank: Sequence[A2ADispatchArgs], quantize: bool, stream: int) -> None:
-        self._require_open()
+    def pack_dispatch_args(self, per_rank: Sequence[A2ADispatchArgs]):
+        """The C array `a2a_dispatch` takes; build it once when the buffers do not change."""
         if len(per_rank) != self.world_size:
             raise RuntimeError(f"expected arguments of {self.world_size} ranks, got {len(per_rank)}")
-        arr = (A2ADispatchArgs * self.world_size)(*per_rank)
+        return (A2ADispatchArgs * self.world_size)(*per_rank)
+
+    def pack_combine_args(self, per_rank: Sequence[A2ACombineArgs]):
+        if len(per_rank) != self.world_size:
+            raise RuntimeError(f"expected arguments of {self.world_size} ranks, got {len(per_rank)}")
+        return (A2ACombineArgs * self.world_size)(*per_rank)
+
+    def dispatch(self, per_rank, quantize: bool, stream: int) -> None:
+        """`per_rank`: one A2ADispatchArgs per rank, or the array from pack_dispatch_args."""
+        self._require_open()
+        arr = per_rank if isinstance(per_rank, ctypes.Array) else self.pack_dispatch_args(per_rank)
         self._check(self._lib.a2a_dispatch(self._handle, arr, int(quantize), _ptr(stream)))
 
-    def combine(self, per_rank: Sequence[A2ACombineArgs], expert_y_dtype: torch.dtype,
-                accumulate: bool, stream: int) -> None:
+    def combine(self, per_rank, expert_y_dtype: torch.dtype, accumulate: bool, stream: int) -> None:
         self._require_open()
-        if len(per_rank) != self.world_size:
-            raise RuntimeError(f"expected arguments of {self.world_size} ranks, got {len(per_rank)}")
         if expert_y_dtype not in SCALAR_TYPE:
             raise RuntimeError(f"unsupported expert_y dtype {expert_y_dtype}")
-        arr = (A2ACombineArgs * self.world_size)(*per_rank)
+        arr = per_rank if isinstance(per_rank, ctypes.Array) else self.pack_combine_args(per_rank)
         self._check(self._lib.a2a_combine(
             self._handle, arr, SCALAR_TYPE[expert_y_dtype], int(bool(accumulate)), _ptr(stream)))
 
