@@ -140,7 +140,15 @@ __device__ __forceinline__ void fma_chunk(const u32x4 raw, float w, float (&acc)
     }
 }
 
-constexpr int kCombineWaves = 4;  // wavefronts per workgroup; each works on its own
+#ifndef A2A_COMBINE_WAVES
+#define A2A_COMBINE_WAVES 1
+#endif
+#ifndef A2A_COMBINE_CHUNKS
+#define A2A_COMBINE_CHUNKS 1
+#endif
+constexpr int kCombineWaves = A2A_COMBINE_WAVES;    // wavefronts per workgroup; each works on its own
+constexpr int kCombineChunks = A2A_COMBINE_CHUNKS;  // 16-byte chunks of a row per lane
+constexpr int kSlabChunks = kWave * kCombineChunks;
 
 // T: type of the expert_y rows, U: type of out_tokens.  One WAVEFRONT handles
 // one slab of 64 sixteen-byte chunks of one token; wavefronts share nothing, so
@@ -156,7 +164,7 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
     const uint32_t E = ws.num_experts;
     const uint32_t K = KFIX > 0 ? (uint32_t)KFIX : ws.topk;
     const uint32_t num_chunks = args.hidden_dim / V;
-    const uint32_t slabs = (num_chunks + kWave - 1) / kWave;
+    const uint32_t slabs = (num_chunks + kSlabChunks - 1) / kSlabChunks;
 
     const uint32_t unit = blockIdx.x * kCombineWaves + wave;
     const uint32_t token_global = unit / slabs;
@@ -212,16 +220,22 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
         if (!ok && slab == 0) atomicOr(ws.err, A2A_DEV_BAD_SLOT);
     }
 
-    const uint32_t c = slab * kWave + lane;
-    const bool active = c < num_chunks;
-    uint8_t *out_chunk = dst.out + (size_t)token * dst.out_stride + (size_t)c * V * Elem<U>::kSize;
-    float acc[V];
+    uint32_t c[kCombineChunks];
+    bool active[kCombineChunks];
+    uint8_t *out_chunk[kCombineChunks];
+    float acc[kCombineChunks][V];
 #pragma unroll
-    for (int j = 0; j < V; ++j) acc[j] = 0.0f;
-    if (args.accumulate && active) load_elems<U, V>(out_chunk, acc, false);
+    for (int u = 0; u < kCombineChunks; ++u) {
+        c[u] = slab * kSlabChunks + u * kWave + lane;
+        active[u] = c[u] < num_chunks;
+        out_chunk[u] = dst.out + (size_t)token * dst.out_stride + (size_t)c[u] * V * Elem<U>::kSize;
+#pragma unroll
+        for (int j = 0; j < V; ++j) acc[u][j] = 0.0f;
+        if (args.accumulate && active[u]) load_elems<U, V>(out_chunk[u], acc[u], false);
+    }
 
     if constexpr (KFIX > 0) {
-        u32x4 raw[KFIX];
+        u32x4 raw[kCombineChunks][KFIX];
         float w[KFIX];
         bool present[KFIX];
 #pragma unroll
@@ -229,27 +243,39 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
             const uint64_t row = read_lane64c(row_ptr, k);
             w[k] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(weight), k));
             present[k] = row != 0;
-            raw[k] = u32x4{0, 0, 0, 0};
-            if (present[k] && active) {
-                raw[k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row) + c);
+#pragma unroll
+            for (int u = 0; u < kCombineChunks; ++u) {
+                raw[u][k] = u32x4{0, 0, 0, 0};
+                if (present[k] && active[u]) {
+                    raw[u][k] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row) + c[u]);
+                }
             }
         }
 #pragma unroll
-        for (int k = 0; k < KFIX; ++k) {
-            if (present[k]) fma_chunk<T, V>(raw[k], w[k], acc);
+        for (int u = 0; u < kCombineChunks; ++u) {
+#pragma unroll
+            for (int k = 0; k < KFIX; ++k) {
+                if (present[k]) fma_chunk<T, V>(raw[u][k], w[k], acc[u]);
+            }
         }
     } else {
         for (uint32_t k = 0; k < K; ++k) {
             const uint64_t row = read_lane64c(row_ptr, k);
             const float wk = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(weight), (int)k));
             if (row != 0) {
-                u32x4 raw = {0, 0, 0, 0};
-                if (active) raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row) + c);
-                fma_chunk<T, V>(raw, wk, acc);
+#pragma unroll
+                for (int u = 0; u < kCombineChunks; ++u) {
+                    u32x4 raw = {0, 0, 0, 0};
+                    if (active[u]) raw = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(row) + c[u]);
+                    fma_chunk<T, V>(raw, wk, acc[u]);
+                }
             }
         }
     }
-    if (active) store_elems<U, V>(out_chunk, acc);
+#pragma unroll
+    for (int u = 0; u < kCombineChunks; ++u) {
+        if (active[u]) store_elems<U, V>(out_chunk[u], acc[u]);
+    }
 }
 
 template <typename T, typename U>
@@ -257,7 +283,7 @@ static hipError_t launch_typed(const CombArgs &args, const Workspace &ws, uint32
                                hipStream_t stream) {
     constexpr int V = vec_elems<T>();
     const uint32_t chunks = args.hidden_dim / V;
-    const uint32_t slabs = (chunks + kWave - 1) / kWave;
+    const uint32_t slabs = (chunks + kSlabChunks - 1) / kSlabChunks;
     const uint64_t units = (uint64_t)total_tokens * slabs;
     const uint32_t blocks = (uint32_t)((units + kCombineWaves - 1) / kCombineWaves);
     if (ws.topk == 8) {
