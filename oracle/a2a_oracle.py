@@ -381,9 +381,10 @@ def e4m3fn_encode(f: np.ndarray) -> np.ndarray:
     and 2^(e-3) in the binade of 2^e.  No saturation: a magnitude that rounds
     beyond 448 becomes the NaN code 0x7F, like torch's cast.
     """
-    f = np.asarray(f, dtype=np.float32)
+    f = np.ascontiguousarray(f, dtype=np.float32)
     sign = (f.view(np.uint32) >> 24).astype(np.uint8) & 0x80
-    a = np.abs(f).astype(np.float64)
+    with np.errstate(invalid="ignore"):
+        a = np.abs(f).astype(np.float64)
     nan = np.isnan(a)
     a = np.where(nan, 0.0, a)
     inf = np.isinf(a)

@@ -1,0 +1,242 @@
+"""bound_m, accumulate, element types, error reporting and the quantiser on every bf16 value."""
+
+from dataclasses import replace
+
+import numpy as np
+import pytest
+import torch
+
+import a2a_oracle as oracle
+from a2a_cases import C0, C1, bf16_codes, make_world
+from a2a_harness import SENTINEL, make_ops, rows_needed, run_oracle
+from a2a_transport import RefConfig, make_ref_rank, oracle_combine, oracle_dispatch, rows_for
+from a2a_transport import make_ops as make_transport_ops
+from pplx_garden_amd.native import p2p_all_to_all as native
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+
+
+def test_quantiser_on_every_bf16_value_and_many_scales():
+    """Each group of 128 holds a run of consecutive bf16 codes plus one element that sets the
+    group maximum, so every finite bf16 value meets many different scales."""
+    H = 2048
+    codes = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    finite = codes[np.isfinite(oracle.bf16_to_f32(codes))]
+    rng = np.random.default_rng(17)
+    groups = []
+    for rep, top in enumerate([1e-3, 0.11, 1.0, 7.5, 300.0, 3e4, 1e9, 3e38]):
+        vals = finite.copy()
+        rng.shuffle(vals)
+        vals = vals[: len(vals) // 127 * 127].reshape(-1, 127)
+        top_code = oracle.f32_to_bf16(np.full((vals.shape[0], 1), top, dtype=np.float32))
+        groups.append(np.concatenate([vals, top_code], axis=1))
+    g = np.concatenate(groups, axis=0)
+    g = g[: g.shape[0] // (H // 128) * (H // 128)]
+    x_codes = g.reshape(-1, H)
+    T = x_codes.shape[0]
+    case = replace(C0, name="quant_all", num_tokens=T, topk=1, num_experts=4, world_size=1)
+    x = torch.from_numpy(x_codes.view(np.int16).copy()).view(torch.bfloat16)
+    idx = torch.zeros((T, 1), dtype=torch.int32)
+    w = torch.ones((T, 1), dtype=torch.float32)
+    _, ops = make_ops(case, DEV, max_num_tokens=T)
+    try:
+        n = torch.zeros(4, dtype=torch.int32, device=DEV)
+        ox = torch.zeros((T, H), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn)
+        os_ = torch.zeros((T, H // 128), dtype=torch.float32, device=DEV)
+        ops[0].dispatch(out_expert_num_tokens=n, out_expert_x=ox, out_expert_x_scale=os_, dp_x=x.to(DEV),
+                        dp_x_scale=None, indices=idx.view(torch.uint32).to(DEV), weights=w.to(DEV))
+        torch.cuda.synchronize(DEV)
+        assert ops[0].context.status() == 0
+        q, s = oracle.quantize_block128(x_codes)
+        np.testing.assert_array_equal(ox.view(torch.uint8).cpu().numpy(), q)       # one expert, token order
+        np.testing.assert_array_equal(os_.cpu().numpy().view(np.uint32), s.view(np.uint32))
+        assert n.cpu().tolist() == [T, 0, 0, 0]
+    finally:
+        ops[0].destroy()
+
+
+@pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
+def test_bound_m_limits_the_tokens(split):
+    case = C0
+    world = make_world(case, "all")
+    bounds = [case.num_tokens, 0, 17, 1]
+    rows = rows_needed(case, world)
+    N, Le, H, Hs = case.world_size, case.experts_per_rank, case.hidden_dim, case.hidden_dim_scale
+    inputs = [oracle.RankInput(x=bf16_codes(rd.x), indices=rd.indices.numpy(), bound_m=b) for rd, b in zip(world, bounds)]
+    want = oracle.dispatch_world(inputs, num_experts=case.num_experts, world_size=N, node_size=N,
+                                 expert_padding=1, out_rows=rows, quantize=True)
+    _, ops = make_ops(case, DEV)
+    try:
+        t = []
+        for r, rd in enumerate(world):
+            t.append(dict(x=rd.x.to(DEV), idx=rd.indices_u32.to(DEV), w=rd.weights.to(DEV),
+                          b=torch.tensor([bounds[r]], dtype=torch.int32, device=DEV),
+                          n=torch.full((Le,), -1, dtype=torch.int32, device=DEV),
+                          ox=torch.full((rows, H), SENTINEL, dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn),
+                          os=torch.full((rows, Hs), -7.0, dtype=torch.float32, device=DEV),
+                          o=torch.full((rd.x.shape[0], H), 3.0, dtype=torch.bfloat16, device=DEV)))
+        phases = [dict(do_send=True, do_recv=False), dict(do_send=False, do_recv=True)] if split else [dict()]
+        for ph in phases:
+            for r in range(N):
+                ops[r].dispatch(out_expert_num_tokens=t[r]["n"], out_expert_x=t[r]["ox"], out_expert_x_scale=t[r]["os"],
+                                dp_x=t[r]["x"], dp_x_scale=None, indices=t[r]["idx"], weights=t[r]["w"],
+                                bound_m=t[r]["b"], **ph)
+        torch.cuda.synchronize(DEV)
+        assert ops[0].context.status() == 0
+        ys = []
+        for r in range(N):
+            np.testing.assert_array_equal(t[r]["n"].cpu().numpy(), want[r].num_tokens)
+            wr = want[r].written
+            got_x = t[r]["ox"].view(torch.uint8).cpu().numpy()
+            np.testing.assert_array_equal(got_x[wr], want[r].x[wr])
+            assert (got_x[~wr] == SENTINEL).all()
+            y = oracle.f32_to_bf16(np.where(wr[:, None], oracle.dequantize_block128(want[r].x, want[r].x_scale), 0).astype(np.float32))
+            ys.append(y)
+        yd = [torch.from_numpy(y.view(np.int16)).view(torch.bfloat16).to(DEV) for y in ys]
+        for ph in phases:
+            for r in range(N):
+                ops[r].combine(out_tokens=t[r]["o"], indices=t[r]["idx"], weights=t[r]["w"], expert_y=yd[r],
+                               bound_m=t[r]["b"], **ph)
+        torch.cuda.synchronize(DEV)
+        assert ops[0].context.status() == 0
+        comb = oracle.combine_world(ys, [rd.indices.numpy() for rd in world], [rd.weights.numpy() for rd in world],
+                                    want[0].slots, num_experts=case.num_experts, world_size=N, bound_m=bounds)
+        for g in range(N):
+            got = t[g]["o"].view(torch.int16).cpu().numpy().view(np.uint16)
+            b = bounds[g]
+            np.testing.assert_allclose(oracle.bf16_to_f32(got[:b]), oracle.bf16_to_f32(comb[g][:b]), rtol=1e-2, atol=1e-3)
+            assert (oracle.bf16_to_f32(got[b:]) == 3.0).all()          # tokens beyond bound_m are not written
+    finally:
+        for op in ops:
+            op.destroy()
+
+
+@pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
+@pytest.mark.parametrize("in_dtype,out_dtype", [
+    (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32), (torch.float16, torch.float16),
+    (torch.bfloat16, torch.float32), (torch.float16, torch.float32),
+], ids=lambda d: str(d).split(".")[-1])
+def test_combine_types_and_accumulate(in_dtype, out_dtype, split):
+    """expert_y in {f16, bf16, f32} x out in {f16, bf16, f32} (launch_utils.cuh:183-194), with and
+    without accumulate (a2a_combine_recv.cu:132).  The split calls stage rows sized for the
+    output type, so there expert_y has the output's element size."""
+    if split and in_dtype.itemsize != out_dtype.itemsize:
+        pytest.skip("staging rows are sized for out_dtype")
+    cfg = RefConfig("types", 4, 1, 48, 16, 256, None, 4, torch.bfloat16, out_dtype, None)
+    world = [make_ref_rank(cfg, r) for r in range(4)]
+    rows = rows_for(cfg, world)
+    want = oracle_dispatch(cfg, world, rows)
+    gen = torch.Generator().manual_seed(9)
+    ys = [torch.randn((rows, cfg.hidden_dim), generator=gen).to(in_dtype) for _ in range(4)]
+    prev = [torch.randn((cfg.max_num_tokens, cfg.hidden_dim), generator=gen).to(out_dtype) for _ in range(4)]
+    ops = make_transport_ops(cfg, DEV)
+    try:
+        t = []
+        for r, rd in enumerate(world):
+            t.append(dict(x=rd.dp_x.to(DEV), idx=rd.indices.view(torch.uint32).to(DEV), w=rd.weights.to(DEV),
+                          n=torch.zeros(4, dtype=torch.int32, device=DEV),
+                          ox=torch.zeros((rows, cfg.hidden_dim), dtype=torch.bfloat16, device=DEV), y=ys[r].to(DEV)))
+        phases = [dict(do_send=True, do_recv=False), dict(do_send=False, do_recv=True)] if split else [dict()]
+        for ph in phases:
+            for r in range(4):
+                ops[r].dispatch(out_expert_num_tokens=t[r]["n"], out_expert_x=t[r]["ox"], out_expert_x_scale=None,
+                                dp_x=t[r]["x"], dp_x_scale=None, indices=t[r]["idx"], weights=t[r]["w"], **ph)
+        for accumulate in (False, True):
+            outs = [p.clone().to(DEV) for p in prev]
+            for ph in phases:
+                for r in range(4):
+                    ops[r].combine(out_tokens=outs[r], indices=t[r]["idx"], weights=t[r]["w"], expert_y=t[r]["y"],
+                                   accumulate=accumulate, **ph)
+            torch.cuda.synchronize(DEV)
+            assert ops[0].context.status() == 0
+            prev_np = None
+            if accumulate:
+                prev_np = [p.numpy() if out_dtype == torch.float32 else p.view(torch.int16).numpy().view(np.uint16) for p in prev]
+            comb = oracle_combine(cfg, world, ys, want[0].slots, out_prev=prev_np)
+            for g in range(4):
+                got = outs[g].cpu().to(torch.float32).numpy()
+                ref = comb[g] if out_dtype == torch.float32 else (
+                    oracle.bf16_to_f32(comb[g]) if out_dtype == torch.bfloat16 else oracle.f16_to_f32(comb[g]))
+                tol = 1e-5 if out_dtype == torch.float32 and in_dtype == torch.float32 else 1e-2
+                np.testing.assert_allclose(got, ref, rtol=tol, atol=tol)
+    finally:
+        for op in ops:
+            op.destroy()
+
+
+def test_errors_are_reported_not_faulted():
+    case = C0
+    world = make_world(case, "one")
+    N, Le, H, Hs = case.world_size, case.experts_per_rank, case.hidden_dim, case.hidden_dim_scale
+    _, ops = make_ops(case, DEV)
+    try:
+        ctx = ops[0].context
+        rd = world[0]
+        bad = rd.indices.clone()
+        bad[3, 1] = case.num_experts + 5                 # an expert id out of range: that copy is dropped
+        rows = 4                                           # far too few rows: overflowing copies are dropped
+        t = [dict(n=torch.zeros(Le, dtype=torch.int32, device=DEV),
+                  ox=torch.full((rows, H), SENTINEL, dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn),
+                  os=torch.zeros((rows, Hs), dtype=torch.float32, device=DEV)) for _ in range(N)]
+        x = rd.x.to(DEV)
+        w = rd.weights.to(DEV)
+        for r in range(N):
+            xr = x if r == 0 else x[:0]
+            ir = (bad if r == 0 else bad[:0]).view(torch.uint32).to(DEV)
+            ops[r].dispatch(out_expert_num_tokens=t[r]["n"], out_expert_x=t[r]["ox"], out_expert_x_scale=t[r]["os"],
+                            dp_x=xr, dp_x_scale=None, indices=ir, weights=w if r == 0 else w[:0])
+        flags = ctx.status()
+        assert flags & native.DEV_BAD_EXPERT_ID and flags & native.DEV_RECV_OVERFLOW
+        assert ctx.status() == 0                           # reading clears the word
+        # host-side errors: too many tokens (a2a_context.rs:290-292), bad rank, combine before dispatch
+        big = torch.zeros((case.num_tokens + 1, H), dtype=torch.bfloat16, device=DEV)
+        with pytest.raises(RuntimeError, match="exceeds maximum"):
+            ctx.dispatch_send(0, case.num_tokens + 1, big.data_ptr(), 2 * H, None, None, None, bad.data_ptr(),
+                              case.topk, 0, case.topk, None, 0, quantize=True)
+        with pytest.raises(RuntimeError, match="rank"):
+            ctx.dispatch_recv(N, 0, 0, H, 0, None, None, None, 0)
+        with pytest.raises(RuntimeError, match="16-byte"):
+            ctx.dispatch_send(0, 4, x.data_ptr() + 2, 2 * H, None, None, None, bad.data_ptr(), case.topk, 0,
+                              case.topk, None, 0, quantize=True)
+    finally:
+        for op in ops:
+            op.destroy()
+    _, ops = make_ops(case, DEV)
+    try:
+        ctx = ops[0].context
+        with pytest.raises(RuntimeError, match="before"):
+            ctx.dispatch_recv(0, 0, 0, H, 0, None, None, None, 0)
+        with pytest.raises(RuntimeError, match="a2a_dispatch"):
+            ctx.combine([native.A2ACombineArgs() for _ in range(N)], torch.bfloat16, False, 0)
+    finally:
+        for op in ops:
+            op.destroy()
+
+
+def test_operator_asserts_like_the_reference():
+    case = C0
+    _, ops = make_ops(case, DEV)
+    try:
+        Le, H, Hs, K = case.experts_per_rank, case.hidden_dim, case.hidden_dim_scale, case.topk
+        good = dict(out_expert_num_tokens=torch.zeros(Le, dtype=torch.int32, device=DEV),
+                    out_expert_x=torch.zeros((8, H), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn),
+                    out_expert_x_scale=torch.zeros((8, Hs), dtype=torch.float32, device=DEV),
+                    dp_x=torch.zeros((2, H), dtype=torch.bfloat16, device=DEV), dp_x_scale=None,
+                    indices=torch.zeros((2, K), dtype=torch.int32, device=DEV).view(torch.uint32),
+                    weights=torch.zeros((2, K), dtype=torch.float32, device=DEV))
+        for key, value in [
+            ("out_expert_num_tokens", torch.zeros(Le + 1, dtype=torch.int32, device=DEV)),    # p2p_all_to_all.py:337
+            ("out_expert_num_tokens", torch.zeros(Le, dtype=torch.int64, device=DEV)),         # :339
+            ("out_expert_x", torch.zeros((8, H), dtype=torch.bfloat16, device=DEV)),           # :346
+            ("indices", torch.zeros((2, K), dtype=torch.int32, device=DEV)),                   # :393 uint32 only
+            ("weights", torch.zeros((2, K), dtype=torch.float64, device=DEV)),                 # :400
+            ("bound_m", torch.zeros(2, dtype=torch.int32, device=DEV)),                        # :407
+        ]:
+            with pytest.raises(AssertionError):
+                ops[0].dispatch(**{**good, key: value})
+        with pytest.raises(AssertionError):
+            ops[0].dispatch(**good, do_send=False, do_recv=False)                              # :332
+    finally:
+        for op in ops:
+            op.destroy()
