@@ -187,6 +187,9 @@ def main() -> int:
     ap.add_argument("--routings", type=int, default=4, help="distinct routings cycled over the steps")
     ap.add_argument("--cpu-reps", type=int, default=3, help="repetitions of the CPU baseline (0 = skip)")
     ap.add_argument("--no-decode", action="store_true", help="skip the 128-token shape")
+    ap.add_argument("--probe-copy", action="store_true",
+                    help="also run plain device-to-device copies of 512 MiB (torch's copy kernel): the "
+                         "known-size kernel that hardware byte counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: every logical rank of the expert-parallel group lives in "
@@ -202,6 +205,14 @@ def main() -> int:
         return 3
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+
+    if args.probe_copy:
+        src = torch.empty(512 << 20, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize(device)
+        del src, dst
 
     case = C3
     wl = Workload(case, device, args.routings)

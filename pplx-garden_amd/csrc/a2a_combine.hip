@@ -226,7 +226,11 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
     float acc[kCombineChunks][V];
 #pragma unroll
     for (int u = 0; u < kCombineChunks; ++u) {
+#ifdef A2A_COMBINE_ADJ
+        c[u] = slab * kSlabChunks + lane * kCombineChunks + u;
+#else
         c[u] = slab * kSlabChunks + u * kWave + lane;
+#endif
         active[u] = c[u] < num_chunks;
         out_chunk[u] = dst.out + (size_t)token * dst.out_stride + (size_t)c[u] * V * Elem<U>::kSize;
 #pragma unroll

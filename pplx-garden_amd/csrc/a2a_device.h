@@ -51,9 +51,7 @@ __device__ __forceinline__ u32x4 quantize16(const u32x4 a, const u32x4 b, float 
         float v[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            v[i] = f[4 * j + i] * inv;
-            v[i] = v[i] > 448.0f ? 448.0f : v[i];
-            v[i] = v[i] < -448.0f ? -448.0f : v[i];
+            v[i] = __builtin_amdgcn_fmed3f(f[4 * j + i] * inv, -448.0f, 448.0f);
         }
         int w = 0;
         w = __builtin_amdgcn_cvt_pk_fp8_f32(v[0], v[1], w, false);

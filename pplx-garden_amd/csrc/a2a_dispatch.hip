@@ -136,7 +136,10 @@ hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool 
                                 uint32_t total_tokens, hipStream_t stream) {
     if (total_tokens == 0) return hipSuccess;
     const uint32_t chunks = quantize ? args.hidden_dim / 16 : args.row_bytes / 16;
-    uint32_t threads = (chunks + kWave - 1) / kWave * kWave;
+#ifndef A2A_PUSH_SLABS
+#define A2A_PUSH_SLABS 1
+#endif
+    uint32_t threads = ((chunks + kWave - 1) / kWave + A2A_PUSH_SLABS - 1) / A2A_PUSH_SLABS * kWave;
     if (threads < (uint32_t)kWave) threads = kWave;
     if (threads > 1024) threads = 1024;
     if (quantize) {

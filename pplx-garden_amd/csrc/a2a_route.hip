@@ -19,12 +19,12 @@
 // stable, reproducible, and never materialised in a second pass over the
 // entries.
 //
-// route_finalize_kernel: one workgroup per logical rank.  Workgroup i turns the
-// chunk histograms of SOURCE i into prefixes over chunks and scans its expert
-// offsets, and lays out RECEIVER i from the chunk histograms of every source.
-// Each workgroup reads what it needs straight from the histograms (one round
-// trip to memory, all loads in flight together), so no workgroup depends on
-// another.
+// route_finalize_kernel: two workgroups per logical rank.  Workgroup i turns
+// the chunk histograms of SOURCE i into prefixes over chunks and scans its
+// expert offsets; workgroup N + i lays out RECEIVER i from the chunk histograms
+// of every source.  Each workgroup reads what it needs straight from the
+// histograms (one round trip to memory, all loads in flight together), so no
+// workgroup depends on another.
 #include "a2a_internal.h"
 
 namespace a2a {
@@ -212,7 +212,10 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
     const RouteSrc src = args.src[g];
     const uint32_t num_entries = effective_tokens(src.bound_m, src.num_tokens) * K;
 
-    for (uint32_t i = tid; i < kRouteWaves * E; i += kRouteBlock) wave_hist[i / E][i % E] = 0;
+    if (tid < E) {
+#pragma unroll
+        for (int w = 0; w < kRouteWaves; ++w) wave_hist[w][tid] = 0;
+    }
     __syncthreads();
 
     const uint32_t entry = chunk * kRouteBlock + tid;
@@ -260,17 +263,19 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
     }
 }
 
-// One workgroup per logical rank: source part, then receiver part.
+// Two workgroups per logical rank, independent of each other: workgroup i folds
+// source i, workgroup N + i lays out receiver i.
 __global__ __launch_bounds__(kRouteBlock) void route_finalize_kernel(const FinalizeArgs args,
                                                                      const Workspace ws) {
     __shared__ uint32_t part_sum[kRouteBlock];
     __shared__ uint32_t tot[A2A_MAX_EXPERTS + kMaxWorld];
     __shared__ uint32_t scratch[kRouteWaves];
-    const uint32_t rank = blockIdx.x;
-    if (args.fold_mask >> rank & 1) fold_source(args, ws, rank, part_sum, scratch);
-    if (args.recv_mask >> rank & 1) {
-        __syncthreads();
-        layout_receiver(args, ws, rank, tot, scratch);
+    if (blockIdx.x < ws.world) {
+        const uint32_t rank = blockIdx.x;
+        if (args.fold_mask >> rank & 1) fold_source(args, ws, rank, part_sum, scratch);
+    } else {
+        const uint32_t rank = blockIdx.x - ws.world;
+        if (args.recv_mask >> rank & 1) layout_receiver(args, ws, rank, tot, scratch);
     }
 }
 
@@ -282,7 +287,7 @@ hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t tot
 }
 
 hipError_t launch_finalize(const FinalizeArgs &args, const Workspace &ws, hipStream_t stream) {
-    hipLaunchKernelGGL(route_finalize_kernel, dim3(ws.world), dim3(kRouteBlock), 0, stream, args, ws);
+    hipLaunchKernelGGL(route_finalize_kernel, dim3(2 * ws.world), dim3(kRouteBlock), 0, stream, args, ws);
     return hipGetLastError();
 }
 
