@@ -153,6 +153,8 @@ int check_send(a2a_ctx *ctx, uint32_t rank, uint64_t num_tokens, const void *x, 
                         "quantise mode needs in_elemsize 1, hidden_dim %% 128 == 0 and "
                         "hidden_dim_scale == hidden_dim / 128 (got %u, %u, %u)",
                         c.in_elemsize, c.hidden_dim, c.hidden_dim_scale);
+        if (c.hidden_dim_scale > 1024)
+            return fail(ctx, A2A_ERR_UNSUPPORTED, "quantise mode supports hidden_dim up to 131072");
         if (xs != nullptr)
             return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "quantise mode computes the scales: x_scale must be null");
     }

@@ -25,6 +25,12 @@ namespace a2a {
 template <bool QUANT>
 __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args,
                                                              const Workspace ws) {
+    // Scales of one token (one per 128 elements) and where each copy's go.
+    constexpr int kMaxLdsScales = 1024;
+    __shared__ float s_scale[QUANT ? kMaxLdsScales : 1];
+    __shared__ uint64_t s_scale_ptr[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint32_t s_scale_stride[A2A_MAX_EXPERTS_PER_TOKEN];
+
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
@@ -92,19 +98,21 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
                     *reinterpret_cast<u32x4 *>(row + (size_t)c * 16) = q;
                 }
             }
-            // Lane L writes the scale of group (L % 8) of this wavefront for
-            // route k0 + L / 8: eight routes per store instruction.
-            const uint32_t j = lane & 7;
-            const float group_scale = __shfl(scale, (int)(j * 8));
-            const uint32_t group = base / 8 + j;
-            for (uint32_t k0 = 0; k0 < K; k0 += 8) {
-                const uint32_t k = k0 + lane / 8;
-                const uint64_t sp = __shfl(scale_ptr, (int)(k & (kWave - 1)));
-                const uint32_t ss = __shfl(scale_stride, (int)(k & (kWave - 1)));
-                if (k < K && sp != 0 && group < Hs) {
-                    reinterpret_cast<float *>(sp)[(size_t)group * ss] = group_scale;
-                }
-            }
+            if (active && (lane & 7) == 0 && c / 8 < kMaxLdsScales) s_scale[c / 8] = scale;
+        }
+        // The token's scales meet in LDS so that each copy's scale row goes out
+        // as one contiguous run instead of one 32-byte piece per wavefront.
+        if (wave == 0 && lane < K) {
+            s_scale_ptr[lane] = scale_ptr;
+            s_scale_stride[lane] = scale_stride;
+        }
+        __syncthreads();
+        const uint32_t Hl = Hs < (uint32_t)kMaxLdsScales ? Hs : (uint32_t)kMaxLdsScales;
+        for (uint32_t i = tid; i < K * Hl; i += blockDim.x) {
+            const uint32_t k = i / Hl;
+            const uint32_t j = i - k * Hl;
+            const uint64_t sp = s_scale_ptr[k];
+            if (sp != 0) reinterpret_cast<float *>(sp)[(size_t)j * s_scale_stride[k]] = s_scale[j];
         }
     } else {
         const uint32_t num_chunks = args.row_bytes / 16;
