@@ -409,10 +409,18 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
     pa.hidden_dim = c.hidden_dim;
     pa.hidden_dim_scale = c.hidden_dim_scale;
 
-    hipError_t e = launch_route(ra, ctx->ws, blocks, s);
-    if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
-    e = launch_finalize(fa, ctx->ws, s);
-    if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+    bool small = true;  // every source fits one routing chunk: one launch does the whole pass
+    for (uint32_t r = 0; r < N; ++r) small = small && fa.num_blocks[r] <= 1;
+    hipError_t e;
+    if (small) {
+        e = launch_route_small(ra, fa, ctx->ws, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_small");
+    } else {
+        e = launch_route(ra, ctx->ws, blocks, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
+        e = launch_finalize(fa, ctx->ws, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+    }
     e = launch_dispatch_push(pa, ctx->ws, quantize != 0, tokens, s);
     if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_push");
 

@@ -135,6 +135,38 @@ __device__ void fold_source(const FinalizeArgs &args, const Workspace &ws, uint3
     if (owner) ws.expert_offsets[g * E + e0] = incl;
 }
 
+// Rows of receiver `r` from `tot[g * Le + le]`, the number of copies source g
+// sends to local expert le.  Whole workgroup.
+__device__ void layout_from_totals(const FinalizeArgs &args, const Workspace &ws, uint32_t r,
+                                   const uint32_t *tot, uint32_t *scratch) {
+    const uint32_t N = ws.world, E = ws.num_experts, Le = ws.experts_per_rank;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t pad = ws.expert_padding;
+    const uint32_t e = r * Le + tid;
+    const bool mine = tid < Le && e < E;
+    uint32_t tpe = 0;
+    if (mine) {
+        for (uint32_t g = 0; g < N; ++g) tpe += tot[g * Le + tid];
+    }
+    const uint32_t padded = (tpe + pad - 1) / pad * pad;
+    const uint32_t poff = block_inclusive_scan(mine ? padded : 0, scratch) - padded;
+    if (mine) {
+        ws.tokens_per_expert[e] = tpe;
+        ws.padded_offset[e] = poff;
+        if (args.out_num_tokens[r] != nullptr) args.out_num_tokens[r][tid] = (int32_t)tpe;
+        if (poff + tpe > args.out_rows[r]) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+        // Sources in the order the reference's host worker visits them
+        // (a2a_worker.rs:681-694); each gets a contiguous run of rows.
+        uint32_t running = poff;
+        for (uint32_t i = 0; i < N; ++i) {
+            const uint32_t g = source_order(r, i, N, ws.node_size);
+            ws.slot_base[g * E + e] = running;
+            running += tot[g * Le + tid];
+        }
+    }
+}
+
+
 // Receiver part of the finalize: rows of receiver `r`, from the chunk
 // histograms of the sources folded by this launch and the published counts of
 // the sources that sent earlier in the step.  Whole workgroup; `tot` holds
@@ -167,49 +199,19 @@ __device__ void layout_receiver(const FinalizeArgs &args, const Workspace &ws, u
         if (sum != 0) atomicAdd(&tot[item], sum);
     }
     __syncthreads();
-
-    const uint32_t pad = ws.expert_padding;
-    const uint32_t e = r * Le + tid;
-    const bool mine = tid < Le && e < E;
-    uint32_t tpe = 0;
-    if (mine) {
-        for (uint32_t g = 0; g < N; ++g) tpe += tot[g * Le + tid];
-    }
-    const uint32_t padded = (tpe + pad - 1) / pad * pad;
-    const uint32_t poff = block_inclusive_scan(mine ? padded : 0, scratch) - padded;
-    if (mine) {
-        ws.tokens_per_expert[e] = tpe;
-        ws.padded_offset[e] = poff;
-        if (args.out_num_tokens[r] != nullptr) args.out_num_tokens[r][tid] = (int32_t)tpe;
-        if (poff + tpe > args.out_rows[r]) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
-        // Sources in the order the reference's host worker visits them
-        // (a2a_worker.rs:681-694); each gets a contiguous run of rows.
-        uint32_t running = poff;
-        for (uint32_t i = 0; i < N; ++i) {
-            const uint32_t g = source_order(r, i, N, ws.node_size);
-            ws.slot_base[g * E + e] = running;
-            running += tot[g * Le + tid];
-        }
-    }
+    layout_from_totals(args, ws, r, tot, scratch);
 }
 
-}  // namespace
-
-__global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs args,
-                                                                 const Workspace ws) {
-    __shared__ uint16_t wave_hist[kRouteWaves][A2A_MAX_EXPERTS];
-
+// Ranks the entries of chunk `chunk` of source `g` inside their experts and
+// returns, to thread e < E, the number of entries of the chunk with expert e.
+// Whole workgroup (kRouteBlock threads).
+__device__ uint32_t rank_chunk(const RouteSrc &src, const Workspace &ws, uint32_t g, uint32_t chunk,
+                               uint16_t (*wave_hist)[A2A_MAX_EXPERTS]) {
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
     const uint32_t E = ws.num_experts;
     const uint32_t K = ws.topk;
-
-    // Which source and which chunk of it this workgroup handles (uniform).
-    uint32_t g = 0;
-    while (g + 1 < ws.world && blockIdx.x >= args.block_start[g + 1]) ++g;
-    const uint32_t chunk = blockIdx.x - args.block_start[g];
-    const RouteSrc src = args.src[g];
     const uint32_t num_entries = effective_tokens(src.bound_m, src.num_tokens) * K;
 
     if (tid < E) {
@@ -244,16 +246,14 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
     __syncthreads();
 
     // Exclusive scan of each expert's column over the 16 wavefronts.
-    uint32_t *block_hist = ws.block_hist + ((size_t)g * ws.nb_max + chunk) * E;
-    for (uint32_t e = tid; e < E; e += kRouteBlock) {
-        uint32_t run = 0;
+    uint32_t run = 0;
+    if (tid < E) {
 #pragma unroll
         for (int w = 0; w < kRouteWaves; ++w) {
-            const uint32_t c = wave_hist[w][e];
-            wave_hist[w][e] = (uint16_t)run;
+            const uint32_t c = wave_hist[w][tid];
+            wave_hist[w][tid] = (uint16_t)run;
             run += c;
         }
-        block_hist[e] = run;
     }
     __syncthreads();
 
@@ -261,6 +261,65 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
         ws.local_rank[(size_t)g * ws.max_tk + entry] =
             valid ? (uint16_t)(wave_hist[wave][expert] + rank_in_wave) : (uint16_t)0;
     }
+    return run;
+}
+
+}  // namespace
+
+__global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs args,
+                                                                 const Workspace ws) {
+    __shared__ uint16_t wave_hist[kRouteWaves][A2A_MAX_EXPERTS];
+    // Which source and which chunk of it this workgroup handles (uniform).
+    uint32_t g = 0;
+    while (g + 1 < ws.world && blockIdx.x >= args.block_start[g + 1]) ++g;
+    const uint32_t chunk = blockIdx.x - args.block_start[g];
+    const uint32_t count = rank_chunk(args.src[g], ws, g, chunk, wave_hist);
+    if (threadIdx.x < ws.num_experts) {
+        ws.block_hist[((size_t)g * ws.nb_max + chunk) * ws.num_experts + threadIdx.x] = count;
+    }
+}
+
+// The whole routing pass in one launch, for steps in which every source has at
+// most one chunk of entries (decode-sized batches): one workgroup per logical
+// rank.  Workgroup i ranks the entries of source i, and lays out receiver i by
+// counting, over the entries of EVERY source, the copies bound for its experts.
+// Nothing is exchanged between workgroups.
+__global__ __launch_bounds__(kRouteBlock) void route_small_kernel(const RouteArgs args,
+                                                                  const FinalizeArgs fin,
+                                                                  const Workspace ws) {
+    __shared__ uint16_t wave_hist[kRouteWaves][A2A_MAX_EXPERTS];
+    __shared__ uint32_t tot[A2A_MAX_EXPERTS + kMaxWorld];
+    __shared__ uint32_t scratch[kRouteWaves];
+    const uint32_t N = ws.world, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
+    const uint32_t rank = blockIdx.x;
+    const uint32_t tid = threadIdx.x;
+
+    // Receiver part first: its loads do not depend on anything.
+    for (uint32_t i = tid; i < N * Le; i += kRouteBlock) tot[i] = 0;
+    __syncthreads();
+    if (fin.recv_mask >> rank & 1) {
+        for (uint32_t g = 0; g < N; ++g) {
+            const RouteSrc &src = args.src[g];
+            const uint32_t entries = effective_tokens(src.bound_m, src.num_tokens) * K;
+            if (tid < entries) {
+                const uint32_t token = tid / K;
+                const uint32_t expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + (tid - token * K)];
+                if (expert < E && expert / Le == rank) atomicAdd(&tot[g * Le + expert - rank * Le], 1u);
+            }
+        }
+    }
+
+    // Source part.
+    const uint32_t count = rank_chunk(args.src[rank], ws, rank, 0, wave_hist);
+    if (tid < E) {
+        ws.num_routed[rank * E + tid] = count;
+        ws.block_prefix[(size_t)rank * ws.nb_max * E + tid] = 0;
+    }
+    const uint32_t incl = block_inclusive_scan(tid < E ? count : 0, scratch);
+    if (tid < E) ws.expert_offsets[rank * E + tid] = incl;
+
+    __syncthreads();
+    if (fin.recv_mask >> rank & 1) layout_from_totals(fin, ws, rank, tot, scratch);
 }
 
 // Two workgroups per logical rank, independent of each other: workgroup i folds
@@ -283,6 +342,12 @@ hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t tot
                         hipStream_t stream) {
     if (total_blocks == 0) return hipSuccess;
     hipLaunchKernelGGL(route_hist_kernel, dim3(total_blocks), dim3(kRouteBlock), 0, stream, args, ws);
+    return hipGetLastError();
+}
+
+hipError_t launch_route_small(const RouteArgs &args, const FinalizeArgs &fin, const Workspace &ws,
+                              hipStream_t stream) {
+    hipLaunchKernelGGL(route_small_kernel, dim3(ws.world), dim3(kRouteBlock), 0, stream, args, fin, ws);
     return hipGetLastError();
 }
 
