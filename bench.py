@@ -187,6 +187,11 @@ def main() -> int:
     ap.add_argument("--routings", type=int, default=4, help="distinct routings cycled over the steps")
     ap.add_argument("--cpu-reps", type=int, default=3, help="repetitions of the CPU baseline (0 = skip)")
     ap.add_argument("--no-decode", action="store_true", help="skip the 128-token shape")
+    ap.add_argument("--decode-only", action="store_true",
+                    help="time only the 128-token shape (for a kernel trace of the decode step alone)")
+    ap.add_argument("--probe-copy", action="store_true",
+                    help="also run plain device-to-device copies of 512 MiB: the known-size kernel that "
+                         "hardware byte counters are scaled by")
     ap.add_argument("--probe-copy", action="store_true",
                     help="also run plain device-to-device copies of 512 MiB (torch's copy kernel): the "
                          "known-size kernel that hardware byte counters are scaled by")
@@ -213,6 +218,23 @@ def main() -> int:
             dst.copy_(src)
         torch.cuda.synchronize(device)
         del src, dst
+
+    if args.probe_copy:
+        src = torch.empty(512 << 20, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize(device)
+        del src, dst
+
+    if args.decode_only:
+        wl2 = Workload(C2, device, args.routings)
+        _, d2, c2, b2 = time_workload(wl2, args.steps, args.warmup)
+        wl2.close()
+        print(json.dumps({"decode_128_only": {"dispatch_us_p50": round(Statistics.create(d2).p50, 2),
+                                              "combine_us_p50": round(Statistics.create(c2).p50, 2),
+                                              "total_us_p50": round(Statistics.create(b2).p50, 2)}}))
+        return 0
 
     case = C3
     wl = Workload(case, device, args.routings)

@@ -240,3 +240,67 @@ def test_operator_asserts_like_the_reference():
     finally:
         for op in ops:
             op.destroy()
+
+
+def test_calls_can_be_captured_in_a_hip_graph():
+    """The calls only enqueue kernels whose arguments travel by value (no allocation, copy or
+    synchronisation inside), so a dispatch + combine can be captured once and replayed
+    (docs/fabric-lib.md:15 lists graph capture as a feature of the reference).  Every replay,
+    with eager work in between, must reproduce the eager result."""
+    case = C1
+    world = make_world(case, "all")
+    rows = rows_needed(case, world)
+    N, Le, H, Hs = case.world_size, case.experts_per_rank, case.hidden_dim, case.hidden_dim_scale
+    _, ops = make_ops(case, DEV)
+    try:
+        t = []
+        gen = torch.Generator().manual_seed(3)
+        for r, rd in enumerate(world):
+            t.append(dict(x=rd.x.to(DEV), idx=rd.indices_u32.to(DEV), w=rd.weights.to(DEV),
+                          n=torch.zeros(Le, dtype=torch.int32, device=DEV),
+                          ox=torch.zeros((rows, H), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn),
+                          os=torch.zeros((rows, Hs), dtype=torch.float32, device=DEV),
+                          y=torch.randn((rows, H), generator=gen).to(torch.bfloat16).to(DEV),
+                          o=torch.zeros((rd.x.shape[0], H), dtype=torch.bfloat16, device=DEV)))
+
+        def step():
+            for r in range(N):
+                ops[r].dispatch(out_expert_num_tokens=t[r]["n"], out_expert_x=t[r]["ox"], out_expert_x_scale=t[r]["os"],
+                                dp_x=t[r]["x"], dp_x_scale=None, indices=t[r]["idx"], weights=t[r]["w"])
+            for r in range(N):
+                ops[r].combine(out_tokens=t[r]["o"], indices=t[r]["idx"], weights=t[r]["w"], expert_y=t[r]["y"])
+
+        def snapshot():
+            torch.cuda.synchronize(DEV)
+            return [(a["n"].clone(), a["ox"].view(torch.uint8).clone(), a["os"].clone(), a["o"].clone()) for a in t]
+
+        def clear():
+            for a in t:
+                a["n"].zero_(); a["ox"].view(torch.uint8).zero_(); a["os"].zero_(); a["o"].zero_()
+
+        step()
+        eager = snapshot()
+        assert ops[0].context.status() == 0
+        graph = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream(device=DEV)
+        side.wait_stream(torch.cuda.current_stream(DEV))
+        with torch.cuda.stream(side):
+            step()                                       # warm-up on the capture stream
+        torch.cuda.current_stream(DEV).wait_stream(side)
+        torch.cuda.synchronize(DEV)
+        with torch.cuda.graph(graph):
+            step()
+        for _ in range(3):
+            clear()
+            scratch = torch.randn(1 << 20, device=DEV).sum()       # eager work between replays
+            torch.cuda.synchronize(DEV)
+            graph.replay()
+            got = snapshot()
+            for (en, ex, es, eo), (gn, gx, gs, go) in zip(eager, got):
+                assert torch.equal(en, gn) and torch.equal(ex, gx) and torch.equal(es, gs)
+                assert torch.equal(eo.view(torch.int16), go.view(torch.int16))
+            del scratch
+        assert ops[0].context.status() == 0
+    finally:
+        for op in ops:
+            op.destroy()
