@@ -190,9 +190,6 @@ def main() -> int:
     ap.add_argument("--decode-only", action="store_true",
                     help="time only the 128-token shape (for a kernel trace of the decode step alone)")
     ap.add_argument("--probe-copy", action="store_true",
-                    help="also run plain device-to-device copies of 512 MiB: the known-size kernel that "
-                         "hardware byte counters are scaled by")
-    ap.add_argument("--probe-copy", action="store_true",
                     help="also run plain device-to-device copies of 512 MiB (torch's copy kernel): the "
                          "known-size kernel that hardware byte counters are scaled by")
     args = ap.parse_args()
@@ -210,14 +207,6 @@ def main() -> int:
         return 3
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-
-    if args.probe_copy:
-        src = torch.empty(512 << 20, dtype=torch.uint8, device=device).fill_(1)
-        dst = torch.empty_like(src)
-        for _ in range(5):
-            dst.copy_(src)
-        torch.cuda.synchronize(device)
-        del src, dst
 
     if args.probe_copy:
         src = torch.empty(512 << 20, dtype=torch.uint8, device=device).fill_(1)
