@@ -38,6 +38,11 @@ for _p in (REPO / "pplx-garden_amd", REPO / "oracle", REPO / "tests"):
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
+# HBM bytes per launch on the default workload, from hardware counters (FETCH_SIZE and WRITE_SIZE
+# passes, scaled by what the same counters read for a 512 MiB copy: x2.000 and x1.000).  The counter
+# runs and their commands are summarised in profiles/hbm_traffic_dsv3_prefill_4096_push_and_combine.md.
+MEASURED_TRAFFIC_BYTES = {"combine_gather_kernel": 531_696_000, "dispatch_push_kernel": 303_049_000}
+
 
 def algorithmic_bytes(T: int, H: int, K: int):
     """One-hop minimum per step: dispatch reads the bf16 row and the indices and
@@ -237,14 +242,18 @@ def main() -> int:
     value = (d_bytes + c_bytes) / (ms_per_step * 1e-3) / 1e9
     d_stats, c_stats, b_stats = Statistics.create(disp), Statistics.create(comb), Statistics.create(both)
 
-    def roof(bytes_, mean_us, kernel):
+    def roof(bytes_, mean_us, kernel, note):
         achieved = bytes_ / (mean_us * 1e-6) / 1e9
         return {"kernel": kernel, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
-                "bytes_per_launch": bytes_, "avg_us": round(mean_us, 2)}
+                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                "traffic": MEASURED_TRAFFIC_BYTES.get(kernel), "bytes_per_launch": bytes_,
+                "avg_us": round(mean_us, 2), "timing": note}
 
-    combine_roof = roof(c_bytes, c_stats.mean, "combine_gather_kernel")
-    dispatch_roof = roof(d_bytes, d_stats.mean, "dispatch_push_kernel (+ route_hist, route_finalize)")
+    combine_roof = roof(c_bytes, c_stats.mean, "combine_gather_kernel",
+                        "events around a2a_combine, which is this one launch")
+    dispatch_roof = roof(d_bytes, d_stats.mean, "dispatch_push_kernel",
+                         "events around a2a_dispatch: route_hist + route_finalize + this kernel, so the "
+                         "kernel alone is faster than avg_us")
     dominant, other = ((combine_roof, dispatch_roof) if c_stats.mean >= d_stats.mean
                        else (dispatch_roof, combine_roof))
 
