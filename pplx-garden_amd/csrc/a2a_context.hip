@@ -211,6 +211,17 @@ uint32_t rows_upper_bound(const a2a_ctx *ctx) {
     return (uint32_t)(rows < cap ? rows : cap);
 }
 
+// The one-launch routing pass recounts earlier chunks in every chunk workgroup
+// and all entries in every receiver workgroup; that is instruction-bound on one
+// compute unit (a 32-chunk source took 32 us against 10 us for the two-launch
+// pass), so it is used for decode-sized steps only.
+bool fused_routing_pays(const FinalizeArgs &fa, uint32_t world, uint32_t total_blocks) {
+    for (uint32_t r = 0; r < world; ++r) {
+        if (fa.num_blocks[r] > 4) return false;
+    }
+    return total_blocks <= 64;
+}
+
 uint32_t all_ranks(const a2a_ctx *ctx) {
     return ctx->cfg.world_size >= 32 ? 0xFFFFFFFFu : ((1u << ctx->cfg.world_size) - 1);
 }
@@ -409,12 +420,10 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
     pa.hidden_dim = c.hidden_dim;
     pa.hidden_dim_scale = c.hidden_dim_scale;
 
-    bool small = true;  // every source fits one routing chunk: one launch does the whole pass
-    for (uint32_t r = 0; r < N; ++r) small = small && fa.num_blocks[r] <= 1;
     hipError_t e;
-    if (small) {
-        e = launch_route_small(ra, fa, ctx->ws, s);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_small");
+    if (fused_routing_pays(fa, N, blocks)) {
+        e = launch_route_fused(ra, fa, ctx->ws, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
     } else {
         e = launch_route(ra, ctx->ws, blocks, s);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
@@ -580,10 +589,16 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     fa.fold_mask = 1u << rank;
     fa.valid_mask = ctx->sent_mask | (1u << rank);
     fa.recv_mask = 0;
-    hipError_t e = launch_route(ra, ctx->ws, nb, s);
-    if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
-    e = launch_finalize(fa, ctx->ws, s);
-    if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+    hipError_t e;
+    if (fused_routing_pays(fa, c.world_size, nb)) {
+        e = launch_route_fused(ra, fa, ctx->ws, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
+    } else {
+        e = launch_route(ra, ctx->ws, nb, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
+        e = launch_finalize(fa, ctx->ws, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+    }
 
     StageSendArgs sa;
     memset(&sa, 0, sizeof sa);

@@ -131,7 +131,7 @@ struct CombArgs {
 hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
                         hipStream_t stream);
 hipError_t launch_finalize(const FinalizeArgs &args, const Workspace &ws, hipStream_t stream);
-hipError_t launch_route_small(const RouteArgs &args, const FinalizeArgs &fin, const Workspace &ws,
+hipError_t launch_route_fused(const RouteArgs &args, const FinalizeArgs &fin, const Workspace &ws,
                               hipStream_t stream);
 hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool quantize,
                                 uint32_t total_tokens, hipStream_t stream);

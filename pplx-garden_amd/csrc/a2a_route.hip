@@ -279,47 +279,158 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
     }
 }
 
-// The whole routing pass in one launch, for steps in which every source has at
-// most one chunk of entries (decode-sized batches): one workgroup per logical
-// rank.  Workgroup i ranks the entries of source i, and lays out receiver i by
-// counting, over the entries of EVERY source, the copies bound for its experts.
-// Nothing is exchanged between workgroups.
-__global__ __launch_bounds__(kRouteBlock) void route_small_kernel(const RouteArgs args,
+// Tables of sources that were routed with no tokens: no chunk workgroup exists
+// for them, so somebody else clears them.
+__device__ void clear_empty_sources(const FinalizeArgs &fin, const Workspace &ws) {
+    const uint32_t E = ws.num_experts;
+    for (uint32_t g = 0; g < ws.world; ++g) {
+        if ((fin.fold_mask >> g & 1) && fin.num_blocks[g] == 0 && threadIdx.x < E) {
+            ws.num_routed[g * E + threadIdx.x] = 0;
+            ws.expert_offsets[g * E + threadIdx.x] = 0;
+        }
+    }
+}
+
+// Per-expert number of entries of source `g` in the chunks before `chunk`,
+// returned to thread e < E.  Every wavefront counts its share of those entries
+// into its own row of `wave_hist` (ballot matching, leader lanes add the match
+// count: no atomics, nothing to contend on), then the columns are summed.
+// Whole workgroup.
+__device__ uint32_t count_prior_chunks(const RouteSrc &src, const Workspace &ws, uint32_t chunk,
+                                       uint16_t (*wave_hist)[A2A_MAX_EXPERTS]) {
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const uint32_t E = ws.num_experts;
+    const uint32_t K = ws.topk;
+    if (chunk == 0) return 0;
+    const uint32_t num_entries = effective_tokens(src.bound_m, src.num_tokens) * K;
+    const uint32_t nbits = 32 - __clz((int)(E - 1) | 1);
+    if (tid < E) {
+#pragma unroll
+        for (int w = 0; w < kRouteWaves; ++w) wave_hist[w][tid] = 0;
+    }
+    __syncthreads();
+    for (uint32_t c0 = 0; c0 < chunk; c0 += 8) {
+        uint32_t expert[8];
+        bool valid[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {       // eight loads in flight per lane
+            const uint32_t entry = (c0 + j) * kRouteBlock + tid;
+            valid[j] = c0 + j < chunk && entry < num_entries;
+            expert[j] = 0;
+            if (valid[j]) {
+                const uint32_t token = entry / K;
+                expert[j] = (uint32_t)src.indices[(size_t)token * src.indices_stride + (entry - token * K)];
+                valid[j] = expert[j] < E;
+            }
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            if (c0 + j >= chunk) break;
+            uint64_t peers = __ballot(valid[j]);
+            for (uint32_t b = 0; b < nbits; ++b) {
+                const bool bit = (expert[j] >> b) & 1;
+                const uint64_t set = __ballot(valid[j] && bit);
+                peers &= bit ? set : ~set;
+            }
+            if (valid[j] && (peers & ((1ull << lane) - 1)) == 0) {
+                wave_hist[wave][expert[j]] += (uint16_t)__popcll(peers);
+            }
+        }
+    }
+    __syncthreads();
+    uint32_t sum = 0;
+    if (tid < E) {
+#pragma unroll
+        for (int w = 0; w < kRouteWaves; ++w) sum += wave_hist[w][tid];
+    }
+    __syncthreads();
+    return sum;
+}
+
+// The whole routing pass in ONE launch, for steps of moderate size.  The grid
+// holds one workgroup per chunk of every source, then one per receiver; none
+// depends on another:
+//  - a chunk workgroup counts the entries of the chunks before its own (that is
+//    its prefix), ranks its own entries, and, if it is the last chunk of its
+//    source, publishes the source's totals and their scan over experts;
+//  - a receiver workgroup counts, over the entries of EVERY source, the copies
+//    bound for its experts and lays out its rows.
+// The redundant counting is quadratic in the number of chunks of a source, so
+// long inputs take the two-launch path (route_hist + route_finalize) instead.
+__global__ __launch_bounds__(kRouteBlock) void route_fused_kernel(const RouteArgs args,
                                                                   const FinalizeArgs fin,
                                                                   const Workspace ws) {
     __shared__ uint16_t wave_hist[kRouteWaves][A2A_MAX_EXPERTS];
     __shared__ uint32_t tot[A2A_MAX_EXPERTS + kMaxWorld];
     __shared__ uint32_t scratch[kRouteWaves];
     const uint32_t N = ws.world, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
-    const uint32_t rank = blockIdx.x;
     const uint32_t tid = threadIdx.x;
+    const uint32_t chunk_blocks = args.block_start[N];
 
-    // Receiver part first: its loads do not depend on anything.
-    for (uint32_t i = tid; i < N * Le; i += kRouteBlock) tot[i] = 0;
-    __syncthreads();
-    if (fin.recv_mask >> rank & 1) {
+    if (blockIdx.x == 0) clear_empty_sources(fin, ws);
+    if (blockIdx.x >= chunk_blocks) {
+        // receiver workgroup
+        const uint32_t rank = blockIdx.x - chunk_blocks;
+        if (!(fin.recv_mask >> rank & 1)) return;
+        for (uint32_t i = tid; i < N * Le; i += kRouteBlock) tot[i] = 0;
+        __syncthreads();
         for (uint32_t g = 0; g < N; ++g) {
+            if (!(fin.valid_mask >> g & 1)) continue;
+            if (!(fin.fold_mask >> g & 1)) {
+                // a source that sent earlier in this step: its counts are published
+                if (tid < Le && rank * Le + tid < E) tot[g * Le + tid] = ws.num_routed[g * E + rank * Le + tid];
+                continue;
+            }
             const RouteSrc &src = args.src[g];
             const uint32_t entries = effective_tokens(src.bound_m, src.num_tokens) * K;
-            if (tid < entries) {
-                const uint32_t token = tid / K;
-                const uint32_t expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + (tid - token * K)];
-                if (expert < E && expert / Le == rank) atomicAdd(&tot[g * Le + expert - rank * Le], 1u);
+            for (uint32_t e0 = 0; e0 < entries; e0 += 8 * kRouteBlock) {
+                uint32_t expert[8];
+#pragma unroll
+                for (uint32_t j = 0; j < 8; ++j) {
+                    const uint32_t entry = e0 + j * kRouteBlock + tid;
+                    expert[j] = 0xFFFFFFFFu;
+                    if (entry < entries) {
+                        const uint32_t token = entry / K;
+                        expert[j] = (uint32_t)src.indices[(size_t)token * src.indices_stride + (entry - token * K)];
+                    }
+                }
+#pragma unroll
+                for (uint32_t j = 0; j < 8; ++j) {
+                    if (expert[j] < E && expert[j] / Le == rank) atomicAdd(&tot[g * Le + expert[j] - rank * Le], 1u);
+                }
             }
         }
+        __syncthreads();
+        layout_from_totals(fin, ws, rank, tot, scratch);
+        return;
     }
 
-    // Source part.
-    const uint32_t count = rank_chunk(args.src[rank], ws, rank, 0, wave_hist);
+    // chunk workgroup
+    uint32_t g = 0;
+    while (g + 1 < N && blockIdx.x >= args.block_start[g + 1]) ++g;
+    const uint32_t chunk = blockIdx.x - args.block_start[g];
+    const RouteSrc &src = args.src[g];
+    const uint32_t prior = count_prior_chunks(src, ws, chunk, wave_hist);
+    const uint32_t own = rank_chunk(src, ws, g, chunk, wave_hist);
     if (tid < E) {
-        ws.num_routed[rank * E + tid] = count;
-        ws.block_prefix[(size_t)rank * ws.nb_max * E + tid] = 0;
+        ws.block_hist[((size_t)g * ws.nb_max + chunk) * E + tid] = own;
+        ws.block_prefix[((size_t)g * ws.nb_max + chunk) * E + tid] = prior;
     }
-    const uint32_t incl = block_inclusive_scan(tid < E ? count : 0, scratch);
-    if (tid < E) ws.expert_offsets[rank * E + tid] = incl;
+    if (chunk + 1 == fin.num_blocks[g]) {
+        const uint32_t total = prior + own;
+        if (tid < E) ws.num_routed[g * E + tid] = total;
+        const uint32_t incl = block_inclusive_scan(tid < E ? total : 0, scratch);
+        if (tid < E) ws.expert_offsets[g * E + tid] = incl;
+    }
+}
 
-    __syncthreads();
-    if (fin.recv_mask >> rank & 1) layout_from_totals(fin, ws, rank, tot, scratch);
+// A step in which no source has tokens and nobody receives: only the tables of
+// the routed sources have to be cleared.  One workgroup.
+__global__ __launch_bounds__(kRouteBlock) void route_clear_empty_kernel(const FinalizeArgs fin,
+                                                                        const Workspace ws) {
+    clear_empty_sources(fin, ws);
 }
 
 // Two workgroups per logical rank, independent of each other: workgroup i folds
@@ -345,9 +456,14 @@ hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t tot
     return hipGetLastError();
 }
 
-hipError_t launch_route_small(const RouteArgs &args, const FinalizeArgs &fin, const Workspace &ws,
+hipError_t launch_route_fused(const RouteArgs &args, const FinalizeArgs &fin, const Workspace &ws,
                               hipStream_t stream) {
-    hipLaunchKernelGGL(route_small_kernel, dim3(ws.world), dim3(kRouteBlock), 0, stream, args, fin, ws);
+    const uint32_t blocks = args.block_start[ws.world] + (fin.recv_mask != 0 ? ws.world : 0);
+    if (blocks != 0) {
+        hipLaunchKernelGGL(route_fused_kernel, dim3(blocks), dim3(kRouteBlock), 0, stream, args, fin, ws);
+    } else {
+        hipLaunchKernelGGL(route_clear_empty_kernel, dim3(1), dim3(kRouteBlock), 0, stream, fin, ws);
+    }
     return hipGetLastError();
 }
 
