@@ -212,14 +212,17 @@ uint32_t rows_upper_bound(const a2a_ctx *ctx) {
 }
 
 // The one-launch routing pass recounts earlier chunks in every chunk workgroup
-// and all entries in every receiver workgroup; that is instruction-bound on one
-// compute unit (a 32-chunk source took 32 us against 10 us for the two-launch
-// pass), so it is used for decode-sized steps only.
+// and all entries in every receiver workgroup: quadratic in the chunks of a
+// source.  Measured at 8 entries per token: 2 us faster than the two-launch
+// pass up to 8 chunks per source, equal at 16, 4 us slower at 32.
+#ifndef A2A_FUSED_MAX_CHUNKS
+#define A2A_FUSED_MAX_CHUNKS 12
+#endif
 bool fused_routing_pays(const FinalizeArgs &fa, uint32_t world, uint32_t total_blocks) {
     for (uint32_t r = 0; r < world; ++r) {
-        if (fa.num_blocks[r] > 4) return false;
+        if (fa.num_blocks[r] > A2A_FUSED_MAX_CHUNKS) return false;
     }
-    return total_blocks <= 64;
+    return total_blocks <= 4 * A2A_FUSED_MAX_CHUNKS;
 }
 
 uint32_t all_ranks(const a2a_ctx *ctx) {

@@ -292,59 +292,37 @@ __device__ void clear_empty_sources(const FinalizeArgs &fin, const Workspace &ws
 }
 
 // Per-expert number of entries of source `g` in the chunks before `chunk`,
-// returned to thread e < E.  Every wavefront counts its share of those entries
-// into its own row of `wave_hist` (ballot matching, leader lanes add the match
-// count: no atomics, nothing to contend on), then the columns are summed.
-// Whole workgroup.
+// returned to thread e < E.  Counts do not depend on the order of arrival, so
+// plain LDS atomics do (eight loads in flight per lane, one atomic per entry).
+// `counts` holds E words.  Whole workgroup.
 __device__ uint32_t count_prior_chunks(const RouteSrc &src, const Workspace &ws, uint32_t chunk,
-                                       uint16_t (*wave_hist)[A2A_MAX_EXPERTS]) {
+                                       uint32_t *counts) {
     const uint32_t tid = threadIdx.x;
-    const uint32_t lane = tid & (kWave - 1);
-    const uint32_t wave = tid / kWave;
     const uint32_t E = ws.num_experts;
     const uint32_t K = ws.topk;
     if (chunk == 0) return 0;
-    const uint32_t num_entries = effective_tokens(src.bound_m, src.num_tokens) * K;
-    const uint32_t nbits = 32 - __clz((int)(E - 1) | 1);
-    if (tid < E) {
-#pragma unroll
-        for (int w = 0; w < kRouteWaves; ++w) wave_hist[w][tid] = 0;
-    }
+    uint32_t num_entries = effective_tokens(src.bound_m, src.num_tokens) * K;
+    if (num_entries > chunk * kRouteBlock) num_entries = chunk * kRouteBlock;
+    if (tid < E) counts[tid] = 0;
     __syncthreads();
-    for (uint32_t c0 = 0; c0 < chunk; c0 += 8) {
+    for (uint32_t e0 = 0; e0 < num_entries; e0 += 8 * kRouteBlock) {
         uint32_t expert[8];
-        bool valid[8];
 #pragma unroll
-        for (uint32_t j = 0; j < 8; ++j) {       // eight loads in flight per lane
-            const uint32_t entry = (c0 + j) * kRouteBlock + tid;
-            valid[j] = c0 + j < chunk && entry < num_entries;
-            expert[j] = 0;
-            if (valid[j]) {
+        for (uint32_t j = 0; j < 8; ++j) {
+            const uint32_t entry = e0 + j * kRouteBlock + tid;
+            expert[j] = 0xFFFFFFFFu;
+            if (entry < num_entries) {
                 const uint32_t token = entry / K;
                 expert[j] = (uint32_t)src.indices[(size_t)token * src.indices_stride + (entry - token * K)];
-                valid[j] = expert[j] < E;
             }
         }
 #pragma unroll
         for (uint32_t j = 0; j < 8; ++j) {
-            if (c0 + j >= chunk) break;
-            uint64_t peers = __ballot(valid[j]);
-            for (uint32_t b = 0; b < nbits; ++b) {
-                const bool bit = (expert[j] >> b) & 1;
-                const uint64_t set = __ballot(valid[j] && bit);
-                peers &= bit ? set : ~set;
-            }
-            if (valid[j] && (peers & ((1ull << lane) - 1)) == 0) {
-                wave_hist[wave][expert[j]] += (uint16_t)__popcll(peers);
-            }
+            if (expert[j] < E) atomicAdd(&counts[expert[j]], 1u);
         }
     }
     __syncthreads();
-    uint32_t sum = 0;
-    if (tid < E) {
-#pragma unroll
-        for (int w = 0; w < kRouteWaves; ++w) sum += wave_hist[w][tid];
-    }
+    const uint32_t sum = tid < E ? counts[tid] : 0;
     __syncthreads();
     return sum;
 }
@@ -412,7 +390,7 @@ __global__ __launch_bounds__(kRouteBlock) void route_fused_kernel(const RouteArg
     while (g + 1 < N && blockIdx.x >= args.block_start[g + 1]) ++g;
     const uint32_t chunk = blockIdx.x - args.block_start[g];
     const RouteSrc &src = args.src[g];
-    const uint32_t prior = count_prior_chunks(src, ws, chunk, wave_hist);
+    const uint32_t prior = count_prior_chunks(src, ws, chunk, tot);
     const uint32_t own = rank_chunk(src, ws, g, chunk, wave_hist);
     if (tid < E) {
         ws.block_hist[((size_t)g * ws.nb_max + chunk) * E + tid] = own;
