@@ -81,7 +81,7 @@ typedef struct a2a_config {
     uint32_t num_experts;            /* E <= A2A_MAX_EXPERTS */
     uint32_t expert_padding;         /* each expert's slot range is rounded up to this */
     uint32_t num_experts_per_token;  /* K <= A2A_MAX_EXPERTS_PER_TOKEN */
-    uint32_t dp_size;                /* must be 1 */
+    uint32_t dp_size;                /* ranks per group that hold the same tokens; divides node_size */
     uint32_t node_size;              /* ranks per node; fixes the order of sources in a receiver */
     uint32_t world_size;             /* N <= A2A_MAX_WORLD_SIZE, divisible by node_size */
     int32_t  device;                 /* HIP device ordinal */
@@ -215,7 +215,9 @@ typedef struct a2a_combine_args {
  * (python/pplx_garden/kernels/p2p_all_to_all.py:317-440 with do_send and
  * do_recv).  Same results as the split calls; every token row is read once
  * and every copy is written once, straight into the receiver's out_x.
- * A rank that sends nothing passes num_tokens 0.
+ * A rank that sends nothing passes num_tokens 0.  With dp_size > 1 the ranks of
+ * a group pass the same tokens and routing (a2a_dispatch_send.cu:304,508): the
+ * send half of the group's first rank is the one that is read.
  */
 int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
                  void *stream);

@@ -571,6 +571,59 @@ def dispatch_world(inputs: Sequence[RankInput], *, num_experts: int,
     return outs
 
 
+def world_by_rows(indices_per_group: Sequence[np.ndarray], payload_per_group: Sequence[np.ndarray],
+                  scales_per_group: Sequence[Optional[np.ndarray]], *, num_experts: int,
+                  world_size: int, node_size: int, dp_size: int, expert_padding: int, out_rows: int):
+    """dispatch() of the whole group, written as the reference's receive loop.
+
+    For every receiver, `process_routing_info` lists the received rows with
+    their source rank, their position in the source's expert-sorted order and
+    their destination row; the row behind a position is found by sorting the
+    source's entries by (expert, token, k).  Handles dp groups (ranks of a group
+    hold the same tokens: a2a_dispatch_send.cu:304,508, a2a_worker.rs:633).
+    Returns (outs, slots): one RankOutput per RANK and, per GROUP, the pair
+    (receiver, row) of every copy as two [T,K] arrays.
+    """
+    G = world_size // dp_size
+    Le = ceil_div(num_experts, world_size)
+    num_routed = np.zeros((G, num_experts), dtype=np.uint32)
+    entry_at = []                          # per group: entry index behind each position
+    for g in range(G):
+        idx = np.asarray(indices_per_group[g]).astype(np.int64)
+        count, _, _ = route(idx, num_experts)
+        num_routed[g] = count
+        entry_at.append(np.argsort(idx.reshape(-1), kind="stable"))
+    row_bytes = payload_per_group[0].shape[1]
+    Hs = scales_per_group[0].shape[1] if scales_per_group[0] is not None else 0
+    outs, slot_rank, slot_row = [], [], []
+    for g in range(G):
+        shape = np.asarray(indices_per_group[g]).shape
+        slot_rank.append(np.full(shape, -1, dtype=np.int64))
+        slot_row.append(np.full(shape, -1, dtype=np.int64))
+    for r in range(world_size):
+        lay = process_routing_info(num_routed, r, world_size, node_size, dp_size, expert_padding, 0)
+        tpe = np.zeros(Le, dtype=np.int32)
+        tpe[: len(lay.tokens_per_expert)] = lay.tokens_per_expert
+        out = RankOutput(num_tokens=tpe, x=np.zeros((out_rows, row_bytes), dtype=np.uint8),
+                         x_scale=np.zeros((out_rows, Hs), dtype=np.float32) if Hs else None,
+                         written=np.zeros(out_rows, dtype=bool))
+        for i in range(lay.num_recv_tokens):
+            g = int(lay.source_rank[i]) // dp_size
+            entry = int(entry_at[g][int(lay.source_position[i])])
+            K = np.asarray(indices_per_group[g]).shape[1]
+            token, k = divmod(entry, K)
+            row = int(lay.padded_index[i])
+            assert not out.written[row]
+            out.x[row] = payload_per_group[g][token]
+            if Hs:
+                out.x_scale[row] = scales_per_group[g][token]
+            out.written[row] = True
+            slot_rank[g][token, k] = r
+            slot_row[g][token, k] = row
+        outs.append(out)
+    return outs, (slot_rank, slot_row)
+
+
 def _load_rows(y: np.ndarray, dtype: str) -> np.ndarray:
     if dtype == "bf16":
         return bf16_to_f32(y)

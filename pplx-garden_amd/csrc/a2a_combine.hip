@@ -174,6 +174,7 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
     while (g + 1 < ws.world && token_global >= args.token_start[g + 1]) ++g;
     const uint32_t token = token_global - args.token_start[g];
     const CombDst &dst = args.dst[g];
+    const uint32_t group = g / ws.dp_size;   // the routing tables belong to the rank's dp group
     if (token >= effective_tokens(dst.bound_m, dst.num_tokens)) return;
 
     // Lane r holds the descriptor of receiver r; lanes 0..K-1 resolve a route
@@ -191,8 +192,8 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
         expert = (uint32_t)dst.indices[(size_t)token * dst.indices_stride + lane];
         weight = dst.weights[(size_t)token * dst.weights_stride + lane];
         slot = args.staged_base != nullptr
-                   ? ws.token_offset[(size_t)g * ws.max_tk + token * K + lane]
-                   : ws.route_slot[(size_t)g * ws.max_tk + token * K + lane];
+                   ? ws.token_offset[(size_t)group * ws.max_tk + token * K + lane]
+                   : ws.route_slot[(size_t)group * ws.max_tk + token * K + lane];
     }
     const bool expert_ok = expert < E;
     const uint32_t r = expert_ok ? expert / ws.experts_per_rank : 0;
@@ -205,11 +206,11 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
         if (args.staged_base != nullptr) {
             // a2a_combine_recv.cu:67-73: position = exclusive offset of the expert + token offset.
             if (expert_ok) {
-                const uint32_t excl = expert > 0 ? ws.expert_offsets[g * E + expert - 1] : 0;
+                const uint32_t excl = expert > 0 ? ws.expert_offsets[group * E + expert - 1] : 0;
                 const uint32_t pos = excl + slot;
                 if (pos < ws.max_tk) {
                     row_ptr = (uint64_t)(args.staged_base +
-                                         ((size_t)g * ws.max_tk + pos) * args.staged_stride);
+                                         ((size_t)group * ws.max_tk + pos) * args.staged_stride);
                     ok = true;
                 }
             }

@@ -88,11 +88,12 @@ int check_config(const a2a_config &c) {
     if (c.world_size == 0 || c.world_size > A2A_MAX_WORLD_SIZE)
         return fail(nullptr, A2A_ERR_UNSUPPORTED, "world_size %u not in [1, %d]", c.world_size,
                     A2A_MAX_WORLD_SIZE);
-    if (c.dp_size != 1)
-        return fail(nullptr, A2A_ERR_UNSUPPORTED, "dp_size %u: only 1 is supported", c.dp_size);
     if (c.node_size == 0 || c.world_size % c.node_size != 0)
         return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "node_size %u does not divide world_size %u",
                     c.node_size, c.world_size);
+    if (c.dp_size == 0 || c.node_size % c.dp_size != 0)
+        return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "dp_size %u does not divide node_size %u", c.dp_size,
+                    c.node_size);
     if (c.num_experts == 0 || c.num_experts > A2A_MAX_EXPERTS)
         return fail(nullptr, A2A_ERR_UNSUPPORTED, "num_experts %u not in [1, %d]", c.num_experts,
                     A2A_MAX_EXPERTS);
@@ -273,6 +274,8 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
     ws.max_tk = config->max_num_tokens * K;
     ws.nb_max = ceil_div_u32(ws.max_tk, kRouteBlock);
     ws.world = N;
+    ws.num_groups = N / config->dp_size;
+    ws.dp_size = config->dp_size;
     ws.num_experts = E;
     ws.topk = K;
     ws.experts_per_rank = ceil_div_u32(E, N);
@@ -381,18 +384,23 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
     memset(&ra, 0, sizeof ra);
     memset(&fa, 0, sizeof fa);
     memset(&pa, 0, sizeof pa);
+    const uint32_t D = c.dp_size, G = N / D;
     uint32_t blocks = 0, tokens = 0;
-    for (uint32_t r = 0; r < N; ++r) {
-        const a2a_dispatch_args &a = args[r];
+    // Sources: one per dp group (its members hold the same tokens; the first member's are read).
+    for (uint32_t g = 0; g < G; ++g) {
+        const a2a_dispatch_args &a = args[g * D];
+        for (uint32_t m = 1; m < D; ++m) {
+            if (args[g * D + m].num_tokens != a.num_tokens)
+                return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "ranks %u and %u share a dp group but pass %llu and %llu tokens",
+                            g * D, g * D + m, (unsigned long long)a.num_tokens,
+                            (unsigned long long)args[g * D + m].num_tokens);
+        }
         const uint32_t T = (uint32_t)a.num_tokens;
-        ra.src[r] = RouteSrc{a.indices, a.bound_m, (uint32_t)a.indices_stride, T};
-        ra.block_start[r] = blocks;
-        fa.num_blocks[r] = ceil_div_u32((uint64_t)T * K, kRouteBlock);
-        blocks += fa.num_blocks[r];
-        fa.out_num_tokens[r] = a.out_num_tokens;
-        fa.out_rows[r] = a.out_x != nullptr ? (uint32_t)(a.out_x_rows > 0xFFFFFFFFull ? 0xFFFFFFFFull : a.out_x_rows)
-                                            : 0xFFFFFFFFu;
-        PushSrc &ps = pa.src[r];
+        ra.src[g] = RouteSrc{a.indices, a.bound_m, (uint32_t)a.indices_stride, T};
+        ra.block_start[g] = blocks;
+        fa.num_blocks[g] = ceil_div_u32((uint64_t)T * K, kRouteBlock);
+        blocks += fa.num_blocks[g];
+        PushSrc &ps = pa.src[g];
         ps.x = static_cast<const uint8_t *>(a.x_ptr);
         ps.x_scale = a.x_scale_ptr;
         ps.indices = a.indices;
@@ -402,6 +410,20 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
         ps.xs_stride_token = (uint32_t)a.x_scale_stride_token;
         ps.indices_stride = (uint32_t)a.indices_stride;
         ps.num_tokens = T;
+        pa.token_start[g] = tokens;
+        tokens += T;
+        ctx->num_tokens[g] = T;
+    }
+    for (uint32_t g = G; g <= (uint32_t)kMaxWorld; ++g) {
+        ra.block_start[g] = blocks;
+        pa.token_start[g] = tokens;
+    }
+    // Receivers: every rank.
+    for (uint32_t r = 0; r < N; ++r) {
+        const a2a_dispatch_args &a = args[r];
+        fa.out_num_tokens[r] = a.out_num_tokens;
+        fa.out_rows[r] = a.out_x != nullptr ? (uint32_t)(a.out_x_rows > 0xFFFFFFFFull ? 0xFFFFFFFFull : a.out_x_rows)
+                                            : 0xFFFFFFFFu;
         PushDst &pd = pa.dst[r];
         pd.out_x = static_cast<uint8_t *>(a.out_x);
         pd.out_scale = a.out_x_scale;
@@ -409,22 +431,15 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
         pd.os_stride_elem = (uint32_t)a.out_x_scale_stride_elem;
         pd.os_stride_token = (uint32_t)a.out_x_scale_stride_token;
         pd.out_rows = fa.out_rows[r];
-        pa.token_start[r] = tokens;
-        tokens += T;
-        ctx->num_tokens[r] = T;
     }
-    for (uint32_t r = N; r <= (uint32_t)kMaxWorld; ++r) {
-        ra.block_start[r] = blocks;
-        pa.token_start[r] = tokens;
-    }
-    fa.fold_mask = fa.valid_mask = fa.recv_mask = all_ranks(ctx);
-
+    fa.fold_mask = fa.valid_mask = G >= 32 ? 0xFFFFFFFFu : ((1u << G) - 1);
+    fa.recv_mask = all_ranks(ctx);
     pa.row_bytes = (uint32_t)row_bytes_of(c);
     pa.hidden_dim = c.hidden_dim;
     pa.hidden_dim_scale = c.hidden_dim_scale;
 
     hipError_t e;
-    if (fused_routing_pays(fa, N, blocks)) {
+    if (fused_routing_pays(fa, G, blocks)) {
         e = launch_route_fused(ra, fa, ctx->ws, s);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
     } else {
@@ -458,6 +473,8 @@ int a2a_combine(a2a_ctx *ctx, const a2a_combine_args *args, uint32_t expert_y_dt
     const uint32_t vec = 16 / in_size;
     if (c.hidden_dim % vec != 0)
         return fail(ctx, A2A_ERR_UNSUPPORTED, "hidden_dim %u is not a multiple of %u", c.hidden_dim, vec);
+    if (accumulate && c.dp_size != 1)   // python/pplx_garden/kernels/p2p_all_to_all.py:457-458
+        return fail(ctx, A2A_ERR_UNSUPPORTED, "accumulate needs dp_size 1");
     CombArgs ca;
     memset(&ca, 0, sizeof ca);
     uint32_t tokens = 0;
@@ -508,6 +525,8 @@ int a2a_ctx_read_table(a2a_ctx *ctx, uint32_t rank, uint32_t which, uint32_t *ou
     const uint32_t E = ws.num_experts;
     const uint32_t *src = nullptr;
     size_t limit = 0;
+    const uint32_t receiver = rank;
+    rank = rank / ws.dp_size;   // sender-side tables belong to the rank's dp group
     switch (which) {
         case A2A_TABLE_NUM_ROUTED:
             src = ws.num_routed + (size_t)rank * E;
@@ -531,7 +550,7 @@ int a2a_ctx_read_table(a2a_ctx *ctx, uint32_t rank, uint32_t which, uint32_t *ou
         case A2A_TABLE_SOURCE_RANK:
         case A2A_TABLE_SOURCE_POSITION:
         case A2A_TABLE_NUM_RECV_TOKENS:
-            src = staging_table(ctx->staging, ctx->cfg, rank, which, &limit);
+            src = staging_table(ctx->staging, ctx->cfg, receiver, which, &limit);
             if (src == nullptr)
                 return fail(ctx, A2A_ERR_BAD_ORDER, "receive tables exist only after a2a_dispatch_recv");
             break;
@@ -586,14 +605,17 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     memset(&ra, 0, sizeof ra);
     memset(&fa, 0, sizeof fa);
     const uint32_t nb = ceil_div_u32((uint64_t)T * K, kRouteBlock);
-    ra.src[rank] = RouteSrc{indices, bound_m, (uint32_t)indices_stride, T};
-    for (uint32_t r = 0; r <= (uint32_t)kMaxWorld; ++r) ra.block_start[r] = r <= rank ? 0 : nb;
-    fa.num_blocks[rank] = nb;
-    fa.fold_mask = 1u << rank;
-    fa.valid_mask = ctx->sent_mask | (1u << rank);
+    // The sender is the rank's dp group; when several members of a group send, each repeats
+    // the same routing and stages the same rows.
+    const uint32_t group = rank / c.dp_size;
+    ra.src[group] = RouteSrc{indices, bound_m, (uint32_t)indices_stride, T};
+    for (uint32_t r = 0; r <= (uint32_t)kMaxWorld; ++r) ra.block_start[r] = r <= group ? 0 : nb;
+    fa.num_blocks[group] = nb;
+    fa.fold_mask = 1u << group;
+    fa.valid_mask = ctx->sent_mask | (1u << group);
     fa.recv_mask = 0;
     hipError_t e;
-    if (fused_routing_pays(fa, c.world_size, nb)) {
+    if (fused_routing_pays(fa, c.world_size / c.dp_size, nb)) {
         e = launch_route_fused(ra, fa, ctx->ws, s);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
     } else {
@@ -621,8 +643,8 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     e = launch_stage_send(sa, ctx->ws, ctx->staging, quantize != 0, s);
     if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send");
 
-    ctx->sent_mask |= 1u << rank;
-    ctx->num_tokens[rank] = T;
+    ctx->sent_mask |= 1u << group;
+    ctx->num_tokens[group] = T;
     ctx->quantized = quantize;
     ctx->group_routing = false;
     return A2A_OK;
@@ -709,6 +731,8 @@ int a2a_combine_recv(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, size_t num_
         return fail(ctx, A2A_ERR_BAD_ORDER, "a2a_combine_recv before any a2a_combine_send of the step");
     if (num_tokens > c.max_num_tokens)
         return fail(ctx, A2A_ERR_TOO_MANY_TOKENS, "Number of tokens exceeds maximum allowed (rank %u)", rank);
+    if (accumulate && c.dp_size != 1)   // python/pplx_garden/kernels/p2p_all_to_all.py:457-458
+        return fail(ctx, A2A_ERR_UNSUPPORTED, "accumulate needs dp_size 1");
     if (elem_size_of(expert_y_dtype) != c.out_elemsize)
         return fail(ctx, A2A_ERR_UNSUPPORTED,
                     "expert_y dtype %u does not have the %u-byte elements the staging rows were sized for",

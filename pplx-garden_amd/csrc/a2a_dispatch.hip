@@ -38,7 +38,7 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
     const uint32_t K = ws.topk;
 
     uint32_t g = 0;
-    while (g + 1 < ws.world && blockIdx.x >= args.token_start[g + 1]) ++g;
+    while (g + 1 < ws.num_groups && blockIdx.x >= args.token_start[g + 1]) ++g;
     const uint32_t token = blockIdx.x - args.token_start[g];
     const PushSrc &src = args.src[g];
     if (token >= effective_tokens(src.bound_m, src.num_tokens)) return;

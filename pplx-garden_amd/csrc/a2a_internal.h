@@ -33,7 +33,9 @@ struct Workspace {
     uint32_t *err;             // [1]            A2A_DEV_* bits, sticky
     uint32_t max_tk;           // max_num_tokens * K
     uint32_t nb_max;           // ceil(max_tk / kRouteBlock)
-    uint32_t world;            // N
+    uint32_t world;            // N logical ranks (receivers)
+    uint32_t num_groups;       // G = N / dp_size: groups of ranks that hold the same tokens (sources)
+    uint32_t dp_size;          // ranks per group
     uint32_t num_experts;      // E
     uint32_t topk;             // K
     uint32_t experts_per_rank; // Le = ceil(E / N)
@@ -101,7 +103,7 @@ struct CombSrc {  // one per receiver rank: the expert outputs it holds
     uint32_t pad_;
 };
 
-struct CombDst {  // one per source rank: where its combined tokens go
+struct CombDst {  // one per rank: where its combined tokens go
     uint8_t *out;
     const int32_t *indices;
     const float *weights;
@@ -147,21 +149,23 @@ __device__ __forceinline__ uint32_t effective_tokens(const int32_t *bound_m, uin
     return (uint32_t)b < num_tokens ? (uint32_t)b : num_tokens;
 }
 
-// i-th source that receiver `rank` lays out (a2a_worker.rs:681-694, dp_size 1):
-// ranks of the other nodes starting at the next node, then the rest of the own
-// node starting after `rank`, then `rank`.
+// i-th source (dp group) that receiver `rank` lays out (a2a_worker.rs:681-694):
+// the groups of the other nodes starting at the next node, then the other
+// groups of the own node starting after the own group, then the own group.
 __host__ __device__ __forceinline__ uint32_t source_order(uint32_t rank, uint32_t i, uint32_t world,
-                                                          uint32_t node_size) {
+                                                          uint32_t node_size, uint32_t dp_size) {
     const uint32_t num_nodes = world / node_size;
+    const uint32_t groups_per_node = node_size / dp_size;
     const uint32_t rank_node = rank / node_size;
-    const uint32_t remote = (num_nodes - 1) * node_size;
+    const uint32_t dp_group = rank / dp_size;
+    const uint32_t remote = (num_nodes - 1) * groups_per_node;
     if (i < remote) {
-        const uint32_t node = (rank_node + 1 + i / node_size) % num_nodes;
-        return node * node_size + i % node_size;
+        const uint32_t node = (rank_node + 1 + i / groups_per_node) % num_nodes;
+        return node * groups_per_node + i % groups_per_node;
     }
-    const uint32_t local = i - remote + 1;  // 1 .. node_size
-    if (local < node_size) return rank_node * node_size + (rank + local) % node_size;
-    return rank;
+    const uint32_t local = i - remote + 1;  // 1 .. groups_per_node
+    if (local < groups_per_node) return rank_node * groups_per_node + (dp_group + local) % groups_per_node;
+    return dp_group;
 }
 
 }  // namespace a2a

@@ -139,7 +139,7 @@ __device__ void fold_source(const FinalizeArgs &args, const Workspace &ws, uint3
 // sends to local expert le.  Whole workgroup.
 __device__ void layout_from_totals(const FinalizeArgs &args, const Workspace &ws, uint32_t r,
                                    const uint32_t *tot, uint32_t *scratch) {
-    const uint32_t N = ws.world, E = ws.num_experts, Le = ws.experts_per_rank;
+    const uint32_t N = ws.num_groups, E = ws.num_experts, Le = ws.experts_per_rank;
     const uint32_t tid = threadIdx.x;
     const uint32_t pad = ws.expert_padding;
     const uint32_t e = r * Le + tid;
@@ -159,7 +159,7 @@ __device__ void layout_from_totals(const FinalizeArgs &args, const Workspace &ws
         // (a2a_worker.rs:681-694); each gets a contiguous run of rows.
         uint32_t running = poff;
         for (uint32_t i = 0; i < N; ++i) {
-            const uint32_t g = source_order(r, i, N, ws.node_size);
+            const uint32_t g = source_order(r, i, ws.world, ws.node_size, ws.dp_size);
             ws.slot_base[g * E + e] = running;
             running += tot[g * Le + tid];
         }
@@ -173,7 +173,7 @@ __device__ void layout_from_totals(const FinalizeArgs &args, const Workspace &ws
 // N * Le words.
 __device__ void layout_receiver(const FinalizeArgs &args, const Workspace &ws, uint32_t r, uint32_t *tot,
                                 uint32_t *scratch) {
-    const uint32_t N = ws.world, E = ws.num_experts, Le = ws.experts_per_rank;
+    const uint32_t N = ws.num_groups, E = ws.num_experts, Le = ws.experts_per_rank;
     const uint32_t tid = threadIdx.x;
     const uint32_t items = N * Le;              // (source, local expert) pairs
     for (uint32_t i = tid; i < items; i += blockDim.x) tot[i] = 0;
@@ -271,7 +271,7 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
     __shared__ uint16_t wave_hist[kRouteWaves][A2A_MAX_EXPERTS];
     // Which source and which chunk of it this workgroup handles (uniform).
     uint32_t g = 0;
-    while (g + 1 < ws.world && blockIdx.x >= args.block_start[g + 1]) ++g;
+    while (g + 1 < ws.num_groups && blockIdx.x >= args.block_start[g + 1]) ++g;
     const uint32_t chunk = blockIdx.x - args.block_start[g];
     const uint32_t count = rank_chunk(args.src[g], ws, g, chunk, wave_hist);
     if (threadIdx.x < ws.num_experts) {
@@ -283,7 +283,7 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
 // for them, so somebody else clears them.
 __device__ void clear_empty_sources(const FinalizeArgs &fin, const Workspace &ws) {
     const uint32_t E = ws.num_experts;
-    for (uint32_t g = 0; g < ws.world; ++g) {
+    for (uint32_t g = 0; g < ws.num_groups; ++g) {
         if ((fin.fold_mask >> g & 1) && fin.num_blocks[g] == 0 && threadIdx.x < E) {
             ws.num_routed[g * E + threadIdx.x] = 0;
             ws.expert_offsets[g * E + threadIdx.x] = 0;
@@ -343,7 +343,7 @@ __global__ __launch_bounds__(kRouteBlock) void route_fused_kernel(const RouteArg
     __shared__ uint16_t wave_hist[kRouteWaves][A2A_MAX_EXPERTS];
     __shared__ uint32_t tot[A2A_MAX_EXPERTS + kMaxWorld];
     __shared__ uint32_t scratch[kRouteWaves];
-    const uint32_t N = ws.world, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
+    const uint32_t N = ws.num_groups, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
     const uint32_t tid = threadIdx.x;
     const uint32_t chunk_blocks = args.block_start[N];
 
@@ -419,8 +419,8 @@ __global__ __launch_bounds__(kRouteBlock) void route_finalize_kernel(const Final
     __shared__ uint32_t tot[A2A_MAX_EXPERTS + kMaxWorld];
     __shared__ uint32_t scratch[kRouteWaves];
     if (blockIdx.x < ws.world) {
-        const uint32_t rank = blockIdx.x;
-        if (args.fold_mask >> rank & 1) fold_source(args, ws, rank, part_sum, scratch);
+        const uint32_t group = blockIdx.x;
+        if (group < ws.num_groups && (args.fold_mask >> group & 1)) fold_source(args, ws, group, part_sum, scratch);
     } else {
         const uint32_t rank = blockIdx.x - ws.world;
         if (args.recv_mask >> rank & 1) layout_receiver(args, ws, rank, tot, scratch);
@@ -436,7 +436,7 @@ hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t tot
 
 hipError_t launch_route_fused(const RouteArgs &args, const FinalizeArgs &fin, const Workspace &ws,
                               hipStream_t stream) {
-    const uint32_t blocks = args.block_start[ws.world] + (fin.recv_mask != 0 ? ws.world : 0);
+    const uint32_t blocks = args.block_start[ws.num_groups] + (fin.recv_mask != 0 ? ws.world : 0);
     if (blocks != 0) {
         hipLaunchKernelGGL(route_fused_kernel, dim3(blocks), dim3(kRouteBlock), 0, stream, args, fin, ws);
     } else {

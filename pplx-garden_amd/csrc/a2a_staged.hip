@@ -23,7 +23,7 @@ __global__ __launch_bounds__(1024) void stage_send_kernel(const StageSendArgs ar
     const uint32_t wave = tid / kWave;
     const uint32_t E = ws.num_experts;
     const uint32_t K = ws.topk;
-    const uint32_t g = args.rank;
+    const uint32_t g = args.rank / ws.dp_size;   // ranks of a dp group hold the same tokens
     const uint32_t token = blockIdx.x;
     const PushSrc &src = args.src;
     if (token >= effective_tokens(src.bound_m, src.num_tokens)) return;
@@ -88,14 +88,14 @@ __global__ __launch_bounds__(1024) void recv_segments_kernel(const StageRecvArgs
                                                              const Workspace ws, const Staging st) {
     __shared__ uint32_t wave_tot[16];
     __shared__ uint32_t carry_s;
-    const uint32_t N = ws.world, E = ws.num_experts, Le = ws.experts_per_rank;
+    const uint32_t G = ws.num_groups, E = ws.num_experts, Le = ws.experts_per_rank;
     const uint32_t r = args.rank;
     const uint32_t first = r * Le;
     const uint32_t n_local = first >= E ? 0 : (E - first < Le ? E - first : Le);
-    const uint32_t num_seg = N * Le;
-    uint32_t *seg = st.seg_start + (size_t)r * (N * Le + 1);
+    const uint32_t num_seg = G * Le;
+    uint32_t *seg = st.seg_start + (size_t)r * (ws.world * Le + 1);
     const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const uint32_t remote_segs = (N / ws.node_size - 1) * ws.node_size * Le;
+    const uint32_t remote_segs = (ws.world / ws.node_size - 1) * (ws.node_size / ws.dp_size) * Le;
 
     if (tid == 0) carry_s = 0;
     __syncthreads();
@@ -103,7 +103,7 @@ __global__ __launch_bounds__(1024) void recv_segments_kernel(const StageRecvArgs
         const uint32_t s = base + tid;
         uint32_t cnt = 0;
         if (s < num_seg) {
-            const uint32_t g = source_order(r, s / Le, N, ws.node_size);
+            const uint32_t g = source_order(r, s / Le, ws.world, ws.node_size, ws.dp_size);
             const uint32_t le = s % Le;
             if (le < n_local && (args.valid_mask >> g & 1)) cnt = ws.num_routed[g * E + first + le];
         }
@@ -153,15 +153,15 @@ __device__ __forceinline__ void locate_row(const uint32_t *seg, uint32_t num_seg
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs args, const Workspace ws,
                                                           const Staging st) {
-    const uint32_t N = ws.world, E = ws.num_experts, Le = ws.experts_per_rank;
+    const uint32_t E = ws.num_experts, Le = ws.experts_per_rank;
     const uint32_t r = args.rank;
-    const uint32_t num_seg = N * Le;
-    const uint32_t *seg = st.seg_start + (size_t)r * (num_seg + 1);
+    const uint32_t num_seg = ws.num_groups * Le;
+    const uint32_t *seg = st.seg_start + (size_t)r * (ws.world * Le + 1);
     const uint32_t i = blockIdx.x;
     if (i >= seg[num_seg]) return;
     uint32_t s, j;
     locate_row(seg, num_seg, i, &s, &j);
-    const uint32_t g = source_order(r, s / Le, N, ws.node_size);
+    const uint32_t g = source_order(r, s / Le, ws.world, ws.node_size, ws.dp_size);
     const uint32_t e = r * Le + s % Le;
     const uint32_t excl = e > 0 ? ws.expert_offsets[g * E + e - 1] : 0;
     const uint32_t pos = excl + j;
@@ -169,7 +169,8 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     const uint32_t tid = threadIdx.x;
     if (tid == 0 && i < st.max_recv) {
         st.padded_index[(size_t)r * st.max_recv + i] = dst_row;
-        st.source_rank[(size_t)r * st.max_recv + i] = g;
+        // the member of the group that sends to this rank (a2a_worker.rs:633)
+        st.source_rank[(size_t)r * st.max_recv + i] = g * ws.dp_size + r % ws.dp_size;
         st.source_position[(size_t)r * st.max_recv + i] = pos;
     }
     const PushDst &dst = args.dst;
@@ -206,7 +207,8 @@ __global__ __launch_bounds__(1024) void combine_send_kernel(const CombineSendArg
     const uint32_t i = blockIdx.x;
     if (i >= st.num_recv[2 * r] || i >= st.max_recv) return;
     const uint32_t row = st.padded_index[(size_t)r * st.max_recv + i];
-    const uint32_t g = st.source_rank[(size_t)r * st.max_recv + i];
+    // every member of the source's dp group reads the same staging rows
+    const uint32_t g = st.source_rank[(size_t)r * st.max_recv + i] / ws.dp_size;
     const uint32_t pos = st.source_position[(size_t)r * st.max_recv + i];
     if (row >= args.y_rows || pos >= ws.max_tk) {
         if (threadIdx.x == 0) atomicOr(ws.err, A2A_DEV_BAD_SLOT);
@@ -335,7 +337,7 @@ hipError_t launch_stage_send(const StageSendArgs &args, const Workspace &ws, con
 
 hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st,
                              hipStream_t stream) {
-    uint32_t seg_threads = (ws.world * ws.experts_per_rank + kWave - 1) / kWave * kWave;
+    uint32_t seg_threads = (ws.num_groups * ws.experts_per_rank + kWave - 1) / kWave * kWave;
     if (seg_threads > 1024) seg_threads = 1024;
     hipLaunchKernelGGL(recv_segments_kernel, dim3(1), dim3(seg_threads), 0, stream, args, ws, st);
     hipError_t e = hipGetLastError();

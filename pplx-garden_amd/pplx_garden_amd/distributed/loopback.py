@@ -42,6 +42,15 @@ class LoopbackGroup:
         """All logical ranks share the caller's thread: nothing to wait for."""
 
 
+@dataclass(frozen=True)
+class LoopbackSubGroup:
+    """A slice of the world, e.g. the ranks that hold the same tokens (`dp_group`) or the ranks of
+    one node (`node_group`): only `size` and the caller's `rank` inside it matter to the operator."""
+
+    size: int
+    rank: int
+
+
 class LoopbackWorld:
     def __init__(self, world_size: int, node_size: Optional[int] = None,
                  device: Optional[torch.device] = None) -> None:
@@ -61,6 +70,12 @@ class LoopbackWorld:
         if not 0 <= rank < self.size:
             raise ValueError(f"rank {rank} out of range [0, {self.size})")
         return LoopbackGroup(self, rank)
+
+    def dp_group(self, rank: int, dp_size: int) -> LoopbackSubGroup:
+        """The group of `dp_size` consecutive ranks that share `rank`'s tokens."""
+        if dp_size < 1 or self.node_size % dp_size != 0:
+            raise ValueError(f"dp_size {dp_size} does not divide node_size {self.node_size}")
+        return LoopbackSubGroup(size=dp_size, rank=rank % dp_size)
 
     @property
     def groups(self) -> List[LoopbackGroup]:

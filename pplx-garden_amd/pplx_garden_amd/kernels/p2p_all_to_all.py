@@ -11,6 +11,8 @@ receive counts as the reference's operator
   the world has made it, in one launch sequence that moves every row once.
   Calls with only `do_send` or only `do_recv` run at once, rank by rank, through
   staging buffers; every send of a step must come before the first recv.
+* ranks of one `dp_group` must pass the same tokens, indices and weights, as in the reference
+  (only one of them sends each copy, all of them receive the combined tokens).
 * `dp_x` may be bfloat16 while `in_dtype` is float8_e4m3fn and `dp_x_scale` is
   None: dispatch then quantises, one float32 scale per 128 elements
   (`hidden_dim_scale` must be `hidden_dim // 128`).  The reference only
@@ -72,9 +74,13 @@ class P2PAllToAll(AllToAllKernel):
 
         if not isinstance(global_group, LoopbackGroup):
             raise TypeError("global_group must be a LoopbackGroup (see LoopbackWorld.group)")
-        if dp_group is not None and dp_group.size != 1:
-            raise NotImplementedError("dp groups larger than 1 are not supported in loopback")
-        self._dp_size = 1
+        # Number of ranks that hold the same tokens (p2p_all_to_all.py:80-87).
+        if dp_group is not None:
+            self._dp_size = dp_group.size
+            if node_group is None and global_group.node_size % dp_group.size != 0:
+                node_group = dp_group
+        else:
+            self._dp_size = 1
 
         rank = global_group.rank
         world_size = global_group.size
@@ -120,7 +126,7 @@ class P2PAllToAll(AllToAllKernel):
         self._key = (
             hidden_dim, hidden_dim_scale, in_dtype, out_dtype, scale_dtype, max_num_tokens,
             max_recv_tokens, max_private_tokens, num_experts, expert_padding,
-            num_experts_per_token, node_size, world_size, device_index,
+            num_experts_per_token, node_size, world_size, device_index, self._dp_size,
         )
 
         def make_context() -> AllToAllContext:

@@ -42,23 +42,17 @@ def test_reference_matrix(cfg, split):
     check(cfg, world, rows, got)
 
 
+@pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
 @pytest.mark.parametrize("cfg", DP2, ids=lambda c: c.name)
-def test_dp_groups_are_refused(cfg):
-    """Ranks that share tokens (dp_size 2) are not built; the operator says so instead of
-    producing wrong rows."""
-    from pplx_garden_amd.distributed.loopback import LoopbackWorld
-    from pplx_garden_amd.kernels.p2p_all_to_all import P2PAllToAll
+def test_reference_matrix_dp2(cfg, split):
+    """The two configurations with ranks that share tokens (dp_size 2): ranks of a group pass the
+    same data, every rank receives its experts' rows and every rank gets the combined tokens."""
+    from a2a_dp import check_dp, run_gpu_dp
 
-    class Group:
-        size = cfg.dp_size
-
-    with pytest.raises(NotImplementedError):
-        P2PAllToAll(max_num_tokens=cfg.max_num_tokens, num_experts=cfg.num_experts, expert_padding=1,
-                    hidden_dim=cfg.hidden_dim, hidden_dim_scale=None, in_dtype=cfg.in_dtype,
-                    out_dtype=cfg.out_dtype, scale_dtype=None,
-                    num_experts_per_token=cfg.num_experts_per_token, nets_per_gpu=1, max_private_tokens=None,
-                    device=torch.device("cuda:0"), dp_group=Group(), node_group=None,
-                    global_group=LoopbackWorld(cfg.world_size).group(0))
+    print(f"cfg={cfg.name} split={split}", flush=True)
+    groups = [make_ref_rank(cfg, g) for g in range(cfg.world_size // cfg.dp_size)]
+    got, rows = run_gpu_dp(cfg, groups, torch.device("cuda:0"), split)
+    check_dp(cfg, groups, rows, got)
 
 
 def test_transposed_scale_output():

@@ -60,7 +60,8 @@ def _config(**over):
 @pytest.mark.parametrize("over,code,needle", [
     (dict(struct_size=4), -1, "struct_size"),
     (dict(world_size=33, node_size=33), -3, "world_size"),
-    (dict(dp_size=2), -3, "dp_size"),
+    (dict(dp_size=3, node_size=4, world_size=4), -1, "dp_size"),
+    (dict(dp_size=0), -1, "dp_size"),
     (dict(node_size=3), -1, "node_size"),
     (dict(num_experts=2000), -3, "num_experts"),
     (dict(num_experts_per_token=65), -3, "num_experts_per_token"),
