@@ -41,7 +41,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch on the default workload, from hardware counters (FETCH_SIZE and WRITE_SIZE
 # passes, scaled by what the same counters read for a 512 MiB copy: x2.000 and x1.000).  The counter
 # runs and their commands are summarised in profiles/hbm_traffic_dsv3_prefill_4096_push_and_combine.md.
-MEASURED_TRAFFIC_BYTES = {"combine_gather_kernel": 531_696_000, "dispatch_push_kernel": 303_049_000}
+MEASURED_TRAFFIC_BYTES = {"combine_gather_kernel": 531_696_000, "dispatch_push_kernel": 303_073_000}
 
 
 def algorithmic_bytes(T: int, H: int, K: int):

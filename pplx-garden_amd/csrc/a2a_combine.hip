@@ -196,7 +196,7 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
                    : ws.route_slot[(size_t)group * ws.max_tk + token * K + lane];
     }
     const bool expert_ok = expert < E;
-    const uint32_t r = expert_ok ? expert / ws.experts_per_rank : 0;
+    const uint32_t r = expert_ok ? owner_of_expert(ws, expert) : 0;
     const uint64_t r_base = __shfl(y_base, (int)r);
     const uint64_t r_stride = __shfl(y_stride, (int)r);
     const uint32_t r_rows = __shfl(y_rows, (int)r);

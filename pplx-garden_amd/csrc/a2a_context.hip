@@ -281,6 +281,7 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
     ws.experts_per_rank = ceil_div_u32(E, N);
     ws.node_size = config->node_size;
     ws.expert_padding = config->expert_padding;
+    ws.le_magic = ws.experts_per_rank > 1 ? 0xFFFFFFFFu / ws.experts_per_rank + 1 : 0;
 
     // One allocation, carved into 256-byte aligned tables.
     size_t off = 0;
@@ -300,6 +301,7 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
     const size_t o_slot = carve((size_t)N * ws.max_tk * sizeof(uint32_t));
     const size_t o_toff = carve((size_t)N * ws.max_tk * sizeof(uint32_t));
     const size_t o_err = carve(sizeof(uint32_t));
+    const size_t o_order = carve((size_t)N * kMaxWorld);
     ctx->arena_bytes = off;
     e = hipMalloc(&ctx->arena, ctx->arena_bytes);
     if (e != hipSuccess) {
@@ -325,6 +327,22 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
     ws.route_slot = reinterpret_cast<uint32_t *>(base + o_slot);
     ws.token_offset = reinterpret_cast<uint32_t *>(base + o_toff);
     ws.err = reinterpret_cast<uint32_t *>(base + o_err);
+    ws.order = reinterpret_cast<const uint32_t *>(base + o_order);
+    {
+        // i-th source each receiver lays out: fixed for the life of the context
+        uint8_t table[kMaxWorld * kMaxWorld] = {0};
+        for (uint32_t r = 0; r < N; ++r) {
+            for (uint32_t i = 0; i < ws.num_groups; ++i) {
+                table[r * kMaxWorld + i] = (uint8_t)source_order(r, i, N, config->node_size, config->dp_size);
+            }
+        }
+        e = hipMemcpy(base + o_order, table, (size_t)N * kMaxWorld, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            (void)hipFree(ctx->arena);
+            delete ctx;
+            return hip_fail(nullptr, e, "hipMemcpy(source order)");
+        }
+    }
 
     if (config->flags & A2A_FLAG_PREALLOC_STAGING) {
         std::string msg;
@@ -437,19 +455,25 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
     pa.row_bytes = (uint32_t)row_bytes_of(c);
     pa.hidden_dim = c.hidden_dim;
     pa.hidden_dim_scale = c.hidden_dim_scale;
+    pa.topk_magic = K > 1 ? (uint32_t)((0x100000000ull + K - 1) / K) : 0;
 
     hipError_t e;
-    if (fused_routing_pays(fa, G, blocks)) {
-        e = launch_route_fused(ra, fa, ctx->ws, s);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
+    if (dispatch_small_fits(pa, ctx->ws, quantize != 0, tokens)) {
+        e = launch_dispatch_small(pa, fa, ctx->ws, quantize != 0, tokens, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_small");
     } else {
-        e = launch_route(ra, ctx->ws, blocks, s);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
-        e = launch_finalize(fa, ctx->ws, s);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+        if (fused_routing_pays(fa, G, blocks)) {
+            e = launch_route_fused(ra, fa, ctx->ws, s);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
+        } else {
+            e = launch_route(ra, ctx->ws, blocks, s);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
+            e = launch_finalize(fa, ctx->ws, s);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+        }
+        e = launch_dispatch_push(pa, ctx->ws, quantize != 0, tokens, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_push");
     }
-    e = launch_dispatch_push(pa, ctx->ws, quantize != 0, tokens, s);
-    if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_push");
 
     ctx->group_routing = true;
     ctx->step_open = false;

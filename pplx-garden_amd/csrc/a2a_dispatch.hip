@@ -19,63 +19,26 @@
 // stores to this many rows at once sustain about two thirds of that rate, and
 // what ordinary stores leave in the cache is what the experts read next.
 #include "a2a_device.h"
+#include "a2a_scan.h"
 
 namespace a2a {
 
-template <bool QUANT>
-__global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args,
-                                                             const Workspace ws) {
-    // Scales of one token (one per 128 elements) and where each copy's go.
-    constexpr int kMaxLdsScales = 1024;
-    __shared__ float s_scale[QUANT ? kMaxLdsScales : 1];
-    __shared__ uint64_t s_scale_ptr[A2A_MAX_EXPERTS_PER_TOKEN];
-    __shared__ uint32_t s_scale_stride[A2A_MAX_EXPERTS_PER_TOKEN];
+namespace {
 
+constexpr int kMaxLdsScales = 1024;
+
+// Moves the row of `token` to its copies.  Lanes 0..K-1 of EVERY wavefront hold
+// the row pointer, scale pointer and scale stride of route k (0 = no copy).
+// With PRELOADED, `pre_a`/`pre_b` already hold the chunk of this thread's first
+// iteration (loaded by the caller before it knew the routes).  Whole workgroup.
+template <bool QUANT, bool PRELOADED>
+__device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &src, uint32_t token, uint32_t K,
+                                          uint64_t row_ptr, uint64_t scale_ptr, uint32_t scale_stride,
+                                          float *s_scale, uint64_t *s_scale_ptr, uint32_t *s_scale_stride,
+                                          u32x4 pre_a, u32x4 pre_b) {
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
-    const uint32_t E = ws.num_experts;
-    const uint32_t K = ws.topk;
-
-    uint32_t g = 0;
-    while (g + 1 < ws.num_groups && blockIdx.x >= args.token_start[g + 1]) ++g;
-    const uint32_t token = blockIdx.x - args.token_start[g];
-    const PushSrc &src = args.src[g];
-    if (token >= effective_tokens(src.bound_m, src.num_tokens)) return;
-
-    // Lanes 0..K-1 of every wavefront resolve one route each.
-    uint64_t row_ptr = 0, scale_ptr = 0;
-    uint32_t scale_stride = 0;
-    if (lane < K) {
-        const uint32_t entry = token * K + lane;
-        const uint32_t expert =
-            (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
-        uint32_t slot = kInvalidSlot, toff = 0;
-        if (expert < E) {
-            const uint32_t chunk = entry / kRouteBlock;
-            toff = ws.block_prefix[((size_t)g * ws.nb_max + chunk) * E + expert] +
-                   ws.local_rank[(size_t)g * ws.max_tk + entry];
-            slot = ws.slot_base[g * E + expert] + toff;
-            const PushDst &dst = args.dst[expert / ws.experts_per_rank];
-            if (dst.out_x != nullptr) {
-                if (slot < dst.out_rows) {
-                    row_ptr = (uint64_t)(dst.out_x + (size_t)slot * dst.out_stride);
-                    if (dst.out_scale != nullptr) {
-                        scale_ptr = (uint64_t)(dst.out_scale + (size_t)slot * dst.os_stride_token);
-                        scale_stride = dst.os_stride_elem;
-                    }
-                } else {
-                    slot = kInvalidSlot;
-                    if (wave == 0) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
-                }
-            }
-        }
-        if (wave == 0) {
-            ws.route_slot[(size_t)g * ws.max_tk + entry] = slot;
-            ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
-        }
-    }
-
     const uint8_t *x_row = src.x + (size_t)token * src.x_stride;
 
     if constexpr (QUANT) {
@@ -85,7 +48,10 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
             const uint32_t c = base + lane;
             const bool active = c < num_chunks;
             u32x4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
-            if (active) {
+            if (PRELOADED && base == wave * kWave) {
+                a = pre_a;
+                b = pre_b;
+            } else if (active) {
                 const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)c * 32);
                 a = __builtin_nontemporal_load(p);
                 b = __builtin_nontemporal_load(p + 1);
@@ -117,8 +83,12 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
     } else {
         const uint32_t num_chunks = args.row_bytes / 16;
         for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
-            const u32x4 v =
-                __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
+            u32x4 v;
+            if (PRELOADED && c == tid) {
+                v = pre_a;
+            } else {
+                v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
+            }
             for (uint32_t k = 0; k < K; ++k) {
                 const uint64_t row = read_lane64(row_ptr, k);
                 if (row != 0) {
@@ -140,9 +110,27 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
     }
 }
 
-hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool quantize,
-                                uint32_t total_tokens, hipStream_t stream) {
-    if (total_tokens == 0) return hipSuccess;
+// Where the copy of one route goes: row `slot` of the receiver described by `dst`.  Returns the slot that is recorded for the combine (kInvalidSlot if
+// the row does not fit the receiver's buffer).
+__device__ __forceinline__ uint32_t resolve_copy(const PushDst &dst, const Workspace &ws, uint32_t slot,
+                                                 bool flag_overflow, uint64_t *row_ptr, uint64_t *scale_ptr,
+                                                 uint32_t *scale_stride) {
+    if (dst.out_x != nullptr) {
+        if (slot < dst.out_rows) {
+            *row_ptr = (uint64_t)(dst.out_x + (size_t)slot * dst.out_stride);
+            if (dst.out_scale != nullptr) {
+                *scale_ptr = (uint64_t)(dst.out_scale + (size_t)slot * dst.os_stride_token);
+                *scale_stride = dst.os_stride_elem;
+            }
+        } else {
+            slot = kInvalidSlot;
+            if (flag_overflow) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+        }
+    }
+    return slot;
+}
+
+uint32_t push_threads(const PushArgs &args, bool quantize) {
     const uint32_t chunks = quantize ? args.hidden_dim / 16 : args.row_bytes / 16;
 #ifndef A2A_PUSH_SLABS
 #define A2A_PUSH_SLABS 1
@@ -150,12 +138,337 @@ hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool 
     uint32_t threads = ((chunks + kWave - 1) / kWave + A2A_PUSH_SLABS - 1) / A2A_PUSH_SLABS * kWave;
     if (threads < (uint32_t)kWave) threads = kWave;
     if (threads > 1024) threads = 1024;
+    return threads;
+}
+
+}  // namespace
+
+template <bool QUANT>
+__global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args,
+                                                             const Workspace ws) {
+    // Scales of one token (one per 128 elements) and where each copy's go.
+    __shared__ float s_scale[QUANT ? kMaxLdsScales : 1];
+    __shared__ uint64_t s_scale_ptr[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint32_t s_scale_stride[A2A_MAX_EXPERTS_PER_TOKEN];
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const uint32_t E = ws.num_experts;
+    const uint32_t K = ws.topk;
+
+    uint32_t g = 0;
+    while (g + 1 < ws.num_groups && blockIdx.x >= args.token_start[g + 1]) ++g;
+    const uint32_t token = blockIdx.x - args.token_start[g];
+    const PushSrc &src = args.src[g];
+    if (token >= effective_tokens(src.bound_m, src.num_tokens)) return;
+
+    // Lanes 0..K-1 of every wavefront resolve one route each.
+    uint64_t row_ptr = 0, scale_ptr = 0;
+    uint32_t scale_stride = 0;
+    if (lane < K) {
+        const uint32_t entry = token * K + lane;
+        const uint32_t expert =
+            (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
+        uint32_t slot = kInvalidSlot, toff = 0;
+        if (expert < E) {
+            const uint32_t chunk = entry / kRouteBlock;
+            toff = ws.block_prefix[((size_t)g * ws.nb_max + chunk) * E + expert] +
+                   ws.local_rank[(size_t)g * ws.max_tk + entry];
+            slot = ws.slot_base[g * E + expert] + toff;
+            slot = resolve_copy(args.dst[owner_of_expert(ws, expert)], ws, slot, wave == 0, &row_ptr, &scale_ptr,
+                                &scale_stride);
+        }
+        if (wave == 0) {
+            ws.route_slot[(size_t)g * ws.max_tk + entry] = slot;
+            ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
+        }
+    }
+    const u32x4 none = {0, 0, 0, 0};
+    push_rows<QUANT, false>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr,
+                            s_scale_stride, none, none);
+}
+
+// Routing pass and dispatch pack in ONE launch, for small steps (decode).  The
+// grid holds one workgroup per token, then one per receiver; none depends on
+// another, because every workgroup counts, by itself, what it needs to know
+// about the whole step:
+//  - a token workgroup asks for its row early, counts the entries of every
+//    source per (source, expert) and the entries of its own source before its
+//    token per expert (LDS atomics: counts do not depend on arrival order), and
+//    from those derives the receiver rows of its K copies exactly as the
+//    two-launch pass does: first row of the expert in its receiver + copies of
+//    the sources the receiver lays out earlier + copies of its own source
+//    before it, in (token, k) order.  The workgroup of a source's first token
+//    also publishes the source's per-expert totals and their scan.
+//  - a receiver workgroup counts the copies bound for its experts and lays out
+//    its rows (expert counts for the caller, first row per expert and source).
+// The counting is redundant: its cost grows with tokens x entries, so the host
+// takes this path only below a bound on the entries of a step.
+//
+// Dynamic LDS: (G + 3) * E words and 8 bytes per token of the step.
+template <bool QUANT>
+__global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs args, const FinalizeArgs fin,
+                                                              const Workspace ws) {
+    extern __shared__ uint64_t s_dyn64[];
+    uint32_t *s_dyn = reinterpret_cast<uint32_t *>(s_dyn64);
+    __shared__ float s_scale[QUANT ? kMaxLdsScales : 1];
+    __shared__ uint64_t s_scale_ptr[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint32_t s_scale_stride[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ PushDst s_dst[kMaxWorld];                      // per receiver: its buffers
+    __shared__ uint32_t s_order[kMaxWorld * kMaxWorld / 4];   // [receiver] bytes: i -> source
+    __shared__ uint32_t scratch[kRouteWaves];
+    __shared__ uint32_t s_carry;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const uint32_t G = ws.num_groups, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
+    const uint32_t total_tokens = args.token_start[G];
+    const uint32_t total_entries = total_tokens * K;
+    const bool receiver = blockIdx.x >= total_tokens;
+
+    // Per token of the step (all sources, in grid order): where its K expert ids
+    // are, with the source in the top byte; 0 for tokens past their source's
+    // bound.  This is what the counting pass below looks up per entry.
+    const uint32_t table_words = ((G + 3) * E + 1) & ~1u;
+    uint64_t *tok_ids = reinterpret_cast<uint64_t *>(s_dyn + table_words);
+    for (uint32_t ft = tid; ft < total_tokens; ft += blockDim.x) {
+        // token_start is non-decreasing and equals the total from G on, so the
+        // fixed trip count is safe and lets the loads go out together
+        uint32_t g = 0, start = 0;
+#pragma unroll
+        for (uint32_t gg = 1; gg < (uint32_t)kMaxWorld; ++gg) {
+            const uint32_t first = args.token_start[gg];
+            if (ft >= first) {
+                g = gg;
+                start = first;
+            }
+        }
+        const PushSrc &from = args.src[g];
+        const uint32_t t = ft - start;
+        const uint64_t ids = (uint64_t)(from.indices + (size_t)t * from.indices_stride) | (uint64_t)g << 56;
+        tok_ids[ft] = t < effective_tokens(from.bound_m, from.num_tokens) ? ids : 0;
+    }
+    uint32_t *cnt = s_dyn;                                  // [G][E] or, receivers, [G][Le]
+    uint32_t *prior = s_dyn + (size_t)G * E;                // [E] own source, tokens before mine
+    uint32_t *rows_before = prior + E;                      // [E] padded rows of all experts before e
+    uint32_t *copies_before = rows_before + E;              // [E] copies of the sources laid out before mine
+    const uint32_t table = receiver ? G * Le : G * E + E;
+    for (uint32_t i = tid; i < table; i += blockDim.x) s_dyn[i] = 0;
+    uint32_t my_g = 0, token = 0;
+    if (!receiver) {
+        while (my_g + 1 < G && blockIdx.x >= args.token_start[my_g + 1]) ++my_g;
+        token = blockIdx.x - args.token_start[my_g];
+        if (tid < ws.world) s_dst[tid] = args.dst[tid];
+    }
+    // Sources without tokens have no workgroup of their own: the first receiver
+    // workgroup (the first workgroup, if nobody receives) clears their tables.
+    if (blockIdx.x == (fin.recv_mask != 0 ? total_tokens : 0)) {
+        for (uint32_t g = 0; g < G; ++g) {
+            if (args.src[g].num_tokens != 0) continue;
+            for (uint32_t e = tid; e < E; e += blockDim.x) {
+                ws.num_routed[g * E + e] = 0;
+                ws.expert_offsets[g * E + e] = 0;
+            }
+        }
+    }
+    __syncthreads();
+
+    // One pass over the entries of all sources, kBatch loads in flight per lane.
+#ifndef A2A_SMALL_BATCH
+#define A2A_SMALL_BATCH 8
+#endif
+    constexpr uint32_t kBatch = A2A_SMALL_BATCH;
+    // The token's own row is requested right after the first batch of indices,
+    // so that counting does not wait for it.
+    const PushSrc &src = args.src[my_g];
+    const uint32_t rank = blockIdx.x - total_tokens;        // receivers only
+    const uint32_t my_first = (args.token_start[my_g] + token) * K;   // flat index of my first entry
+    uint32_t my_expert = 0xFFFFFFFFu;
+    u32x4 pre_a = {0, 0, 0, 0}, pre_b = {0, 0, 0, 0};
+    // The order in which every receiver lays out the sources comes from device
+    // memory: asked for here, stored to LDS after the counting.
+    const uint32_t order_words = receiver ? 0 : ws.world * (kMaxWorld / 4);
+    const uint32_t order_word = tid < order_words ? ws.order[tid] : 0;
+    for (uint32_t f0 = 0; f0 < total_entries || f0 == 0; f0 += kBatch * blockDim.x) {
+        uint32_t expert[kBatch], src_of[kBatch];
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t f = f0 + j * blockDim.x + tid;
+            expert[j] = 0xFFFFFFFFu;
+            src_of[j] = 0;
+            if (f < total_entries) {
+                const uint32_t flat_token = K > 1 ? __umulhi(f, args.topk_magic) : f;
+                const uint64_t ids = tok_ids[flat_token];
+                src_of[j] = (uint32_t)(ids >> 56);
+                if (ids != 0) {
+                    expert[j] = (uint32_t) reinterpret_cast<const int32_t *>(ids & 0x00FFFFFFFFFFFFFFull)[f - flat_token * K];
+                }
+            }
+        }
+        if (f0 == 0 && !receiver) {
+            if (lane < K) my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
+            const uint8_t *x_row = src.x + (size_t)token * src.x_stride;
+            if constexpr (QUANT) {
+                if (tid < args.hidden_dim / 16) {
+                    const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)tid * 32);
+                    pre_a = __builtin_nontemporal_load(p);
+                    pre_b = __builtin_nontemporal_load(p + 1);
+                }
+            } else {
+                if (tid < args.row_bytes / 16) {
+                    pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + tid);
+                }
+            }
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t x = expert[j];
+            if (x >= E) continue;
+            if (receiver) {
+                const uint32_t le = x - rank * Le;   // wraps for experts of lower ranks
+                if (le < Le) atomicAdd(&cnt[src_of[j] * Le + le], 1u);
+            } else {
+                atomicAdd(&cnt[src_of[j] * E + x], 1u);
+                const uint32_t f = f0 + j * blockDim.x + tid;
+                if (src_of[j] == my_g && f < my_first) atomicAdd(&prior[x], 1u);
+            }
+        }
+    }
+    if (tid < order_words) s_order[tid] = order_word;
+    for (uint32_t i = tid + blockDim.x; i < order_words; i += blockDim.x) s_order[i] = ws.order[i];
+    __syncthreads();
+
+    if (receiver) {
+        if (fin.recv_mask >> rank & 1) layout_from_totals(fin, ws, rank, cnt, scratch);
+        return;
+    }
+
+    const uint32_t pad = ws.expert_padding;
+    // Per expert: padded rows of the experts before it (a scan; the difference to
+    // the scan at the first expert of a receiver is the expert's first row there)
+    // and the copies of the sources its receiver lays out before mine.
+    uint32_t carry = 0;
+    for (uint32_t e0 = 0; e0 < E; e0 += blockDim.x) {
+        const uint32_t e = e0 + tid;
+        uint32_t total = 0, before = 0;
+        if (e < E) {
+            const uint32_t r = owner_of_expert(ws, e);
+            bool seen = false;
+            // eight sources at a time, their LDS reads in flight together
+            for (uint32_t i0 = 0; i0 < G; i0 += 8) {
+                const uint32_t w0 = s_order[r * (kMaxWorld / 4) + i0 / 4];
+                const uint32_t w1 = s_order[r * (kMaxWorld / 4) + i0 / 4 + 1];
+                uint32_t g[8], c[8];
+#pragma unroll
+                for (uint32_t j = 0; j < 8; ++j) {
+                    g[j] = (j < 4 ? w0 >> (8 * j) : w1 >> (8 * (j - 4))) & 0xFFu;
+                    c[j] = i0 + j < G ? cnt[g[j] * E + e] : 0;
+                }
+#pragma unroll
+                for (uint32_t j = 0; j < 8; ++j) {
+                    seen = seen || (i0 + j < G && g[j] == my_g);
+                    if (!seen) before += c[j];
+                    total += c[j];
+                }
+            }
+        }
+        const uint32_t padded = e < E ? (total + pad - 1) / pad * pad : 0;
+        const uint32_t incl = carry + block_inclusive_scan(padded, scratch);
+        if (e < E) {
+            rows_before[e] = incl - padded;
+            copies_before[e] = before;
+        }
+        if (e0 + blockDim.x < E) {   // uniform: another round follows
+            if (tid == blockDim.x - 1) s_carry = incl;
+            __syncthreads();
+            carry = s_carry;
+        }
+    }
+    __syncthreads();
+
+    // The first token's workgroup publishes its source's totals (last wavefront).
+    if (token == 0 && wave == blockDim.x / kWave - 1) {
+        uint32_t run = 0;
+        for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
+            const uint32_t e = e0 + lane;
+            const uint32_t v = e < E ? cnt[my_g * E + e] : 0;
+            const uint32_t incl = run + wave_inclusive_scan(v, lane);
+            if (e < E) {
+                ws.num_routed[my_g * E + e] = v;
+                ws.expert_offsets[my_g * E + e] = incl;
+            }
+            run = __shfl(incl, kWave - 1);
+        }
+    }
+    if (token >= effective_tokens(src.bound_m, src.num_tokens)) return;   // nothing to send (uniform)
+
+    // Lanes 0..K-1 of every wavefront resolve one route each, from LDS alone.
+    uint32_t repeats = 0;   // copies of this token to the same expert at an earlier k
+    for (uint32_t k = 0; k + 1 < K; ++k) {
+        const uint32_t other = (uint32_t)__builtin_amdgcn_readlane((int)my_expert, (int)k);
+        if (k < lane && other == my_expert) ++repeats;
+    }
+    uint64_t row_ptr = 0, scale_ptr = 0;
+    uint32_t scale_stride = 0;
+    if (lane < K) {
+        const uint32_t entry = token * K + lane;
+        uint32_t slot = kInvalidSlot, toff = 0;
+        if (my_expert < E) {
+            // copies of my source before this one: earlier tokens, then earlier k of this token
+            toff = prior[my_expert] + repeats;
+            const uint32_t r = owner_of_expert(ws, my_expert);
+            const uint32_t row = rows_before[my_expert] - rows_before[r * Le] + copies_before[my_expert];
+            slot = resolve_copy(s_dst[r], ws, row + toff, wave == 0, &row_ptr, &scale_ptr, &scale_stride);
+        } else if (wave == 0) {
+            atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
+        }
+        if (wave == 0) {
+            ws.route_slot[(size_t)my_g * ws.max_tk + entry] = slot;
+            ws.token_offset[(size_t)my_g * ws.max_tk + entry] = toff;
+        }
+    }
+    push_rows<QUANT, true>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr,
+                           s_scale_stride, pre_a, pre_b);
+}
+
+hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool quantize,
+                                uint32_t total_tokens, hipStream_t stream) {
+    if (total_tokens == 0) return hipSuccess;
+    const uint32_t threads = push_threads(args, quantize);
     if (quantize) {
         hipLaunchKernelGGL(dispatch_push_kernel<true>, dim3(total_tokens), dim3(threads), 0, stream,
                            args, ws);
     } else {
         hipLaunchKernelGGL(dispatch_push_kernel<false>, dim3(total_tokens), dim3(threads), 0,
                            stream, args, ws);
+    }
+    return hipGetLastError();
+}
+
+bool dispatch_small_fits(const PushArgs &args, const Workspace &ws, bool quantize, uint32_t total_tokens) {
+    const uint64_t entries = (uint64_t)total_tokens * ws.topk;
+    const uint64_t table = ((uint64_t)ws.num_groups + 3) * ws.num_experts;
+    // The counting is redundant: every token workgroup visits every entry.  Measured with 8
+    // sources and 8 entries per token, the one launch is ahead of routing + push launches by
+    // 10 us at 512 tokens x 4096 entries (17 against 27 us) and by 3 us at 1024 x 8192.
+    return entries <= A2A_SMALL_MAX_ENTRIES && entries * total_tokens <= A2A_SMALL_MAX_VISITS &&
+           total_tokens <= 1024 && table <= 8192 + 3072 &&
+           ws.experts_per_rank <= push_threads(args, quantize);
+}
+
+hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
+                                 bool quantize, uint32_t total_tokens, hipStream_t stream) {
+    const uint32_t threads = push_threads(args, quantize);
+    const uint32_t blocks = total_tokens + (fin.recv_mask != 0 ? ws.world : 0);
+    if (blocks == 0) return hipSuccess;
+    const size_t table_words = (((size_t)ws.num_groups + 3) * ws.num_experts + 1) & ~(size_t)1;
+    const size_t lds = table_words * sizeof(uint32_t) + (size_t)total_tokens * sizeof(uint64_t);
+    if (quantize) {
+        hipLaunchKernelGGL(dispatch_small_kernel<true>, dim3(blocks), dim3(threads), lds, stream, args, fin, ws);
+    } else {
+        hipLaunchKernelGGL(dispatch_small_kernel<false>, dim3(blocks), dim3(threads), lds, stream, args, fin, ws);
     }
     return hipGetLastError();
 }

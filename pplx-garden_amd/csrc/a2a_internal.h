@@ -31,6 +31,7 @@ struct Workspace {
     uint32_t *route_slot;      // [N][max_tk]    receiver row of every copy (kInvalidSlot if dropped)
     uint32_t *token_offset;    // [N][max_tk]    rank of every copy inside its (source, expert)
     uint32_t *err;             // [1]            A2A_DEV_* bits, sticky
+    const uint32_t *order;     // [N][8] words   byte i of receiver r's row: the i-th source it lays out
     uint32_t max_tk;           // max_num_tokens * K
     uint32_t nb_max;           // ceil(max_tk / kRouteBlock)
     uint32_t world;            // N logical ranks (receivers)
@@ -41,6 +42,7 @@ struct Workspace {
     uint32_t experts_per_rank; // Le = ceil(E / N)
     uint32_t node_size;
     uint32_t expert_padding;
+    uint32_t le_magic;         // ceil(2^32 / Le) (0 for Le = 1): e / Le = mulhi(e, le_magic) for every expert id
 };
 
 struct RouteSrc {
@@ -94,6 +96,7 @@ struct PushArgs {
     uint32_t row_bytes;                   // bytes of a dispatched row
     uint32_t hidden_dim;
     uint32_t hidden_dim_scale;
+    uint32_t topk_magic;                  // ceil(2^32 / K) (0 for K = 1): n / K = mulhi(n, magic) while n * K < 2^32
 };
 
 struct CombSrc {  // one per receiver rank: the expert outputs it holds
@@ -137,6 +140,16 @@ hipError_t launch_route_fused(const RouteArgs &args, const FinalizeArgs &fin, co
                               hipStream_t stream);
 hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool quantize,
                                 uint32_t total_tokens, hipStream_t stream);
+// One-launch routing + pack for small steps: whether a step qualifies, and the launch.
+#ifndef A2A_SMALL_MAX_ENTRIES
+#define A2A_SMALL_MAX_ENTRIES 8192
+#endif
+#ifndef A2A_SMALL_MAX_VISITS
+#define A2A_SMALL_MAX_VISITS (8u << 20)   // entries x tokens
+#endif
+bool dispatch_small_fits(const PushArgs &args, const Workspace &ws, bool quantize, uint32_t total_tokens);
+hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
+                                 bool quantize, uint32_t total_tokens, hipStream_t stream);
 hipError_t launch_combine_gather(const CombArgs &args, const Workspace &ws, uint32_t in_dtype,
                                  uint32_t out_dtype, uint32_t total_tokens, hipStream_t stream);
 
@@ -166,6 +179,18 @@ __host__ __device__ __forceinline__ uint32_t source_order(uint32_t rank, uint32_
     const uint32_t local = i - remote + 1;  // 1 .. groups_per_node
     if (local < groups_per_node) return rank_node * groups_per_node + (dp_group + local) % groups_per_node;
     return dp_group;
+}
+
+
+// Rank that owns expert `e` (e < num_experts), without a division.
+__device__ __forceinline__ uint32_t owner_of_expert(const Workspace &ws, uint32_t e) {
+    return ws.experts_per_rank > 1 ? __umulhi(e, ws.le_magic) : e;
+}
+
+// The same order from the table the context computes once (kMaxWorld bytes per
+// receiver, four to a word).  With a uniform `rank` and `i` the loads are scalar.
+__device__ __forceinline__ uint32_t source_order_lookup(const uint32_t *order, uint32_t rank, uint32_t i) {
+    return order[rank * (kMaxWorld / 4) + (i >> 2)] >> (8 * (i & 3)) & 0xFFu;
 }
 
 }  // namespace a2a

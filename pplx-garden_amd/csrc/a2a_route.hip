@@ -25,37 +25,11 @@
 // of every source.  Each workgroup reads what it needs straight from the
 // histograms (one round trip to memory, all loads in flight together), so no
 // workgroup depends on another.
-#include "a2a_internal.h"
+#include "a2a_scan.h"
 
 namespace a2a {
 
 namespace {
-
-constexpr int kRouteWaves = kRouteBlock / kWave;
-
-// Inclusive scan over the 64 lanes of a wavefront.
-__device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, uint32_t lane) {
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        const uint32_t up = __shfl_up(v, d);
-        if (lane >= (uint32_t)d) v += up;
-    }
-    return v;
-}
-
-// Inclusive scan over the first blockDim.x values (one per thread); `scratch`
-// holds one word per wavefront.  Every thread of the workgroup must call.
-__device__ __forceinline__ uint32_t block_inclusive_scan(uint32_t v, uint32_t *scratch) {
-    const uint32_t lane = threadIdx.x & (kWave - 1);
-    const uint32_t wave = threadIdx.x / kWave;
-    const uint32_t incl = wave_inclusive_scan(v, lane);
-    __syncthreads();
-    if (lane == kWave - 1) scratch[wave] = incl;
-    __syncthreads();
-    uint32_t before = 0;
-    for (uint32_t w = 0; w < wave; ++w) before += scratch[w];
-    return before + incl;
-}
 
 // Sum of `n` words spaced `stride` apart, loads batched eight at a time so
 // that they are in flight together.
@@ -134,38 +108,6 @@ __device__ void fold_source(const FinalizeArgs &args, const Workspace &ws, uint3
     const uint32_t incl = block_inclusive_scan(owner ? total : 0, scratch);
     if (owner) ws.expert_offsets[g * E + e0] = incl;
 }
-
-// Rows of receiver `r` from `tot[g * Le + le]`, the number of copies source g
-// sends to local expert le.  Whole workgroup.
-__device__ void layout_from_totals(const FinalizeArgs &args, const Workspace &ws, uint32_t r,
-                                   const uint32_t *tot, uint32_t *scratch) {
-    const uint32_t N = ws.num_groups, E = ws.num_experts, Le = ws.experts_per_rank;
-    const uint32_t tid = threadIdx.x;
-    const uint32_t pad = ws.expert_padding;
-    const uint32_t e = r * Le + tid;
-    const bool mine = tid < Le && e < E;
-    uint32_t tpe = 0;
-    if (mine) {
-        for (uint32_t g = 0; g < N; ++g) tpe += tot[g * Le + tid];
-    }
-    const uint32_t padded = (tpe + pad - 1) / pad * pad;
-    const uint32_t poff = block_inclusive_scan(mine ? padded : 0, scratch) - padded;
-    if (mine) {
-        ws.tokens_per_expert[e] = tpe;
-        ws.padded_offset[e] = poff;
-        if (args.out_num_tokens[r] != nullptr) args.out_num_tokens[r][tid] = (int32_t)tpe;
-        if (poff + tpe > args.out_rows[r]) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
-        // Sources in the order the reference's host worker visits them
-        // (a2a_worker.rs:681-694); each gets a contiguous run of rows.
-        uint32_t running = poff;
-        for (uint32_t i = 0; i < N; ++i) {
-            const uint32_t g = source_order(r, i, ws.world, ws.node_size, ws.dp_size);
-            ws.slot_base[g * E + e] = running;
-            running += tot[g * Le + tid];
-        }
-    }
-}
-
 
 // Receiver part of the finalize: rows of receiver `r`, from the chunk
 // histograms of the sources folded by this launch and the published counts of

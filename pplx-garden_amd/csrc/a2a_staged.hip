@@ -103,7 +103,7 @@ __global__ __launch_bounds__(1024) void recv_segments_kernel(const StageRecvArgs
         const uint32_t s = base + tid;
         uint32_t cnt = 0;
         if (s < num_seg) {
-            const uint32_t g = source_order(r, s / Le, ws.world, ws.node_size, ws.dp_size);
+            const uint32_t g = source_order_lookup(ws.order, r, s / Le);
             const uint32_t le = s % Le;
             if (le < n_local && (args.valid_mask >> g & 1)) cnt = ws.num_routed[g * E + first + le];
         }
@@ -161,7 +161,7 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     if (i >= seg[num_seg]) return;
     uint32_t s, j;
     locate_row(seg, num_seg, i, &s, &j);
-    const uint32_t g = source_order(r, s / Le, ws.world, ws.node_size, ws.dp_size);
+    const uint32_t g = source_order_lookup(ws.order, r, s / Le);
     const uint32_t e = r * Le + s % Le;
     const uint32_t excl = e > 0 ? ws.expert_offsets[g * E + e - 1] : 0;
     const uint32_t pos = excl + j;
