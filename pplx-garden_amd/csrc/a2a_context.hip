@@ -687,17 +687,8 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
     DeviceGuard guard(c.device);
     hipStream_t s = static_cast<hipStream_t>(stream);
 
-    FinalizeArgs fa;
-    memset(&fa, 0, sizeof fa);
-    fa.fold_mask = 0;
-    fa.valid_mask = ctx->sent_mask;
-    fa.recv_mask = 1u << rank;
-    fa.out_num_tokens[rank] = out_num_tokens;
-    fa.out_rows[rank] = out_x != nullptr ? (uint32_t)(out_x_rows > 0xFFFFFFFFull ? 0xFFFFFFFFull : out_x_rows)
-                                         : 0xFFFFFFFFu;
-    hipError_t e = launch_finalize(fa, ctx->ws, s);
-    if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
-
+    const uint32_t out_rows = out_x != nullptr ? (uint32_t)(out_x_rows > 0xFFFFFFFFull ? 0xFFFFFFFFull : out_x_rows)
+                                               : 0xFFFFFFFFu;
     StageRecvArgs rv;
     memset(&rv, 0, sizeof rv);
     rv.rank = rank;
@@ -707,11 +698,12 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
     rv.dst.out_stride = out_x_stride;
     rv.dst.os_stride_elem = (uint32_t)out_x_scale_stride_elem;
     rv.dst.os_stride_token = (uint32_t)out_x_scale_stride_token;
-    rv.dst.out_rows = fa.out_rows[rank];
+    rv.dst.out_rows = out_rows;
+    rv.out_num_tokens = out_num_tokens;
     rv.row_bytes = (uint32_t)row_bytes_of(c);
     rv.hidden_dim_scale = c.hidden_dim_scale;
     rv.max_rows = rows_upper_bound(ctx);
-    e = launch_stage_recv(rv, ctx->ws, ctx->staging, s);
+    hipError_t e = launch_stage_recv(rv, ctx->ws, ctx->staging, s);
     if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_recv");
     ctx->recv_seen = true;
     ctx->staging.recv_mask |= 1u << rank;

@@ -25,7 +25,6 @@ struct Staging {
     uint8_t *send_buf = nullptr;         // [N][max_num_tokens][disp_stride]: payload, scales, 16 spare bytes
     uint32_t *pos_token = nullptr;       // [N][max_tk]: token behind each row of a sender's expert-sorted order
     uint8_t *comb_buf = nullptr;         // [N][max_tk][comb_stride]: combine rows at the sender's positions
-    uint32_t *seg_start = nullptr;       // [N][N*Le + 1]: first received row of each (source, local expert) run
     uint32_t *padded_index = nullptr;    // [N][max_recv]
     uint32_t *source_rank = nullptr;     // [N][max_recv]
     uint32_t *source_position = nullptr; // [N][max_recv]
@@ -49,11 +48,13 @@ struct StageSendArgs {
 
 struct StageRecvArgs {
     PushDst dst;
+    int32_t *out_num_tokens;  // rows per local expert for the caller, may be null
     uint32_t rank;
     uint32_t valid_mask;
     uint32_t row_bytes;
     uint32_t hidden_dim_scale;
     uint32_t max_rows;        // upper bound of received rows known to the host
+    uint32_t team_waves;      // wavefronts that share a row (set by the launcher)
 };
 
 struct CombineSendArgs {
@@ -63,6 +64,7 @@ struct CombineSendArgs {
     uint32_t rank;
     uint32_t row_bytes;
     uint32_t max_rows;
+    uint32_t team_waves;      // wavefronts that share a row (set by the launcher)
 };
 
 struct CombineRecvArgs {

@@ -4,6 +4,7 @@
 #include <cstring>
 
 #include "a2a_device.h"
+#include "a2a_scan.h"
 
 namespace a2a {
 
@@ -79,119 +80,176 @@ __global__ __launch_bounds__(1024) void stage_send_kernel(const StageSendArgs ar
     }
 }
 
+// A team of `team` threads (one or more whole wavefronts) copies a row of
+// `num_chunks` 16-byte pieces: eight loads per thread in flight, non-temporal
+// both ways (rows are read once and written once).
+__device__ __forceinline__ void copy_row_by_team(const u32x4 *src, u32x4 *dst, uint32_t num_chunks, uint32_t member,
+                                                 uint32_t team) {
+    for (uint32_t c0 = 0; c0 < num_chunks; c0 += 8 * team) {
+        u32x4 v[8];
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) {
+            const uint32_t c = c0 + u * team + member;
+            if (c < num_chunks) v[u] = __builtin_nontemporal_load(src + c);
+        }
+#pragma unroll
+        for (uint32_t u = 0; u < 8; ++u) {
+            const uint32_t c = c0 + u * team + member;
+            if (c < num_chunks) __builtin_nontemporal_store(v[u], dst + c);
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
-// dispatch recv, step 1: first received row of every (source, local expert)
-// run, in the order the reference's host worker visits them
-// (a2a_worker.rs:621-634,681-694).  One workgroup.
+// dispatch recv, one launch.  Every workgroup first lays out the receiver from
+// the published per-source counts of its experts (what the reference's host
+// worker does, a2a_worker.rs:577-606,621-694): rows per expert, padded first
+// row of every expert, first row of every (source, expert) run inside it, and
+// the order in which the runs ARRIVE (sources in the worker's order, experts
+// inside a source).  Workgroup 0 publishes those tables.  Then the workgroups
+// share the received rows between them, one team of wavefronts per row: its metadata (padded_index,
+// source_rank, source position: a2a_worker.rs:636-671) is written and payload
+// and scales are copied from the sender's staged token
+// (a2a_dispatch_recv.cu:139-155).
+//
+// Dynamic LDS: 4 * G * Le + 1 words.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void recv_segments_kernel(const StageRecvArgs args,
-                                                             const Workspace ws, const Staging st) {
-    __shared__ uint32_t wave_tot[16];
-    __shared__ uint32_t carry_s;
+__global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs args, const Workspace ws,
+                                                          const Staging st) {
+    extern __shared__ uint32_t s_recv[];
+    __shared__ uint32_t scratch[kRouteWaves];
+    __shared__ uint32_t s_carry;
     const uint32_t G = ws.num_groups, E = ws.num_experts, Le = ws.experts_per_rank;
     const uint32_t r = args.rank;
     const uint32_t first = r * Le;
     const uint32_t n_local = first >= E ? 0 : (E - first < Le ? E - first : Le);
-    const uint32_t num_seg = G * Le;
-    uint32_t *seg = st.seg_start + (size_t)r * (ws.world * Le + 1);
-    const uint32_t tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
-    const uint32_t remote_segs = (ws.world / ws.node_size - 1) * (ws.node_size / ws.dp_size) * Le;
+    const uint32_t items = G * Le;
+    const uint32_t tid = threadIdx.x;
+    const bool publish = blockIdx.x == 0;
+    uint32_t *tot = s_recv;              // [g][le]  copies source g sends to local expert le
+    uint32_t *excl = tot + items;        // [g][le]  position of the run in the sender's expert-sorted order
+    uint32_t *run_row = excl + items;    // [i][le]  first row of the run in the receiver's buffer (i = order index)
+    uint32_t *seg = run_row + items;     // [i][le]  first ARRIVAL index of the run; seg[items] = rows received
 
-    if (tid == 0) carry_s = 0;
-    __syncthreads();
-    for (uint32_t base = 0; base < num_seg; base += blockDim.x) {
-        const uint32_t s = base + tid;
-        uint32_t cnt = 0;
-        if (s < num_seg) {
-            const uint32_t g = source_order_lookup(ws.order, r, s / Le);
-            const uint32_t le = s % Le;
-            if (le < n_local && (args.valid_mask >> g & 1)) cnt = ws.num_routed[g * E + first + le];
-        }
-        // block-wide exclusive scan of cnt
-        uint32_t incl = cnt;
-#pragma unroll
-        for (int d = 1; d < kWave; d <<= 1) {
-            const uint32_t up = __shfl_up(incl, d);
-            if (lane >= (uint32_t)d) incl += up;
-        }
-        if (lane == kWave - 1) wave_tot[wave] = incl;
-        __syncthreads();
-        uint32_t before = carry_s;
-        for (uint32_t w = 0; w < wave; ++w) before += wave_tot[w];
-        if (s < num_seg) seg[s] = before + incl - cnt;
-        __syncthreads();
-        if (tid == blockDim.x - 1) carry_s = before + incl;
-        __syncthreads();
+    for (uint32_t w = tid; w < items; w += blockDim.x) {
+        const uint32_t g = Le > 1 ? __umulhi(w, ws.le_magic) : w;
+        const uint32_t le = w - g * Le;
+        const uint32_t e = first + le;
+        const bool live = le < n_local && (args.valid_mask >> g & 1);
+        tot[w] = live ? ws.num_routed[g * E + e] : 0;
+        excl[w] = live && e > 0 ? ws.expert_offsets[g * E + e - 1] : 0;
     }
-    if (tid == 0) {
-        const uint32_t total = carry_s;
-        seg[num_seg] = total;
+    __syncthreads();
+
+    // Rows per expert, padded offsets, first row of every run.
+    const uint32_t pad = ws.expert_padding;
+    uint32_t carry = 0;
+    for (uint32_t l0 = 0; l0 < Le; l0 += blockDim.x) {
+        const uint32_t le = l0 + tid;
+        const bool mine = le < n_local;
+        uint32_t tpe = 0;
+        if (mine) {
+            for (uint32_t g = 0; g < G; ++g) tpe += tot[g * Le + le];
+        }
+        const uint32_t padded = (tpe + pad - 1) / pad * pad;
+        const uint32_t incl = carry + block_inclusive_scan(mine ? padded : 0, scratch);
+        if (mine) {
+            const uint32_t poff = incl - padded;
+            const uint32_t e = first + le;
+            uint32_t running = poff;
+            for (uint32_t i = 0; i < G; ++i) {
+                const uint32_t g = source_order_lookup(ws.order, r, i);
+                run_row[i * Le + le] = running;
+                if (publish) ws.slot_base[g * E + e] = running;
+                running += tot[g * Le + le];
+            }
+            if (publish) {
+                ws.tokens_per_expert[e] = tpe;
+                ws.padded_offset[e] = poff;
+                if (args.out_num_tokens != nullptr) args.out_num_tokens[le] = (int32_t)tpe;
+                if (poff + tpe > args.dst.out_rows) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+            }
+        }
+        if (l0 + blockDim.x < Le) {   // uniform: another round follows
+            if (tid == blockDim.x - 1) s_carry = incl;
+            __syncthreads();
+            carry = s_carry;
+        }
+    }
+
+    // Arrival order: sources as the worker visits them, local experts inside a source.
+    carry = 0;
+    for (uint32_t b = 0; b < items; b += blockDim.x) {
+        const uint32_t s = b + tid;
+        uint32_t cnt = 0;
+        if (s < items) {
+            const uint32_t i = Le > 1 ? __umulhi(s, ws.le_magic) : s;
+            cnt = tot[source_order_lookup(ws.order, r, i) * Le + (s - i * Le)];
+        }
+        const uint32_t incl = carry + block_inclusive_scan(cnt, scratch);
+        if (s < items) seg[s] = incl - cnt;
+        if (tid == blockDim.x - 1) s_carry = incl;
+        __syncthreads();
+        carry = s_carry;
+    }
+    const uint32_t total = carry;
+    if (tid == 0) seg[items] = total;
+    __syncthreads();
+    if (publish && tid == 0) {
         st.num_recv[2 * r] = total;
         // rows that come from other nodes (num_efa_tokens, a2a_worker.rs:681-687)
-        st.num_recv[2 * r + 1] = remote_segs < num_seg ? seg[remote_segs] : total;
+        const uint32_t remote_segs = (ws.world / ws.node_size - 1) * (ws.node_size / ws.dp_size) * Le;
+        st.num_recv[2 * r + 1] = remote_segs < items ? seg[remote_segs] : total;
     }
-}
 
-// Locate received row `i` of receiver `r`: its run (source, local expert) and
-// its index inside the run.  Binary search over seg_start (ascending).
-__device__ __forceinline__ void locate_row(const uint32_t *seg, uint32_t num_seg, uint32_t i,
-                                           uint32_t *seg_out, uint32_t *j_out) {
-    uint32_t lo = 0, hi = num_seg;  // seg[lo] <= i < seg[hi]
-    while (hi - lo > 1) {
-        const uint32_t mid = (lo + hi) / 2;
-        if (seg[mid] <= i) lo = mid; else hi = mid;
-    }
-    *seg_out = lo;
-    *j_out = i - seg[lo];
-}
-
-// ---------------------------------------------------------------------------
-// dispatch recv, step 2: one workgroup per received row.  Writes the row's
-// metadata (padded_index, source_rank, source position: a2a_worker.rs:636-671)
-// and copies payload and scales from the sender's staged token
-// (a2a_dispatch_recv.cu:139-155).
-// ---------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs args, const Workspace ws,
-                                                          const Staging st) {
-    const uint32_t E = ws.num_experts, Le = ws.experts_per_rank;
-    const uint32_t r = args.rank;
-    const uint32_t num_seg = ws.num_groups * Le;
-    const uint32_t *seg = st.seg_start + (size_t)r * (ws.world * Le + 1);
-    const uint32_t i = blockIdx.x;
-    if (i >= seg[num_seg]) return;
-    uint32_t s, j;
-    locate_row(seg, num_seg, i, &s, &j);
-    const uint32_t g = source_order_lookup(ws.order, r, s / Le);
-    const uint32_t e = r * Le + s % Le;
-    const uint32_t excl = e > 0 ? ws.expert_offsets[g * E + e - 1] : 0;
-    const uint32_t pos = excl + j;
-    const uint32_t dst_row = ws.slot_base[g * E + e] + j;
-    const uint32_t tid = threadIdx.x;
-    if (tid == 0 && i < st.max_recv) {
-        st.padded_index[(size_t)r * st.max_recv + i] = dst_row;
-        // the member of the group that sends to this rank (a2a_worker.rs:633)
-        st.source_rank[(size_t)r * st.max_recv + i] = g * ws.dp_size + r % ws.dp_size;
-        st.source_position[(size_t)r * st.max_recv + i] = pos;
-    }
+    // From here on the workgroup is split into teams of args.team_waves
+    // wavefronts that work alone (no barrier): one received row per team at a
+    // time.  Every wavefront of a team finds the row's run by itself.
     const PushDst &dst = args.dst;
-    if (dst.out_x == nullptr) return;
-    if (dst_row >= dst.out_rows) {
-        if (tid == 0) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
-        return;
-    }
-    const uint32_t token = st.pos_token[(size_t)g * ws.max_tk + pos];
-    const uint8_t *src = st.send_buf + ((size_t)g * st.max_tokens + token) * st.disp_stride;
-    uint8_t *out = dst.out_x + (size_t)dst_row * dst.out_stride;
     const uint32_t num_chunks = args.row_bytes / 16;
-    for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
-        __builtin_nontemporal_store(reinterpret_cast<const u32x4 *>(src)[c],
-                                    reinterpret_cast<u32x4 *>(out) + c);
-    }
-    if (dst.out_scale != nullptr) {
-        const float *ss = reinterpret_cast<const float *>(src + st.payload_bytes);
-        float *os = dst.out_scale + (size_t)dst_row * dst.os_stride_token;
-        for (uint32_t q = tid; q < args.hidden_dim_scale; q += blockDim.x) {
-            os[(size_t)q * dst.os_stride_elem] = ss[q];
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t team = args.team_waves * kWave;
+    const uint32_t teams = blockDim.x / team;
+    const uint32_t member = tid % team;
+    for (uint32_t row = blockIdx.x * teams + tid / team; row < total; row += gridDim.x * teams) {
+        // the run this arrival belongs to: the one non-empty run with seg[s] <= row < seg[s + 1]
+        uint32_t s = 0;
+        for (uint32_t s0 = 0; s0 < items; s0 += kWave) {
+            const uint32_t cand = s0 + lane;
+            const uint64_t hit = __ballot(cand < items && seg[cand] <= row && row < seg[cand + 1]);
+            if (hit != 0) {
+                s = s0 + (uint32_t)__builtin_ctzll(hit);
+                break;
+            }
+        }
+        const uint32_t i = Le > 1 ? __umulhi(s, ws.le_magic) : s;
+        const uint32_t le = s - i * Le;
+        const uint32_t g = source_order_lookup(ws.order, r, i);
+        const uint32_t j = row - seg[s];
+        const uint32_t pos = excl[g * Le + le] + j;
+        const uint32_t dst_row = run_row[s] + j;
+        if (member == 0 && row < st.max_recv) {
+            st.padded_index[(size_t)r * st.max_recv + row] = dst_row;
+            // the member of the group that sends to this rank (a2a_worker.rs:633)
+            st.source_rank[(size_t)r * st.max_recv + row] = g * ws.dp_size + r % ws.dp_size;
+            st.source_position[(size_t)r * st.max_recv + row] = pos;
+        }
+        if (dst.out_x == nullptr) continue;
+        if (dst_row >= dst.out_rows) {
+            if (member == 0) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+            continue;
+        }
+        const uint32_t token = st.pos_token[(size_t)g * ws.max_tk + pos];
+        const uint8_t *src = st.send_buf + ((size_t)g * st.max_tokens + token) * st.disp_stride;
+        copy_row_by_team(reinterpret_cast<const u32x4 *>(src),
+                         reinterpret_cast<u32x4 *>(dst.out_x + (size_t)dst_row * dst.out_stride), num_chunks, member,
+                         team);
+        if (dst.out_scale != nullptr) {
+            const float *ss = reinterpret_cast<const float *>(src + st.payload_bytes);
+            float *os = dst.out_scale + (size_t)dst_row * dst.os_stride_token;
+            for (uint32_t q = member; q < args.hidden_dim_scale; q += team) {
+                os[(size_t)q * dst.os_stride_elem] = ss[q];
+            }
         }
     }
 }
@@ -204,21 +262,24 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
 __global__ __launch_bounds__(1024) void combine_send_kernel(const CombineSendArgs args,
                                                             const Workspace ws, const Staging st) {
     const uint32_t r = args.rank;
-    const uint32_t i = blockIdx.x;
-    if (i >= st.num_recv[2 * r] || i >= st.max_recv) return;
-    const uint32_t row = st.padded_index[(size_t)r * st.max_recv + i];
-    // every member of the source's dp group reads the same staging rows
-    const uint32_t g = st.source_rank[(size_t)r * st.max_recv + i] / ws.dp_size;
-    const uint32_t pos = st.source_position[(size_t)r * st.max_recv + i];
-    if (row >= args.y_rows || pos >= ws.max_tk) {
-        if (threadIdx.x == 0) atomicOr(ws.err, A2A_DEV_BAD_SLOT);
-        return;
-    }
-    const u32x4 *src = reinterpret_cast<const u32x4 *>(args.y + (size_t)row * args.y_stride);
-    u32x4 *dst = reinterpret_cast<u32x4 *>(st.comb_buf + ((size_t)g * ws.max_tk + pos) * st.comb_stride);
+    uint32_t total = st.num_recv[2 * r];
+    if (total > st.max_recv) total = st.max_recv;
     const uint32_t num_chunks = args.row_bytes / 16;
-    for (uint32_t c = threadIdx.x; c < num_chunks; c += blockDim.x) {
-        dst[c] = __builtin_nontemporal_load(src + c);
+    const uint32_t team = args.team_waves * kWave;   // threads that share a row
+    const uint32_t teams = blockDim.x / team;
+    const uint32_t member = threadIdx.x % team;
+    for (uint32_t i = blockIdx.x * teams + threadIdx.x / team; i < total; i += gridDim.x * teams) {
+        const uint32_t row = st.padded_index[(size_t)r * st.max_recv + i];
+        // every member of the source's dp group reads the same staging rows
+        const uint32_t g = st.source_rank[(size_t)r * st.max_recv + i] / ws.dp_size;
+        const uint32_t pos = st.source_position[(size_t)r * st.max_recv + i];
+        if (row >= args.y_rows || pos >= ws.max_tk) {
+            if (member == 0) atomicOr(ws.err, A2A_DEV_BAD_SLOT);
+            continue;
+        }
+        copy_row_by_team(reinterpret_cast<const u32x4 *>(args.y + (size_t)row * args.y_stride),
+                         reinterpret_cast<u32x4 *>(st.comb_buf + ((size_t)g * ws.max_tk + pos) * st.comb_stride),
+                         num_chunks, member, team);
     }
 }
 
@@ -229,6 +290,37 @@ uint32_t block_for_chunks(uint32_t chunks) {
     return threads;
 }
 
+// How the rows of a receiver are shared out.  Few rows (decode): one workgroup
+// per row, as wide as the row needs, because then the latency of a row is what
+// counts.  Many rows: teams of one wavefront, four to a workgroup, each with
+// eight pieces per lane in flight, in workgroups that stride over the rows,
+// because then memory-level parallelism is what counts (measured per receiver,
+// rows of 7 KB: 19 us against 24 us at 4096 rows, 13 against 16 us at 1024).
+constexpr uint32_t kMaxRowWorkgroups = 2048;
+constexpr uint32_t kManyRows = 2048;
+constexpr uint32_t kFewRowWorkgroups = 512;
+
+struct RowLaunch {
+    uint32_t blocks, threads, team_waves;
+};
+
+RowLaunch row_launch(uint32_t max_rows, uint32_t chunks) {
+    // max_rows is the host's upper bound; a receiver typically gets 1/N of it, and
+    // workgroups without a row still pay for the layout, so the grids stay modest.
+    RowLaunch l;
+    if (max_rows <= kManyRows) {
+        l.threads = block_for_chunks(chunks);
+        l.team_waves = l.threads / kWave;
+        l.blocks = max_rows < kFewRowWorkgroups ? max_rows : kFewRowWorkgroups;
+    } else {
+        l.threads = 4 * kWave;
+        l.team_waves = 1;
+        const uint32_t blocks = (max_rows + 3) / 4;
+        l.blocks = blocks < kMaxRowWorkgroups ? blocks : kMaxRowWorkgroups;
+    }
+    return l;
+}
+
 }  // namespace
 
 int staging_allocate(Staging &st, const a2a_config &cfg, std::string *error) {
@@ -236,7 +328,6 @@ int staging_allocate(Staging &st, const a2a_config &cfg, std::string *error) {
     const size_t N = cfg.world_size;
     const size_t K = cfg.num_experts_per_token;
     const size_t max_tk = (size_t)cfg.max_num_tokens * K;
-    const size_t Le = (cfg.num_experts + N - 1) / N;
     st.disp_stride = a2a_dispatch_token_stride(&cfg);
     st.comb_stride = a2a_combine_token_stride(&cfg);
     st.payload_bytes = (uint32_t)align_up_sz((size_t)cfg.hidden_dim * cfg.in_elemsize, 16);
@@ -258,7 +349,6 @@ int staging_allocate(Staging &st, const a2a_config &cfg, std::string *error) {
     const size_t o_send = carve(N * cfg.max_num_tokens * st.disp_stride);
     const size_t o_pos = carve(N * max_tk * sizeof(uint32_t));
     const size_t o_comb = carve(N * max_tk * st.comb_stride);
-    const size_t o_seg = carve(N * (N * Le + 1) * sizeof(uint32_t));
     const size_t o_pidx = carve(N * max_recv * sizeof(uint32_t));
     const size_t o_srank = carve(N * max_recv * sizeof(uint32_t));
     const size_t o_spos = carve(N * max_recv * sizeof(uint32_t));
@@ -275,14 +365,13 @@ int staging_allocate(Staging &st, const a2a_config &cfg, std::string *error) {
     st.send_buf = base + o_send;
     st.pos_token = reinterpret_cast<uint32_t *>(base + o_pos);
     st.comb_buf = base + o_comb;
-    st.seg_start = reinterpret_cast<uint32_t *>(base + o_seg);
     st.padded_index = reinterpret_cast<uint32_t *>(base + o_pidx);
     st.source_rank = reinterpret_cast<uint32_t *>(base + o_srank);
     st.source_position = reinterpret_cast<uint32_t *>(base + o_spos);
     st.num_recv = reinterpret_cast<uint32_t *>(base + o_nrecv);
     // Tables are read before they are written only through misuse; start from zero.
     e = hipMemset(base + o_pos, 0, o_comb - o_pos);
-    if (e == hipSuccess) e = hipMemset(base + o_seg, 0, off - o_seg);
+    if (e == hipSuccess) e = hipMemset(base + o_pidx, 0, off - o_pidx);
     if (e == hipSuccess) e = hipDeviceSynchronize();
     if (e != hipSuccess) {
         if (error) *error = std::string("hipMemset(staging): ") + hipGetErrorString(e);
@@ -337,21 +426,22 @@ hipError_t launch_stage_send(const StageSendArgs &args, const Workspace &ws, con
 
 hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st,
                              hipStream_t stream) {
-    uint32_t seg_threads = (ws.num_groups * ws.experts_per_rank + kWave - 1) / kWave * kWave;
-    if (seg_threads > 1024) seg_threads = 1024;
-    hipLaunchKernelGGL(recv_segments_kernel, dim3(1), dim3(seg_threads), 0, stream, args, ws, st);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess || args.max_rows == 0) return e;
-    hipLaunchKernelGGL(stage_recv_kernel, dim3(args.max_rows), dim3(block_for_chunks(args.row_bytes / 16)),
-                       0, stream, args, ws, st);
+    RowLaunch l = row_launch(args.max_rows, args.row_bytes / 16);
+    if (l.blocks == 0) l.blocks = 1;    // the layout is published even when nothing was sent
+    StageRecvArgs a = args;
+    a.team_waves = l.team_waves;
+    const size_t lds = (4 * (size_t)ws.num_groups * ws.experts_per_rank + 1) * sizeof(uint32_t);
+    hipLaunchKernelGGL(stage_recv_kernel, dim3(l.blocks), dim3(l.threads), lds, stream, a, ws, st);
     return hipGetLastError();
 }
 
 hipError_t launch_combine_send(const CombineSendArgs &args, const Workspace &ws, const Staging &st,
                                hipStream_t stream) {
     if (args.max_rows == 0) return hipSuccess;
-    hipLaunchKernelGGL(combine_send_kernel, dim3(args.max_rows),
-                       dim3(block_for_chunks(args.row_bytes / 16)), 0, stream, args, ws, st);
+    const RowLaunch l = row_launch(args.max_rows, args.row_bytes / 16);
+    CombineSendArgs a = args;
+    a.team_waves = l.team_waves;
+    hipLaunchKernelGGL(combine_send_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, a, ws, st);
     return hipGetLastError();
 }
 
