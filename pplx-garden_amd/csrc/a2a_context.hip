@@ -624,31 +624,9 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     const uint32_t K = c.num_experts_per_token;
     const uint32_t T = (uint32_t)num_tokens;
 
-    RouteArgs ra;
-    FinalizeArgs fa;
-    memset(&ra, 0, sizeof ra);
-    memset(&fa, 0, sizeof fa);
-    const uint32_t nb = ceil_div_u32((uint64_t)T * K, kRouteBlock);
     // The sender is the rank's dp group; when several members of a group send, each repeats
     // the same routing and stages the same rows.
     const uint32_t group = rank / c.dp_size;
-    ra.src[group] = RouteSrc{indices, bound_m, (uint32_t)indices_stride, T};
-    for (uint32_t r = 0; r <= (uint32_t)kMaxWorld; ++r) ra.block_start[r] = r <= group ? 0 : nb;
-    fa.num_blocks[group] = nb;
-    fa.fold_mask = 1u << group;
-    fa.valid_mask = ctx->sent_mask | (1u << group);
-    fa.recv_mask = 0;
-    hipError_t e;
-    if (fused_routing_pays(fa, c.world_size / c.dp_size, nb)) {
-        e = launch_route_fused(ra, fa, ctx->ws, s);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
-    } else {
-        e = launch_route(ra, ctx->ws, nb, s);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
-        e = launch_finalize(fa, ctx->ws, s);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
-    }
-
     StageSendArgs sa;
     memset(&sa, 0, sizeof sa);
     sa.rank = rank;
@@ -664,8 +642,36 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     sa.row_bytes = (uint32_t)row_bytes_of(c);
     sa.hidden_dim = c.hidden_dim;
     sa.hidden_dim_scale = c.hidden_dim_scale;
-    e = launch_stage_send(sa, ctx->ws, ctx->staging, quantize != 0, s);
-    if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send");
+    sa.topk_magic = K > 1 ? (uint32_t)((0x100000000ull + K - 1) / K) : 0;
+
+    hipError_t e;
+    if (stage_send_small_fits(sa, ctx->ws)) {
+        e = launch_stage_send_small(sa, ctx->ws, ctx->staging, quantize != 0, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send_small");
+    } else {
+        RouteArgs ra;
+        FinalizeArgs fa;
+        memset(&ra, 0, sizeof ra);
+        memset(&fa, 0, sizeof fa);
+        const uint32_t nb = ceil_div_u32((uint64_t)T * K, kRouteBlock);
+        ra.src[group] = RouteSrc{indices, bound_m, (uint32_t)indices_stride, T};
+        for (uint32_t r = 0; r <= (uint32_t)kMaxWorld; ++r) ra.block_start[r] = r <= group ? 0 : nb;
+        fa.num_blocks[group] = nb;
+        fa.fold_mask = 1u << group;
+        fa.valid_mask = ctx->sent_mask | (1u << group);
+        fa.recv_mask = 0;
+        if (fused_routing_pays(fa, c.world_size / c.dp_size, nb)) {
+            e = launch_route_fused(ra, fa, ctx->ws, s);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
+        } else {
+            e = launch_route(ra, ctx->ws, nb, s);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
+            e = launch_finalize(fa, ctx->ws, s);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+        }
+        e = launch_stage_send(sa, ctx->ws, ctx->staging, quantize != 0, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send");
+    }
 
     ctx->sent_mask |= 1u << group;
     ctx->num_tokens[group] = T;

@@ -44,6 +44,7 @@ struct StageSendArgs {
     uint32_t row_bytes;
     uint32_t hidden_dim;
     uint32_t hidden_dim_scale;
+    uint32_t topk_magic;      // ceil(2^32 / K) (0 for K = 1), for entry -> token without a division
 };
 
 struct StageRecvArgs {
@@ -82,6 +83,10 @@ const uint32_t *staging_table(const Staging &st, const a2a_config &cfg, uint32_t
 
 hipError_t launch_stage_send(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                              bool quantize, hipStream_t stream);
+// One-launch send (routing counted inside) for small steps: whether a step qualifies, and the launch.
+bool stage_send_small_fits(const StageSendArgs &args, const Workspace &ws);
+hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &ws, const Staging &st,
+                                   bool quantize, hipStream_t stream);
 hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st,
                              hipStream_t stream);
 hipError_t launch_combine_send(const CombineSendArgs &args, const Workspace &ws, const Staging &st,

@@ -16,6 +16,57 @@ size_t align_up_sz(size_t n, size_t a) { return (n + a - 1) / a * a; }
 // dispatch send: stage one (quantised) row per token, record which token sits
 // behind every row of the sender's expert-sorted order.
 // ---------------------------------------------------------------------------
+
+// Stages the row of `token` (payload, then scales).  With PRELOADED the chunk of
+// this thread's first iteration is already in `pre_a` / `pre_b`.  Whole workgroup.
+template <bool QUANT, bool PRELOADED>
+__device__ __forceinline__ void stage_row(const StageSendArgs &args, const Staging &st, uint32_t g, uint32_t token,
+                                          u32x4 pre_a, u32x4 pre_b) {
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const PushSrc &src = args.src;
+    const uint8_t *x_row = src.x + (size_t)token * src.x_stride;
+    uint8_t *row = st.send_buf + ((size_t)g * st.max_tokens + token) * st.disp_stride;
+    float *row_scale = reinterpret_cast<float *>(row + st.payload_bytes);
+
+    if constexpr (QUANT) {
+        const uint32_t num_chunks = args.hidden_dim / 16;
+        for (uint32_t base = wave * kWave; base < num_chunks; base += blockDim.x) {
+            const uint32_t c = base + lane;
+            const bool active = c < num_chunks;
+            u32x4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
+            if (PRELOADED && base == wave * kWave) {
+                a = pre_a;
+                b = pre_b;
+            } else if (active) {
+                const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)c * 32);
+                a = __builtin_nontemporal_load(p);
+                b = __builtin_nontemporal_load(p + 1);
+            }
+            float scale;
+            const u32x4 q = quantize16(a, b, &scale);
+            if (active) {
+                reinterpret_cast<u32x4 *>(row)[c] = q;
+                if ((lane & 7) == 0) row_scale[c / 8] = scale;
+            }
+        }
+    } else {
+        const uint32_t num_chunks = args.row_bytes / 16;
+        for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
+            reinterpret_cast<u32x4 *>(row)[c] =
+                PRELOADED && c == tid ? pre_a
+                                      : __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
+        }
+        if (src.x_scale != nullptr) {
+            const float *xs = src.x_scale + (size_t)token * src.xs_stride_token;
+            for (uint32_t j = tid; j < args.hidden_dim_scale; j += blockDim.x) {
+                row_scale[j] = xs[(size_t)j * src.xs_stride_elem];
+            }
+        }
+    }
+}
+
 template <bool QUANT>
 __global__ __launch_bounds__(1024) void stage_send_kernel(const StageSendArgs args, const Workspace ws,
                                                           const Staging st) {
@@ -42,42 +93,123 @@ __global__ __launch_bounds__(1024) void stage_send_kernel(const StageSendArgs ar
         }
         ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
     }
+    const u32x4 none = {0, 0, 0, 0};
+    stage_row<QUANT, false>(args, st, g, token, none, none);
+}
 
-    const uint8_t *x_row = src.x + (size_t)token * src.x_stride;
-    uint8_t *row = st.send_buf + ((size_t)g * st.max_tokens + token) * st.disp_stride;
-    float *row_scale = reinterpret_cast<float *>(row + st.payload_bytes);
+// The send of a small step in ONE launch (the reference's dispatch-send kernel
+// is one launch too, a2a_dispatch_send.cu:158-523): every token workgroup asks
+// for its row, counts the entries of the sender per expert and those before its
+// own token (LDS atomics; counts do not depend on arrival order), scans the
+// counts over the experts, and has the position of each of its K copies in the
+// sender's expert-sorted order.  The workgroup of token 0 publishes the counts
+// and their scan.  Cost grows with tokens x entries, so the host uses it for
+// small steps only.  Dynamic LDS: 3 * E words.
+template <bool QUANT>
+__global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendArgs args, const Workspace ws,
+                                                                const Staging st) {
+    extern __shared__ uint32_t s_send[];
+    __shared__ uint32_t scratch[kRouteWaves];
+    __shared__ uint32_t s_carry;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const uint32_t E = ws.num_experts;
+    const uint32_t K = ws.topk;
+    const uint32_t g = args.rank / ws.dp_size;
+    const uint32_t token = blockIdx.x;
+    const PushSrc &src = args.src;
+    const uint32_t eff = effective_tokens(src.bound_m, src.num_tokens);
+    const uint32_t entries = eff * K;
+    const uint32_t my_first = token * K;
+    uint32_t *cnt = s_send;          // [E] entries of the sender per expert
+    uint32_t *prior = cnt + E;       // [E] those of the tokens before mine
+    uint32_t *excl = prior + E;      // [E] exclusive scan of cnt
 
-    if constexpr (QUANT) {
-        const uint32_t num_chunks = args.hidden_dim / 16;
-        for (uint32_t base = wave * kWave; base < num_chunks; base += blockDim.x) {
-            const uint32_t c = base + lane;
-            const bool active = c < num_chunks;
-            u32x4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
-            if (active) {
-                const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)c * 32);
-                a = __builtin_nontemporal_load(p);
-                b = __builtin_nontemporal_load(p + 1);
-            }
-            float scale;
-            const u32x4 q = quantize16(a, b, &scale);
-            if (active) {
-                reinterpret_cast<u32x4 *>(row)[c] = q;
-                if ((lane & 7) == 0) row_scale[c / 8] = scale;
+    for (uint32_t i = tid; i < 2 * E; i += blockDim.x) s_send[i] = 0;
+    __syncthreads();
+
+    uint32_t my_expert = 0xFFFFFFFFu;
+    u32x4 pre_a = {0, 0, 0, 0}, pre_b = {0, 0, 0, 0};
+    for (uint32_t f0 = 0; f0 < entries || f0 == 0; f0 += 8 * blockDim.x) {
+        uint32_t expert[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            const uint32_t f = f0 + j * blockDim.x + tid;
+            expert[j] = 0xFFFFFFFFu;
+            if (f < entries) {
+                const uint32_t t = K > 1 ? __umulhi(f, args.topk_magic) : f;
+                expert[j] = (uint32_t)src.indices[(size_t)t * src.indices_stride + (f - t * K)];
             }
         }
-    } else {
-        const uint32_t num_chunks = args.row_bytes / 16;
-        for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
-            reinterpret_cast<u32x4 *>(row)[c] =
-                __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
-        }
-        if (src.x_scale != nullptr) {
-            const float *xs = src.x_scale + (size_t)token * src.xs_stride_token;
-            for (uint32_t j = tid; j < args.hidden_dim_scale; j += blockDim.x) {
-                row_scale[j] = xs[(size_t)j * src.xs_stride_elem];
+        if (f0 == 0) {
+            // the token's own ids and row, asked for after the first batch of the count
+            if (lane < K) my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
+            const uint8_t *x_row = src.x + (size_t)token * src.x_stride;
+            if constexpr (QUANT) {
+                if (tid < args.hidden_dim / 16) {
+                    const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)tid * 32);
+                    pre_a = __builtin_nontemporal_load(p);
+                    pre_b = __builtin_nontemporal_load(p + 1);
+                }
+            } else {
+                if (tid < args.row_bytes / 16) {
+                    pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + tid);
+                }
             }
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < 8; ++j) {
+            const uint32_t x = expert[j];
+            if (x >= E) continue;
+            atomicAdd(&cnt[x], 1u);
+            if (f0 + j * blockDim.x + tid < my_first) atomicAdd(&prior[x], 1u);
         }
     }
+    __syncthreads();
+
+    // Scan over the experts (a2a_dispatch_send.cu:236-242); token 0 publishes.
+    uint32_t carry = 0;
+    for (uint32_t e0 = 0; e0 < E; e0 += blockDim.x) {
+        const uint32_t e = e0 + tid;
+        const uint32_t c = e < E ? cnt[e] : 0;
+        const uint32_t incl = carry + block_inclusive_scan(c, scratch);
+        if (e < E) {
+            excl[e] = incl - c;
+            if (token == 0) {
+                ws.num_routed[g * E + e] = c;
+                ws.expert_offsets[g * E + e] = incl;
+            }
+        }
+        if (e0 + blockDim.x < E) {   // uniform: another round follows
+            if (tid == blockDim.x - 1) s_carry = incl;
+            __syncthreads();
+            carry = s_carry;
+        }
+    }
+    __syncthreads();
+    if (token >= eff) return;   // past bound_m: nothing to stage (uniform)
+
+    if (wave == 0) {
+        uint32_t repeats = 0;   // copies of this token to the same expert at an earlier k
+        for (uint32_t k = 0; k + 1 < K; ++k) {
+            const uint32_t other = (uint32_t)__builtin_amdgcn_readlane((int)my_expert, (int)k);
+            if (k < lane && other == my_expert) ++repeats;
+        }
+        if (lane < K) {
+            const uint32_t entry = token * K + lane;
+            uint32_t toff = 0;
+            if (my_expert < E) {
+                toff = prior[my_expert] + repeats;
+                // position of the copy (a2a_dispatch_send.cu:54)
+                st.pos_token[(size_t)g * ws.max_tk + excl[my_expert] + toff] = token;
+            } else {
+                atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
+            }
+            ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
+        }
+    }
+    stage_row<QUANT, true>(args, st, g, token, pre_a, pre_b);
 }
 
 // A team of `team` threads (one or more whole wavefronts) copies a row of
@@ -419,6 +551,26 @@ hipError_t launch_stage_send(const StageSendArgs &args, const Workspace &ws, con
                            args, ws, st);
     } else {
         hipLaunchKernelGGL(stage_send_kernel<false>, dim3(args.src.num_tokens), dim3(threads), 0, stream,
+                           args, ws, st);
+    }
+    return hipGetLastError();
+}
+
+bool stage_send_small_fits(const StageSendArgs &args, const Workspace &ws) {
+    const uint64_t T = args.src.num_tokens;
+    const uint64_t entries = T * ws.topk;
+    return T != 0 && entries <= A2A_SMALL_MAX_ENTRIES && entries * T <= A2A_SMALL_MAX_VISITS;
+}
+
+hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &ws, const Staging &st,
+                                   bool quantize, hipStream_t stream) {
+    const uint32_t threads = block_for_chunks(quantize ? args.hidden_dim / 16 : args.row_bytes / 16);
+    const size_t lds = 3 * (size_t)ws.num_experts * sizeof(uint32_t);
+    if (quantize) {
+        hipLaunchKernelGGL(stage_send_small_kernel<true>, dim3(args.src.num_tokens), dim3(threads), lds, stream,
+                           args, ws, st);
+    } else {
+        hipLaunchKernelGGL(stage_send_small_kernel<false>, dim3(args.src.num_tokens), dim3(threads), lds, stream,
                            args, ws, st);
     }
     return hipGetLastError();
