@@ -458,7 +458,7 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
     pa.topk_magic = K > 1 ? (uint32_t)((0x100000000ull + K - 1) / K) : 0;
 
     hipError_t e;
-    if (dispatch_small_fits(pa, ctx->ws, quantize != 0, tokens)) {
+    if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && dispatch_small_fits(pa, ctx->ws, quantize != 0, tokens)) {
         e = launch_dispatch_small(pa, fa, ctx->ws, quantize != 0, tokens, s);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_small");
     } else {
@@ -645,7 +645,7 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     sa.topk_magic = K > 1 ? (uint32_t)((0x100000000ull + K - 1) / K) : 0;
 
     hipError_t e;
-    if (stage_send_small_fits(sa, ctx->ws)) {
+    if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && stage_send_small_fits(sa, ctx->ws)) {
         e = launch_stage_send_small(sa, ctx->ws, ctx->staging, quantize != 0, s);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send_small");
     } else {

@@ -53,7 +53,7 @@ class LoopbackSubGroup:
 
 class LoopbackWorld:
     def __init__(self, world_size: int, node_size: Optional[int] = None,
-                 device: Optional[torch.device] = None) -> None:
+                 device: Optional[torch.device] = None, context_flags: int = 0) -> None:
         if world_size < 1:
             raise ValueError("world_size must be at least 1")
         node_size = world_size if node_size is None else node_size
@@ -62,6 +62,7 @@ class LoopbackWorld:
         self.size = world_size
         self.node_size = node_size
         self.device = device
+        self.context_flags = context_flags   # A2A_FLAG_* bits for the contexts created in this world
         self._contexts: Dict[Tuple, Any] = {}
         self._users: Dict[Tuple, int] = {}
         self._pending: Dict[Tuple[Tuple, str], Dict[int, Any]] = {}

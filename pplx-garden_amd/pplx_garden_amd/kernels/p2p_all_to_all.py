@@ -147,6 +147,7 @@ class P2PAllToAll(AllToAllKernel):
                 node_size=node_size,
                 world_size=world_size,
                 device=device_index,
+                flags=getattr(global_group.world, "context_flags", 0),
             )
 
         self._all_to_all = global_group.world.acquire_context(self._key, make_context)

@@ -44,6 +44,7 @@ DEV_RECV_OVERFLOW = 2
 DEV_BAD_SLOT = 4
 
 FLAG_PREALLOC_STAGING = 1
+FLAG_SEPARATE_ROUTING = 2   # never take the one-launch paths of small steps
 
 
 class A2AConfig(ctypes.Structure):

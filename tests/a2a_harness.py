@@ -65,11 +65,11 @@ def run_oracle(case: Case, world: Sequence[RankData], rows: int) -> WorldResult:
     return res
 
 
-def make_ops(case: Case, device: torch.device, max_num_tokens: Optional[int] = None):
+def make_ops(case: Case, device: torch.device, max_num_tokens: Optional[int] = None, context_flags: int = 0):
     from pplx_garden_amd.distributed.loopback import LoopbackWorld
     from pplx_garden_amd.kernels.p2p_all_to_all import P2PAllToAll
 
-    world = LoopbackWorld(case.world_size, node_size=case.node_size, device=device)
+    world = LoopbackWorld(case.world_size, node_size=case.node_size, device=device, context_flags=context_flags)
     ops = [
         P2PAllToAll(
             max_num_tokens=max_num_tokens or max(case.num_tokens, 1), num_experts=case.num_experts,
@@ -84,14 +84,14 @@ def make_ops(case: Case, device: torch.device, max_num_tokens: Optional[int] = N
 
 
 def run_gpu(case: Case, world_data: Sequence[RankData], rows: int, device: torch.device,
-            split: bool = False, expert_y_override=None) -> WorldResult:
+            split: bool = False, expert_y_override=None, context_flags: int = 0) -> WorldResult:
     """dispatch -> 2*dequant -> combine on the GPU through the operator API.
 
     split=False: every rank calls dispatch()/combine() with do_send and do_recv
     (the group calls of the library); split=True: all sends, then all recvs (the
     four split calls)."""
     N, H, Hs, Le = case.world_size, case.hidden_dim, case.hidden_dim_scale, case.experts_per_rank
-    _, ops = make_ops(case, device)
+    _, ops = make_ops(case, device, context_flags=context_flags)
     try:
         dev = [
             dict(x=rd.x.to(device), idx=rd.indices_u32.to(device), w=rd.weights.to(device))
