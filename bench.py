@@ -40,8 +40,9 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 
 # HBM bytes per launch on the default workload, from hardware counters (FETCH_SIZE and WRITE_SIZE
 # passes, scaled by what the same counters read for a 512 MiB copy: x2.000 and x1.000).  The counter
-# runs and their commands are summarised in profiles/hbm_traffic_dsv3_prefill_4096_push_and_combine.md.
-MEASURED_TRAFFIC_BYTES = {"combine_gather_kernel": 531_696_000, "dispatch_push_kernel": 303_073_000}
+# runs and their commands are summarised in profiles/hbm_traffic_dsv3_prefill_4096_pack_and_combine.md.
+MEASURED_TRAFFIC_BYTES = {"combine_gather_kernel": 531_696_000, "dispatch_resolve_kernel": 303_572_000,
+                          "dispatch_push_kernel": 303_073_000}
 
 
 def algorithmic_bytes(T: int, H: int, K: int):
@@ -56,7 +57,7 @@ def algorithmic_bytes(T: int, H: int, K: int):
 class Workload:
     """Buffers of one case with the GPU as rank 0 of N logical ranks."""
 
-    def __init__(self, case, device, num_routings: int):
+    def __init__(self, case, device, num_routings: int, context_flags: int = 0):
         import torch
         from a2a_cases import make_rank
         from a2a_harness import rows_needed
@@ -72,7 +73,7 @@ class Workload:
             out_dtype=torch.bfloat16, scale_elemsize=4, max_num_tokens=T, max_recv_tokens=T * K,
             max_private_tokens=0, num_experts=case.num_experts, expert_padding=case.expert_padding,
             num_experts_per_token=K, dp_size=1, node_size=case.node_size or N, world_size=N,
-            device=device.index or 0)
+            device=device.index or 0, flags=context_flags)
         self.routings = []
         rows = 1
         for i in range(num_routings):
@@ -194,6 +195,9 @@ def main() -> int:
     ap.add_argument("--no-decode", action="store_true", help="skip the 128-token shape")
     ap.add_argument("--decode-only", action="store_true",
                     help="time only the 128-token shape (for a kernel trace of the decode step alone)")
+    ap.add_argument("--separate-routing", action="store_true",
+                    help="create the context with A2A_FLAG_SEPARATE_ROUTING (routing kernels, then the pack): "
+                         "for comparisons with the default paths")
     ap.add_argument("--probe-copy", action="store_true",
                     help="also run plain device-to-device copies of 512 MiB (torch's copy kernel): the "
                          "known-size kernel that hardware byte counters are scaled by")
@@ -221,8 +225,9 @@ def main() -> int:
         torch.cuda.synchronize(device)
         del src, dst
 
+    ctx_flags = 2 if args.separate_routing else 0   # A2A_FLAG_SEPARATE_ROUTING
     if args.decode_only:
-        wl2 = Workload(C2, device, args.routings)
+        wl2 = Workload(C2, device, args.routings, ctx_flags)
         _, d2, c2, b2 = time_workload(wl2, args.steps, args.warmup)
         wl2.close()
         print(json.dumps({"decode_128_only": {"dispatch_us_p50": round(Statistics.create(d2).p50, 2),
@@ -231,7 +236,7 @@ def main() -> int:
         return 0
 
     case = C3
-    wl = Workload(case, device, args.routings)
+    wl = Workload(case, device, args.routings, ctx_flags)
     wall_s, disp, comb, both = time_workload(wl, args.steps, args.warmup)
     rows = wl.rows
     cpu_rd = wl.cpu_first
@@ -251,15 +256,20 @@ def main() -> int:
 
     combine_roof = roof(c_bytes, c_stats.mean, "combine_gather_kernel",
                         "events around a2a_combine, which is this one launch")
-    dispatch_roof = roof(d_bytes, d_stats.mean, "dispatch_push_kernel",
-                         "events around a2a_dispatch: route_hist + route_finalize + this kernel, so the "
-                         "kernel alone is faster than avg_us")
+    if args.separate_routing:
+        dispatch_roof = roof(d_bytes, d_stats.mean, "dispatch_push_kernel",
+                             "events around a2a_dispatch: route_hist + route_finalize + this kernel, so the "
+                             "kernel alone is faster than avg_us")
+    else:
+        dispatch_roof = roof(d_bytes, d_stats.mean, "dispatch_resolve_kernel",
+                             "events around a2a_dispatch: route_hist + this kernel, so the kernel alone is "
+                             "faster than avg_us")
     dominant, other = ((combine_roof, dispatch_roof) if c_stats.mean >= d_stats.mean
                        else (dispatch_roof, combine_roof))
 
     decode = None
     if not args.no_decode:
-        wl2 = Workload(C2, device, args.routings)
+        wl2 = Workload(C2, device, args.routings, ctx_flags)
         _, d2, c2, b2 = time_workload(wl2, max(args.steps, 200), args.warmup)
         wl2.close()
         decode = {

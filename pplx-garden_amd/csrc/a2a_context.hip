@@ -302,6 +302,10 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
     const size_t o_toff = carve((size_t)N * ws.max_tk * sizeof(uint32_t));
     const size_t o_err = carve(sizeof(uint32_t));
     const size_t o_order = carve((size_t)N * kMaxWorld);
+    const size_t o_before = carve((size_t)N * ws.num_groups * sizeof(uint32_t));
+    const size_t o_chunk_counts = carve((size_t)N * ws.nb_max * E * sizeof(uint32_t));
+    const size_t o_totals = carve(2 * ((size_t)ws.num_groups + 1) * E * sizeof(uint32_t));
+    const size_t o_turn = carve(2 * sizeof(uint32_t));
     ctx->arena_bytes = off;
     e = hipMalloc(&ctx->arena, ctx->arena_bytes);
     if (e != hipSuccess) {
@@ -328,15 +332,27 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
     ws.token_offset = reinterpret_cast<uint32_t *>(base + o_toff);
     ws.err = reinterpret_cast<uint32_t *>(base + o_err);
     ws.order = reinterpret_cast<const uint32_t *>(base + o_order);
+    ws.laid_before = reinterpret_cast<const uint32_t *>(base + o_before);
+    ws.chunk_counts = reinterpret_cast<uint32_t *>(base + o_chunk_counts);
+    ws.totals = reinterpret_cast<uint32_t *>(base + o_totals);
+    ws.turn = reinterpret_cast<uint32_t *>(base + o_turn);
     {
-        // i-th source each receiver lays out: fixed for the life of the context
+        // i-th source each receiver lays out, and which sources come before which: fixed for the
+        // life of the context
         uint8_t table[kMaxWorld * kMaxWorld] = {0};
+        uint32_t before[kMaxWorld * kMaxWorld] = {0};
         for (uint32_t r = 0; r < N; ++r) {
+            uint32_t seen = 0;
             for (uint32_t i = 0; i < ws.num_groups; ++i) {
-                table[r * kMaxWorld + i] = (uint8_t)source_order(r, i, N, config->node_size, config->dp_size);
+                const uint32_t g = source_order(r, i, N, config->node_size, config->dp_size);
+                table[r * kMaxWorld + i] = (uint8_t)g;
+                before[r * ws.num_groups + g] = seen;
+                seen |= 1u << g;
             }
         }
         e = hipMemcpy(base + o_order, table, (size_t)N * kMaxWorld, hipMemcpyHostToDevice);
+        if (e == hipSuccess)
+            e = hipMemcpy(base + o_before, before, (size_t)N * ws.num_groups * sizeof(uint32_t), hipMemcpyHostToDevice);
         if (e != hipSuccess) {
             (void)hipFree(ctx->arena);
             delete ctx;
@@ -461,7 +477,7 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
     if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && dispatch_small_fits(pa, ctx->ws, quantize != 0, tokens)) {
         e = launch_dispatch_small(pa, fa, ctx->ws, quantize != 0, tokens, s);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_small");
-    } else {
+    } else if (c.flags & A2A_FLAG_SEPARATE_ROUTING) {
         if (fused_routing_pays(fa, G, blocks)) {
             e = launch_route_fused(ra, fa, ctx->ws, s);
             if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
@@ -473,6 +489,13 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
         }
         e = launch_dispatch_push(pa, ctx->ws, quantize != 0, tokens, s);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_push");
+    } else {
+        // Two launches: chunk histograms that also add up the step's totals, then a pack whose
+        // workgroups resolve their own rows from them.
+        e = launch_route_accumulate(ra, ctx->ws, blocks, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist (accumulating)");
+        e = launch_dispatch_resolve(pa, fa, ctx->ws, quantize != 0, tokens, s);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_resolve");
     }
 
     ctx->group_routing = true;

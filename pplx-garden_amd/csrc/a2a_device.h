@@ -22,6 +22,19 @@ __device__ __forceinline__ float group8_max(float v) {
     return v;
 }
 
+// Sum over the aligned group of 8 lanes this lane belongs to (every lane gets it).
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_move_u32(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+
+__device__ __forceinline__ uint32_t group8_sum(uint32_t v) {
+    v += dpp_move_u32<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_move_u32<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_move_u32<0x141>(v);  // row_half_mirror
+    return v;
+}
+
 __device__ __forceinline__ uint64_t read_lane64(uint64_t v, uint32_t lane) {
     const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)v, (int)lane);
     const uint32_t hi = __builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), (int)lane);

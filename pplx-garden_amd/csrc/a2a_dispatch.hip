@@ -27,6 +27,9 @@ namespace {
 
 constexpr int kMaxLdsScales = 1024;
 
+// Arguments travel by value; a launch can carry 4 KB of them.
+static_assert(sizeof(PushArgs) + sizeof(FinalizeArgs) + sizeof(Workspace) <= 4096, "kernel arguments too large");
+
 // Moves the row of `token` to its copies.  Lanes 0..K-1 of EVERY wavefront hold
 // the row pointer, scale pointer and scale stride of route k (0 = no copy).
 // With PRELOADED, `pre_a`/`pre_b` already hold the chunk of this thread's first
@@ -110,24 +113,30 @@ __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &s
     }
 }
 
-// Where the copy of one route goes: row `slot` of the receiver described by `dst`.  Returns the slot that is recorded for the combine (kInvalidSlot if
-// the row does not fit the receiver's buffer).
+// Where the copy of one route goes: row `slot` of the receiver described by `dst`.
+// Returns the slot that is recorded for the combine (kInvalidSlot if the row
+// does not fit the receiver's buffer).  Written without branches on purpose:
+// the descriptor is read in one go and everything else is a select, so a lane
+// that resolves a route makes ONE trip to memory here, not one per condition
+// (under a saturated memory system every dependent trip costs microseconds).
 __device__ __forceinline__ uint32_t resolve_copy(const PushDst &dst, const Workspace &ws, uint32_t slot,
                                                  bool flag_overflow, uint64_t *row_ptr, uint64_t *scale_ptr,
                                                  uint32_t *scale_stride) {
-    if (dst.out_x != nullptr) {
-        if (slot < dst.out_rows) {
-            *row_ptr = (uint64_t)(dst.out_x + (size_t)slot * dst.out_stride);
-            if (dst.out_scale != nullptr) {
-                *scale_ptr = (uint64_t)(dst.out_scale + (size_t)slot * dst.os_stride_token);
-                *scale_stride = dst.os_stride_elem;
-            }
-        } else {
-            slot = kInvalidSlot;
-            if (flag_overflow) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
-        }
-    }
-    return slot;
+    const uint64_t out_x = (uint64_t)dst.out_x;
+    const uint64_t out_scale = (uint64_t)dst.out_scale;
+    const uint64_t out_stride = dst.out_stride;
+    const uint32_t os_elem = dst.os_stride_elem;
+    const uint32_t os_token = dst.os_stride_token;
+    const uint32_t out_rows = dst.out_rows;
+    const bool wanted = out_x != 0;
+    const bool fits = slot < out_rows;
+    const bool copy = wanted && fits;
+    const bool scales = copy && out_scale != 0;
+    *row_ptr = copy ? out_x + (uint64_t)slot * out_stride : 0;
+    *scale_ptr = scales ? out_scale + (uint64_t)slot * os_token * sizeof(float) : 0;
+    *scale_stride = scales ? os_elem : 0;
+    if (wanted && !fits && flag_overflow) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+    return wanted && !fits ? kInvalidSlot : slot;
 }
 
 uint32_t push_threads(const PushArgs &args, bool quantize) {
@@ -150,6 +159,9 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
     __shared__ float s_scale[QUANT ? kMaxLdsScales : 1];
     __shared__ uint64_t s_scale_ptr[A2A_MAX_EXPERTS_PER_TOKEN];
     __shared__ uint32_t s_scale_stride[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint64_t s_row_ptr[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint64_t s_route_scale_ptr[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint32_t s_route_scale_stride[A2A_MAX_EXPERTS_PER_TOKEN];
 
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
@@ -163,10 +175,11 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
     const PushSrc &src = args.src[g];
     if (token >= effective_tokens(src.bound_m, src.num_tokens)) return;
 
-    // Lanes 0..K-1 of every wavefront resolve one route each.
-    uint64_t row_ptr = 0, scale_ptr = 0;
-    uint32_t scale_stride = 0;
-    if (lane < K) {
+    // Lanes 0..K-1 of wavefront 0 resolve one route each and hand the result to
+    // the other wavefronts through LDS.
+    if (wave == 0 && lane < K) {
+        uint64_t row_ptr = 0, scale_ptr = 0;
+        uint32_t scale_stride = 0;
         const uint32_t entry = token * K + lane;
         const uint32_t expert =
             (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
@@ -176,13 +189,22 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
             toff = ws.block_prefix[((size_t)g * ws.nb_max + chunk) * E + expert] +
                    ws.local_rank[(size_t)g * ws.max_tk + entry];
             slot = ws.slot_base[g * E + expert] + toff;
-            slot = resolve_copy(args.dst[owner_of_expert(ws, expert)], ws, slot, wave == 0, &row_ptr, &scale_ptr,
+            slot = resolve_copy(args.dst[owner_of_expert(ws, expert)], ws, slot, true, &row_ptr, &scale_ptr,
                                 &scale_stride);
         }
-        if (wave == 0) {
-            ws.route_slot[(size_t)g * ws.max_tk + entry] = slot;
-            ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
-        }
+        ws.route_slot[(size_t)g * ws.max_tk + entry] = slot;
+        ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
+        s_row_ptr[lane] = row_ptr;
+        s_route_scale_ptr[lane] = scale_ptr;
+        s_route_scale_stride[lane] = scale_stride;
+    }
+    __syncthreads();
+    uint64_t row_ptr = 0, scale_ptr = 0;
+    uint32_t scale_stride = 0;
+    if (lane < K) {
+        row_ptr = s_row_ptr[lane];
+        scale_ptr = s_route_scale_ptr[lane];
+        scale_stride = s_route_scale_stride[lane];
     }
     const u32x4 none = {0, 0, 0, 0};
     push_rows<QUANT, false>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr,
@@ -433,6 +455,173 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
                            s_scale_stride, pre_a, pre_b);
 }
 
+// Pack of a large group step, after a routing launch that left, per chunk, the
+// histogram and the rank of every entry inside its chunk, and, for the whole
+// step, the totals per (source, expert) and per expert.  No launch in between
+// lays anything out: wavefront 0 of a token workgroup resolves the K rows
+// itself, eight lanes per route, each route with three short sums whose terms
+// are spread over the lanes and added on the DPP path:
+//   copies of the same source and expert in earlier chunks      (chunk histograms)
+//   copies of the sources the receiver lays out before mine     (totals per source)
+//   padded rows of the receiver's experts before mine           (totals per expert)
+// The terms come from tables of a few KB that stay in cache, and they travel
+// while the token's row is on its way from memory.  Before the token workgroups
+// the grid holds one workgroup per receiver (expert counts for the caller,
+// layout tables) and one per source (its totals and their scan); the last of
+// them hands the totals over to the next step.
+template <bool QUANT>
+__global__ __launch_bounds__(1024) void dispatch_resolve_kernel(const PushArgs args, const FinalizeArgs fin,
+                                                                const Workspace ws) {
+    __shared__ float s_scale[QUANT ? kMaxLdsScales : 1];
+    __shared__ uint64_t s_scale_ptr[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint32_t s_scale_stride[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint64_t s_row_ptr[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint64_t s_route_scale_ptr[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint32_t s_route_scale_stride[A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint32_t tot[A2A_MAX_EXPERTS + kMaxWorld];
+    __shared__ uint32_t scratch[kRouteWaves];
+    __shared__ uint32_t s_carry;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const uint32_t G = ws.num_groups, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
+    const uint32_t total_tokens = args.token_start[G];
+    const uint32_t use = ws.turn[1] & 1u;
+    const uint32_t *per_source = ws.totals + (size_t)use * (G + 1) * E;   // [E][G]
+    const uint32_t *per_expert = per_source + (size_t)G * E;              // [E]
+
+    // The receiver and source workgroups come first in the grid, so that they run
+    // beside the token workgroups instead of after them.
+    const uint32_t extras = ws.world + G;
+    if (blockIdx.x < extras) {
+        const uint32_t extra = blockIdx.x;
+        if (extra < ws.world) {
+            // receiver: rows per expert, padded offsets, first row of every (source, expert) run
+            const uint32_t r = extra;
+            if (!(fin.recv_mask >> r & 1)) return;
+            for (uint32_t w = tid; w < G * Le; w += blockDim.x) {
+                const uint32_t g = Le > 1 ? __umulhi(w, ws.le_magic) : w;
+                const uint32_t e = r * Le + (w - g * Le);
+                tot[w] = e < E ? per_source[e * G + g] : 0;
+            }
+            __syncthreads();
+            layout_from_totals(fin, ws, r, tot, scratch);
+            return;
+        }
+        // source: its totals and their inclusive scan over the experts
+        const uint32_t g = extra - ws.world;
+        uint32_t carry = 0;
+        for (uint32_t e0 = 0; e0 < E; e0 += blockDim.x) {
+            const uint32_t e = e0 + tid;
+            const uint32_t c = e < E ? per_source[e * G + g] : 0;
+            const uint32_t incl = carry + block_inclusive_scan(c, scratch);
+            if (e < E) {
+                ws.num_routed[g * E + e] = c;
+                ws.expert_offsets[g * E + e] = incl;
+            }
+            if (e0 + blockDim.x < E) {   // uniform: another round follows
+                if (tid == blockDim.x - 1) s_carry = incl;
+                __syncthreads();
+                carry = s_carry;
+            }
+        }
+        // the next routing launch fills the other copy of the totals
+        if (g + 1 == G && tid == 0) ws.turn[0] = use ^ 1u;
+        return;
+    }
+
+    const uint32_t work = blockIdx.x - extras;
+    if (work >= total_tokens) return;
+    uint32_t g = 0;
+    while (g + 1 < G && work >= args.token_start[g + 1]) ++g;
+    const uint32_t token = work - args.token_start[g];
+    const PushSrc &src = args.src[g];
+    if (token >= effective_tokens(src.bound_m, src.num_tokens)) return;
+
+    // Wavefront 0 resolves the K routes, eight at a time with eight lanes per
+    // route, and hands them to the others through LDS.  Two dependent trips to
+    // memory: the expert ids and in-chunk ranks, then every term of the sums and
+    // the receivers' descriptors in one go.  Measured on the prefill shape: done
+    // by all seven wavefronts the lookups were three times the cache requests of
+    // the rows themselves and cost 7 us; asking for the token's row BEFORE the
+    // lookups (to hide its latency) cost another 4 us, because under a saturated
+    // memory system what counts is to store a row as soon as it has arrived.
+    const uint32_t *counts = ws.chunk_counts + (size_t)g * E * ws.nb_max;   // [E][nb_max]
+    const uint32_t pad = ws.expert_padding;
+    const uint32_t part = lane & 7, route = lane >> 3;
+    const uint32_t passes = wave == 0 ? (K + 7) / 8 : 0;
+    for (uint32_t pass = 0; pass < passes; ++pass) {
+        const uint32_t k = pass * 8 + route;
+        const bool in = k < K;
+        const uint32_t kk = in ? k : 0;   // a lane without a route reads route 0 and is dropped below
+        const uint32_t id = (uint32_t)src.indices[(size_t)token * src.indices_stride + kk];
+        const uint32_t local = ws.local_rank[(size_t)g * ws.max_tk + token * K + kk];
+        const bool live = in && id < E;
+        const uint32_t e = live ? id : 0;
+        const uint32_t upto = live ? (token * K + k) / kRouteBlock : 0;   // chunk of this entry
+        const uint32_t r = owner_of_expert(ws, e);
+        const uint32_t le = live ? e - r * Le : 0;
+        // four terms of each sum per lane without a branch (clamped index, masked value)
+        const uint32_t before = ws.laid_before[r * G + g];
+        const PushDst dst = args.dst[r];
+        uint32_t v_chunk[4], v_source[4], v_rows[4];
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            const uint32_t n = part + 8 * i;
+            v_chunk[i] = counts[(size_t)e * ws.nb_max + (n < upto ? n : 0)];
+            v_source[i] = per_source[e * G + (n < G ? n : 0)];
+            v_rows[i] = per_expert[r * Le + (n < le ? n : 0)];
+        }
+        uint32_t earlier = 0, base = 0;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) {
+            const uint32_t n = part + 8 * i;
+            earlier += n < upto ? v_chunk[i] : 0;
+            base += n < G && (before >> n & 1) ? v_source[i] : 0;
+            const uint32_t padded = pad > 1 ? (v_rows[i] + pad - 1) / pad * pad : v_rows[i];
+            base += n < le ? padded : 0;
+        }
+        // longer sums (more than 32 chunks in a source, more than 32 experts in a rank)
+        for (uint32_t c = 32 + part; c < upto; c += 8) earlier += counts[(size_t)e * ws.nb_max + c];
+        for (uint32_t q = 32 + part; q < le; q += 8) {
+            const uint32_t rows = per_expert[r * Le + q];
+            base += pad > 1 ? (rows + pad - 1) / pad * pad : rows;
+        }
+        earlier = group8_sum(earlier);
+        base = group8_sum(base);
+        const uint32_t toff = live ? earlier + local : 0;
+        uint64_t to_row, to_scale;
+        uint32_t to_stride;
+        uint32_t slot = resolve_copy(dst, ws, base + toff, part == 0 && live, &to_row, &to_scale, &to_stride);
+        if (!live) {
+            slot = kInvalidSlot;
+            to_row = 0;
+            to_scale = 0;
+            to_stride = 0;
+        }
+        if (part == 0 && in) {
+            const uint32_t entry = token * K + k;
+            ws.route_slot[(size_t)g * ws.max_tk + entry] = slot;
+            ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
+            s_row_ptr[k] = to_row;
+            s_route_scale_ptr[k] = to_scale;
+            s_route_scale_stride[k] = to_stride;
+        }
+    }
+    __syncthreads();
+    uint64_t row_ptr = 0, scale_ptr = 0;   // lane k: where the copy of route k goes
+    uint32_t scale_stride = 0;
+    if (lane < K) {
+        row_ptr = s_row_ptr[lane];
+        scale_ptr = s_route_scale_ptr[lane];
+        scale_stride = s_route_scale_stride[lane];
+    }
+    const u32x4 none = {0, 0, 0, 0};
+    push_rows<QUANT, false>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr,
+                            s_scale_stride, none, none);
+}
+
 hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool quantize,
                                 uint32_t total_tokens, hipStream_t stream) {
     if (total_tokens == 0) return hipSuccess;
@@ -469,6 +658,21 @@ hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, 
         hipLaunchKernelGGL(dispatch_small_kernel<true>, dim3(blocks), dim3(threads), lds, stream, args, fin, ws);
     } else {
         hipLaunchKernelGGL(dispatch_small_kernel<false>, dim3(blocks), dim3(threads), lds, stream, args, fin, ws);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_dispatch_resolve(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
+                                   bool quantize, uint32_t total_tokens, hipStream_t stream) {
+    uint32_t threads = push_threads(args, quantize);
+    if (threads < ws.experts_per_rank) {   // a receiver workgroup has one thread per local expert
+        threads = (ws.experts_per_rank + kWave - 1) / kWave * kWave;
+    }
+    const uint32_t blocks = total_tokens + ws.world + ws.num_groups;
+    if (quantize) {
+        hipLaunchKernelGGL(dispatch_resolve_kernel<true>, dim3(blocks), dim3(threads), 0, stream, args, fin, ws);
+    } else {
+        hipLaunchKernelGGL(dispatch_resolve_kernel<false>, dim3(blocks), dim3(threads), 0, stream, args, fin, ws);
     }
     return hipGetLastError();
 }

@@ -32,6 +32,12 @@ struct Workspace {
     uint32_t *token_offset;    // [N][max_tk]    rank of every copy inside its (source, expert)
     uint32_t *err;             // [1]            A2A_DEV_* bits, sticky
     const uint32_t *order;     // [N][8] words   byte i of receiver r's row: the i-th source it lays out
+    const uint32_t *laid_before; // [N][G]       bit s of word [r][g]: receiver r lays out source s before source g
+    uint32_t *chunk_counts;    // [N][E][nb_max] block_hist with the chunks of an expert side by side (large group steps)
+    uint32_t *totals;          // [2][(G+1)*E]   counts of a step per expert and source ([E][G]), then per expert ([E]),
+                               //                accumulated by the routing launch of large group steps; two copies
+                               //                used in turn
+    uint32_t *turn;            // [2]            [0] copy the next routing launch fills, [1] copy the current step uses
     uint32_t max_tk;           // max_num_tokens * K
     uint32_t nb_max;           // ceil(max_tk / kRouteBlock)
     uint32_t world;            // N logical ranks (receivers)
@@ -135,6 +141,13 @@ struct CombArgs {
 // launch.
 hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
                         hipStream_t stream);
+// The same, and every chunk adds its counts to the step's totals (large group steps).
+hipError_t launch_route_accumulate(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
+                                   hipStream_t stream);
+// Pack that resolves its rows from the chunk histograms and the step's totals, with the
+// receiver layout and the per-source tables computed by extra workgroups of the same launch.
+hipError_t launch_dispatch_resolve(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
+                                   bool quantize, uint32_t total_tokens, hipStream_t stream);
 hipError_t launch_finalize(const FinalizeArgs &args, const Workspace &ws, hipStream_t stream);
 hipError_t launch_route_fused(const RouteArgs &args, const FinalizeArgs &fin, const Workspace &ws,
                               hipStream_t stream);

@@ -208,16 +208,45 @@ __device__ uint32_t rank_chunk(const RouteSrc &src, const Workspace &ws, uint32_
 
 }  // namespace
 
+// ACCUM: the launch also adds every chunk's counts to the step's totals (per
+// source and expert, and per expert), which the pack of a large group step
+// resolves its rows from.  The totals exist twice and are used in turn, so that
+// this launch can clear the copy of the NEXT step while it fills its own:
+// turn[0] says which copy to fill (flipped by the pack launch that follows),
+// turn[1] tells that pack which copy this launch filled.  All of it lives on
+// the device, so a recorded sequence of launches can be replayed.
+template <bool ACCUM>
 __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs args,
                                                                  const Workspace ws) {
     __shared__ uint16_t wave_hist[kRouteWaves][A2A_MAX_EXPERTS];
+    const uint32_t G = ws.num_groups, E = ws.num_experts;
+    const uint32_t words = (G + 1) * E;
+    uint32_t fill = 0;
+    if constexpr (ACCUM) {
+        fill = ws.turn[0] & 1u;
+        if (blockIdx.x == 0) {
+            uint32_t *next = ws.totals + (size_t)(fill ^ 1u) * words;
+            for (uint32_t i = threadIdx.x; i < words; i += kRouteBlock) next[i] = 0;
+            if (threadIdx.x == 0) ws.turn[1] = fill;
+        }
+        if (blockIdx.x >= args.block_start[G]) return;   // a step without entries: only the duties above
+    }
     // Which source and which chunk of it this workgroup handles (uniform).
     uint32_t g = 0;
-    while (g + 1 < ws.num_groups && blockIdx.x >= args.block_start[g + 1]) ++g;
+    while (g + 1 < G && blockIdx.x >= args.block_start[g + 1]) ++g;
     const uint32_t chunk = blockIdx.x - args.block_start[g];
     const uint32_t count = rank_chunk(args.src[g], ws, g, chunk, wave_hist);
-    if (threadIdx.x < ws.num_experts) {
-        ws.block_hist[((size_t)g * ws.nb_max + chunk) * ws.num_experts + threadIdx.x] = count;
+    if (threadIdx.x < E) {
+        ws.block_hist[((size_t)g * ws.nb_max + chunk) * E + threadIdx.x] = count;
+        if constexpr (ACCUM) {
+            // the pack reads all chunks of ONE expert, and all sources of one expert: keep those together
+            ws.chunk_counts[((size_t)g * E + threadIdx.x) * ws.nb_max + chunk] = count;
+            if (count != 0) {
+                uint32_t *mine = ws.totals + (size_t)fill * words;
+                atomicAdd(&mine[threadIdx.x * G + g], count);
+                atomicAdd(&mine[G * E + threadIdx.x], count);
+            }
+        }
     }
 }
 
@@ -372,7 +401,15 @@ __global__ __launch_bounds__(kRouteBlock) void route_finalize_kernel(const Final
 hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
                         hipStream_t stream) {
     if (total_blocks == 0) return hipSuccess;
-    hipLaunchKernelGGL(route_hist_kernel, dim3(total_blocks), dim3(kRouteBlock), 0, stream, args, ws);
+    hipLaunchKernelGGL(route_hist_kernel<false>, dim3(total_blocks), dim3(kRouteBlock), 0, stream, args, ws);
+    return hipGetLastError();
+}
+
+hipError_t launch_route_accumulate(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
+                                   hipStream_t stream) {
+    // at least one workgroup: the launch also hands over the totals between steps
+    hipLaunchKernelGGL(route_hist_kernel<true>, dim3(total_blocks != 0 ? total_blocks : 1), dim3(kRouteBlock), 0,
+                       stream, args, ws);
     return hipGetLastError();
 }
 
