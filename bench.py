@@ -117,9 +117,11 @@ class Workload:
             self.combine_args.append(self.ctx.pack_combine_args(c))
 
     def step(self, i: int, stream: int, events=None):
+        """One dispatch + combine.  `events` = (start, middle, end); a start of None means the previous
+        step's end event marks this step's start too (one event less between two steps)."""
         import torch
         j = i % len(self.routings)
-        if events is not None:
+        if events is not None and events[0] is not None:
             events[0].record()
         self.ctx.dispatch(self.dispatch_args[j], True, stream)
         if events is not None:
@@ -139,19 +141,22 @@ def time_workload(wl: Workload, steps: int, warmup: int):
     for i in range(warmup):
         wl.step(i, stream)
     torch.cuda.synchronize(wl.device)
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(3)] for _ in range(steps)]
+    # steps + 1 boundary events (the end of a step is the start of the next) and one in the middle of each
+    bounds = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    middle = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
     torch.cuda.synchronize(wl.device)
     t0 = time.perf_counter()
+    bounds[0].record()
     for i in range(steps):
-        wl.step(warmup + i, stream, events[i])
+        wl.step(warmup + i, stream, (None, middle[i], bounds[i + 1]))
     torch.cuda.synchronize(wl.device)
     wall_s = time.perf_counter() - t0
     flags = wl.ctx.status(stream)
     if flags:
         raise RuntimeError(f"device error flags {flags}")
-    disp = [e[0].elapsed_time(e[1]) * 1e3 for e in events]   # microseconds
-    comb = [e[1].elapsed_time(e[2]) * 1e3 for e in events]
-    both = [e[0].elapsed_time(e[2]) * 1e3 for e in events]
+    disp = [bounds[i].elapsed_time(middle[i]) * 1e3 for i in range(steps)]   # microseconds
+    comb = [middle[i].elapsed_time(bounds[i + 1]) * 1e3 for i in range(steps)]
+    both = [bounds[i].elapsed_time(bounds[i + 1]) * 1e3 for i in range(steps)]
     return wall_s, disp, comb, both
 
 

@@ -237,7 +237,7 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
     const uint32_t chunk = blockIdx.x - args.block_start[g];
     const uint32_t count = rank_chunk(args.src[g], ws, g, chunk, wave_hist);
     if (threadIdx.x < E) {
-        ws.block_hist[((size_t)g * ws.nb_max + chunk) * E + threadIdx.x] = count;
+        if constexpr (!ACCUM) ws.block_hist[((size_t)g * ws.nb_max + chunk) * E + threadIdx.x] = count;
         if constexpr (ACCUM) {
             // the pack reads all chunks of ONE expert, and all sources of one expert: keep those together
             ws.chunk_counts[((size_t)g * E + threadIdx.x) * ws.nb_max + chunk] = count;
