@@ -7,7 +7,7 @@ import pytest
 import torch
 
 import a2a_oracle as oracle
-from a2a_cases import C0, C1, bf16_codes, make_world
+from a2a_cases import C0, C1, bf16_codes, make_world, scaled
 from a2a_harness import SENTINEL, make_ops, rows_needed, run_oracle
 from a2a_transport import RefConfig, make_ref_rank, oracle_combine, oracle_dispatch, rows_for
 from a2a_transport import make_ops as make_transport_ops
@@ -242,13 +242,16 @@ def test_operator_asserts_like_the_reference():
             op.destroy()
 
 
-def test_calls_can_be_captured_in_a_hip_graph():
+@pytest.mark.parametrize("case,sources", [(C1, "all"), (scaled(C1, 1200), "one"), (scaled(C1, 300), "all")],
+                         ids=["one_launch_dispatch", "two_launch_dispatch_one_source", "two_launch_dispatch"])
+def test_calls_can_be_captured_in_a_hip_graph(case, sources):
     """The calls only enqueue kernels whose arguments travel by value (no allocation, copy or
     synchronisation inside), so a dispatch + combine can be captured once and replayed
     (docs/fabric-lib.md:15 lists graph capture as a feature of the reference).  Every replay,
-    with eager work in between, must reproduce the eager result."""
-    case = C1
-    world = make_world(case, "all")
+    with eager work in between, must reproduce the eager result.  The larger cases take the
+    two-launch dispatch, whose step totals alternate between two copies in device memory: the
+    replays land on either copy."""
+    world = make_world(case, sources)
     rows = rows_needed(case, world)
     N, Le, H, Hs = case.world_size, case.experts_per_rank, case.hidden_dim, case.hidden_dim_scale
     _, ops = make_ops(case, DEV)
