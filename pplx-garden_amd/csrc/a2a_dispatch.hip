@@ -640,8 +640,9 @@ bool dispatch_small_fits(const PushArgs &args, const Workspace &ws, bool quantiz
     const uint64_t entries = (uint64_t)total_tokens * ws.topk;
     const uint64_t table = ((uint64_t)ws.num_groups + 3) * ws.num_experts;
     // The counting is redundant: every token workgroup visits every entry.  Measured with 8
-    // sources and 8 entries per token, the one launch is ahead of routing + push launches by
-    // 10 us at 512 tokens x 4096 entries (17 against 27 us) and by 3 us at 1024 x 8192.
+    // sources and 8 entries per token against the two-launch dispatch: 13.0 against 15.4 us at
+    // 256 tokens x 2048 entries, 17.0 against 16.3 us at 512 x 4096, 32.8 against 25.8 us at
+    // 1024 x 8192.
     return entries <= A2A_SMALL_MAX_ENTRIES && entries * total_tokens <= A2A_SMALL_MAX_VISITS &&
            total_tokens <= 1024 && table <= 8192 + 3072 &&
            ws.experts_per_rank <= push_threads(args, quantize);

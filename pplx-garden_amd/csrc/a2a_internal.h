@@ -158,7 +158,7 @@ hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool 
 #define A2A_SMALL_MAX_ENTRIES 8192
 #endif
 #ifndef A2A_SMALL_MAX_VISITS
-#define A2A_SMALL_MAX_VISITS (8u << 20)   // entries x tokens
+#define A2A_SMALL_MAX_VISITS (3u << 19)   // entries x tokens
 #endif
 bool dispatch_small_fits(const PushArgs &args, const Workspace &ws, bool quantize, uint32_t total_tokens);
 hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
