@@ -84,14 +84,17 @@ def make_ops(case: Case, device: torch.device, max_num_tokens: Optional[int] = N
 
 
 def run_gpu(case: Case, world_data: Sequence[RankData], rows: int, device: torch.device,
-            split: bool = False, expert_y_override=None, context_flags: int = 0) -> WorldResult:
+            split: bool = False, expert_y_override=None, context_flags: int = 0, ops=None) -> WorldResult:
     """dispatch -> 2*dequant -> combine on the GPU through the operator API.
 
     split=False: every rank calls dispatch()/combine() with do_send and do_recv
     (the group calls of the library); split=True: all sends, then all recvs (the
-    four split calls)."""
+    four split calls).  With `ops` the given operators are used (and kept): several
+    steps on one context."""
     N, H, Hs, Le = case.world_size, case.hidden_dim, case.hidden_dim_scale, case.experts_per_rank
-    _, ops = make_ops(case, device, context_flags=context_flags)
+    own_ops = ops is None
+    if own_ops:
+        _, ops = make_ops(case, device, context_flags=context_flags)
     try:
         dev = [
             dict(x=rd.x.to(device), idx=rd.indices_u32.to(device), w=rd.weights.to(device))
@@ -155,8 +158,9 @@ def run_gpu(case: Case, world_data: Sequence[RankData], rows: int, device: torch
             [o["o"].view(torch.int16).cpu().numpy().view(np.uint16) for o in outs])
         return res
     finally:
-        for op in ops:
-            op.destroy()
+        if own_ops:
+            for op in ops:
+                op.destroy()
 
 
 def assert_dispatch_equal(case: Case, got: WorldResult, want: WorldResult) -> None:

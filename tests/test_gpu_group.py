@@ -52,3 +52,30 @@ def test_small_steps_with_separate_routing_kernels(case, sources, split, device)
         got = run_gpu(case, world, rows, device, split=split, context_flags=flags)
         assert_dispatch_equal(case, got, want)
         assert_combine_close(case, got, want)
+
+
+def test_steps_of_different_sizes_on_one_context(device):
+    """One set of operators, a sequence of steps that take the one-launch dispatch, the two-launch
+    dispatch (whose step totals alternate between two copies on the device) and the split calls in
+    turn: every step must match the oracle, whatever ran before it."""
+    from a2a_cases import Case, make_rank
+    from a2a_harness import make_ops
+    case = Case("mixed_steps", 1500, 256, 32, 8, 8, 8100, expert_padding=4)
+    _, ops = make_ops(case, device)
+    try:
+        steps = [([40, 0, 13, 1, 0, 0, 40, 7], False), ([1500, 0, 0, 0, 0, 0, 0, 0], False),
+                 ([1500, 300, 0, 1, 90, 0, 0, 1200], False), ([128] * 8, True), ([600] * 8, False),
+                 ([0] * 8, False), ([64] * 8, False), ([1100, 0, 0, 0, 0, 0, 0, 5], True),
+                 ([1100, 0, 0, 0, 0, 0, 0, 5], False), ([700] * 8, False)]
+        for i, (tokens, split) in enumerate(steps):
+            print(f"step {i}: tokens={tokens} split={split}", flush=True)
+            step_case = scaled(case, max(tokens))
+            world = [make_rank(step_case, r, t) for r, t in enumerate(tokens)]
+            rows = rows_needed(step_case, world)
+            want = run_oracle(step_case, world, rows)
+            got = run_gpu(step_case, world, rows, device, split=split, ops=ops)
+            assert_dispatch_equal(step_case, got, want)
+            assert_combine_close(step_case, got, want)
+    finally:
+        for op in ops:
+            op.destroy()
