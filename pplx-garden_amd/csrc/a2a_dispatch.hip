@@ -32,13 +32,13 @@ static_assert(sizeof(PushArgs) + sizeof(FinalizeArgs) + sizeof(Workspace) <= 409
 
 // Moves the row of `token` to its copies.  Lanes 0..K-1 of EVERY wavefront hold
 // the row pointer, scale pointer and scale stride of route k (0 = no copy).
-// With PRELOADED, `pre_a`/`pre_b` already hold the chunk of this thread's first
-// iteration (loaded by the caller before it knew the routes).  Whole workgroup.
-template <bool QUANT, bool PRELOADED>
+// The row is loaded here, AFTER the routes are known: asking for it earlier to
+// hide its latency was measured slower at every size (4 us on the 4096-token
+// pack, 0.4 us on the 128-token one).  Whole workgroup.
+template <bool QUANT>
 __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &src, uint32_t token, uint32_t K,
                                           uint64_t row_ptr, uint64_t scale_ptr, uint32_t scale_stride,
-                                          float *s_scale, uint64_t *s_scale_ptr, uint32_t *s_scale_stride,
-                                          u32x4 pre_a, u32x4 pre_b) {
+                                          float *s_scale, uint64_t *s_scale_ptr, uint32_t *s_scale_stride) {
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
@@ -51,10 +51,7 @@ __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &s
             const uint32_t c = base + lane;
             const bool active = c < num_chunks;
             u32x4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
-            if (PRELOADED && base == wave * kWave) {
-                a = pre_a;
-                b = pre_b;
-            } else if (active) {
+            if (active) {
                 const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)c * 32);
                 a = __builtin_nontemporal_load(p);
                 b = __builtin_nontemporal_load(p + 1);
@@ -86,12 +83,7 @@ __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &s
     } else {
         const uint32_t num_chunks = args.row_bytes / 16;
         for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
-            u32x4 v;
-            if (PRELOADED && c == tid) {
-                v = pre_a;
-            } else {
-                v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
-            }
+            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
             for (uint32_t k = 0; k < K; ++k) {
                 const uint64_t row = read_lane64(row_ptr, k);
                 if (row != 0) {
@@ -206,16 +198,14 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
         scale_ptr = s_route_scale_ptr[lane];
         scale_stride = s_route_scale_stride[lane];
     }
-    const u32x4 none = {0, 0, 0, 0};
-    push_rows<QUANT, false>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr,
-                            s_scale_stride, none, none);
+    push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride);
 }
 
 // Routing pass and dispatch pack in ONE launch, for small steps (decode).  The
 // grid holds one workgroup per token, then one per receiver; none depends on
 // another, because every workgroup counts, by itself, what it needs to know
 // about the whole step:
-//  - a token workgroup asks for its row early, counts the entries of every
+//  - a token workgroup counts the entries of every
 //    source per (source, expert) and the entries of its own source before its
 //    token per expert (LDS atomics: counts do not depend on arrival order), and
 //    from those derives the receiver rows of its K copies exactly as the
@@ -302,13 +292,10 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
 #define A2A_SMALL_BATCH 8
 #endif
     constexpr uint32_t kBatch = A2A_SMALL_BATCH;
-    // The token's own row is requested right after the first batch of indices,
-    // so that counting does not wait for it.
     const PushSrc &src = args.src[my_g];
     const uint32_t rank = blockIdx.x - total_tokens;        // receivers only
     const uint32_t my_first = (args.token_start[my_g] + token) * K;   // flat index of my first entry
     uint32_t my_expert = 0xFFFFFFFFu;
-    u32x4 pre_a = {0, 0, 0, 0}, pre_b = {0, 0, 0, 0};
     // The order in which every receiver lays out the sources comes from device
     // memory: asked for here, stored to LDS after the counting.
     const uint32_t order_words = receiver ? 0 : ws.world * (kMaxWorld / 4);
@@ -331,18 +318,6 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
         }
         if (f0 == 0 && !receiver) {
             if (lane < K) my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
-            const uint8_t *x_row = src.x + (size_t)token * src.x_stride;
-            if constexpr (QUANT) {
-                if (tid < args.hidden_dim / 16) {
-                    const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)tid * 32);
-                    pre_a = __builtin_nontemporal_load(p);
-                    pre_b = __builtin_nontemporal_load(p + 1);
-                }
-            } else {
-                if (tid < args.row_bytes / 16) {
-                    pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + tid);
-                }
-            }
         }
 #pragma unroll
         for (uint32_t j = 0; j < kBatch; ++j) {
@@ -451,8 +426,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
             ws.token_offset[(size_t)my_g * ws.max_tk + entry] = toff;
         }
     }
-    push_rows<QUANT, true>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr,
-                           s_scale_stride, pre_a, pre_b);
+    push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride);
 }
 
 // Pack of a large group step, after a routing launch that left, per chunk, the
@@ -617,9 +591,7 @@ __global__ __launch_bounds__(1024) void dispatch_resolve_kernel(const PushArgs a
         scale_ptr = s_route_scale_ptr[lane];
         scale_stride = s_route_scale_stride[lane];
     }
-    const u32x4 none = {0, 0, 0, 0};
-    push_rows<QUANT, false>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr,
-                            s_scale_stride, none, none);
+    push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride);
 }
 
 hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool quantize,

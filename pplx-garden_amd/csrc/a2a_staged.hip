@@ -17,11 +17,9 @@ size_t align_up_sz(size_t n, size_t a) { return (n + a - 1) / a * a; }
 // behind every row of the sender's expert-sorted order.
 // ---------------------------------------------------------------------------
 
-// Stages the row of `token` (payload, then scales).  With PRELOADED the chunk of
-// this thread's first iteration is already in `pre_a` / `pre_b`.  Whole workgroup.
-template <bool QUANT, bool PRELOADED>
-__device__ __forceinline__ void stage_row(const StageSendArgs &args, const Staging &st, uint32_t g, uint32_t token,
-                                          u32x4 pre_a, u32x4 pre_b) {
+// Stages the row of `token` (payload, then scales).  Whole workgroup.
+template <bool QUANT>
+__device__ __forceinline__ void stage_row(const StageSendArgs &args, const Staging &st, uint32_t g, uint32_t token) {
     const uint32_t tid = threadIdx.x;
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
@@ -36,10 +34,7 @@ __device__ __forceinline__ void stage_row(const StageSendArgs &args, const Stagi
             const uint32_t c = base + lane;
             const bool active = c < num_chunks;
             u32x4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
-            if (PRELOADED && base == wave * kWave) {
-                a = pre_a;
-                b = pre_b;
-            } else if (active) {
+            if (active) {
                 const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)c * 32);
                 a = __builtin_nontemporal_load(p);
                 b = __builtin_nontemporal_load(p + 1);
@@ -55,8 +50,7 @@ __device__ __forceinline__ void stage_row(const StageSendArgs &args, const Stagi
         const uint32_t num_chunks = args.row_bytes / 16;
         for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
             reinterpret_cast<u32x4 *>(row)[c] =
-                PRELOADED && c == tid ? pre_a
-                                      : __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
+                __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
         }
         if (src.x_scale != nullptr) {
             const float *xs = src.x_scale + (size_t)token * src.xs_stride_token;
@@ -93,13 +87,12 @@ __global__ __launch_bounds__(1024) void stage_send_kernel(const StageSendArgs ar
         }
         ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
     }
-    const u32x4 none = {0, 0, 0, 0};
-    stage_row<QUANT, false>(args, st, g, token, none, none);
+    stage_row<QUANT>(args, st, g, token);
 }
 
 // The send of a small step in ONE launch (the reference's dispatch-send kernel
-// is one launch too, a2a_dispatch_send.cu:158-523): every token workgroup asks
-// for its row, counts the entries of the sender per expert and those before its
+// is one launch too, a2a_dispatch_send.cu:158-523): every token workgroup
+// counts the entries of the sender per expert and those before its
 // own token (LDS atomics; counts do not depend on arrival order), scans the
 // counts over the experts, and has the position of each of its K copies in the
 // sender's expert-sorted order.  The workgroup of token 0 publishes the counts
@@ -130,7 +123,6 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
     __syncthreads();
 
     uint32_t my_expert = 0xFFFFFFFFu;
-    u32x4 pre_a = {0, 0, 0, 0}, pre_b = {0, 0, 0, 0};
     for (uint32_t f0 = 0; f0 < entries || f0 == 0; f0 += 8 * blockDim.x) {
         uint32_t expert[8];
 #pragma unroll
@@ -142,21 +134,8 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
                 expert[j] = (uint32_t)src.indices[(size_t)t * src.indices_stride + (f - t * K)];
             }
         }
-        if (f0 == 0) {
-            // the token's own ids and row, asked for after the first batch of the count
-            if (lane < K) my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
-            const uint8_t *x_row = src.x + (size_t)token * src.x_stride;
-            if constexpr (QUANT) {
-                if (tid < args.hidden_dim / 16) {
-                    const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)tid * 32);
-                    pre_a = __builtin_nontemporal_load(p);
-                    pre_b = __builtin_nontemporal_load(p + 1);
-                }
-            } else {
-                if (tid < args.row_bytes / 16) {
-                    pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + tid);
-                }
-            }
+        if (f0 == 0 && lane < K) {
+            my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
         }
 #pragma unroll
         for (uint32_t j = 0; j < 8; ++j) {
@@ -209,7 +188,7 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
             ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
         }
     }
-    stage_row<QUANT, true>(args, st, g, token, pre_a, pre_b);
+    stage_row<QUANT>(args, st, g, token);
 }
 
 // A team of `team` threads (one or more whole wavefronts) copies a row of
