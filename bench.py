@@ -15,7 +15,8 @@ reference's benchmark (benchmarks/bench_all_to_all.py:382-389).
 
 Prints one JSON line.  `value` is algorithmic bytes per step over the wall time
 of the timed region; per-phase times come from events recorded on the stream
-the kernels run on.  The 128-token decode shape is timed too and reported in
+the kernels run on, around every eighth step of the same region (an event
+between two launches idles the GPU for about 3 us, so they are kept sparse).  The 128-token decode shape is timed too and reported in
 the same line.  The CPU baseline is the oracle's C restatement, single thread,
 on the same workload.
 """
@@ -41,7 +42,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch on the default workload, from hardware counters (FETCH_SIZE and WRITE_SIZE
 # passes, scaled by what the same counters read for a 512 MiB copy: x2.000 and x1.000).  The counter
 # runs and their commands are summarised in profiles/hbm_traffic_dsv3_prefill_4096_pack_and_combine.md.
-MEASURED_TRAFFIC_BYTES = {"combine_gather_kernel": 531_696_000, "dispatch_resolve_kernel": 303_572_000,
+MEASURED_TRAFFIC_BYTES = {"combine_gather_kernel": 531_696_000, "dispatch_resolve_kernel": 303_576_000,
                           "dispatch_push_kernel": 303_073_000}
 
 
@@ -117,11 +118,10 @@ class Workload:
             self.combine_args.append(self.ctx.pack_combine_args(c))
 
     def step(self, i: int, stream: int, events=None):
-        """One dispatch + combine.  `events` = (start, middle, end); a start of None means the previous
-        step's end event marks this step's start too (one event less between two steps)."""
+        """One dispatch + combine; `events` = (start, middle, end) or None."""
         import torch
         j = i % len(self.routings)
-        if events is not None and events[0] is not None:
+        if events is not None:
             events[0].record()
         self.ctx.dispatch(self.dispatch_args[j], True, stream)
         if events is not None:
@@ -134,29 +134,32 @@ class Workload:
         self.ctx.destroy()
 
 
-def time_workload(wl: Workload, steps: int, warmup: int):
-    """W untimed steps, then exactly K timed steps between two synchronisations."""
+def time_workload(wl: Workload, steps: int, warmup: int, event_every: int = 8):
+    """W untimed steps, then exactly K timed steps between two synchronisations.
+
+    Every `event_every`-th step of the timed region carries three events (before the dispatch, between
+    dispatch and combine, after the combine); the phase times come from those steps.  An event between
+    two launches costs about 3 us of idle GPU (measured: 146.8 us per 4096-token step without events,
+    152.5 us with two per step), which is why not every step carries them."""
     import torch
     stream = torch.cuda.current_stream(wl.device).cuda_stream
     for i in range(warmup):
         wl.step(i, stream)
     torch.cuda.synchronize(wl.device)
-    # steps + 1 boundary events (the end of a step is the start of the next) and one in the middle of each
-    bounds = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
-    middle = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    sampled = [i for i in range(steps) if i % max(event_every, 1) == 0]
+    events = {i: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for i in sampled}
     torch.cuda.synchronize(wl.device)
     t0 = time.perf_counter()
-    bounds[0].record()
     for i in range(steps):
-        wl.step(warmup + i, stream, (None, middle[i], bounds[i + 1]))
+        wl.step(warmup + i, stream, events.get(i))
     torch.cuda.synchronize(wl.device)
     wall_s = time.perf_counter() - t0
     flags = wl.ctx.status(stream)
     if flags:
         raise RuntimeError(f"device error flags {flags}")
-    disp = [bounds[i].elapsed_time(middle[i]) * 1e3 for i in range(steps)]   # microseconds
-    comb = [middle[i].elapsed_time(bounds[i + 1]) * 1e3 for i in range(steps)]
-    both = [bounds[i].elapsed_time(bounds[i + 1]) * 1e3 for i in range(steps)]
+    disp = [events[i][0].elapsed_time(events[i][1]) * 1e3 for i in sampled]   # microseconds
+    comb = [events[i][1].elapsed_time(events[i][2]) * 1e3 for i in sampled]
+    both = [events[i][0].elapsed_time(events[i][2]) * 1e3 for i in sampled]
     return wall_s, disp, comb, both
 
 
@@ -196,6 +199,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--routings", type=int, default=4, help="distinct routings cycled over the steps")
+    ap.add_argument("--event-every", type=int, default=8,
+                    help="every how many timed steps carry the three events the phase times come from")
     ap.add_argument("--cpu-reps", type=int, default=3, help="repetitions of the CPU baseline (0 = skip)")
     ap.add_argument("--no-decode", action="store_true", help="skip the 128-token shape")
     ap.add_argument("--decode-only", action="store_true",
@@ -233,16 +238,17 @@ def main() -> int:
     ctx_flags = 2 if args.separate_routing else 0   # A2A_FLAG_SEPARATE_ROUTING
     if args.decode_only:
         wl2 = Workload(C2, device, args.routings, ctx_flags)
-        _, d2, c2, b2 = time_workload(wl2, args.steps, args.warmup)
+        w2, d2, c2, b2 = time_workload(wl2, args.steps, args.warmup, args.event_every)
         wl2.close()
-        print(json.dumps({"decode_128_only": {"dispatch_us_p50": round(Statistics.create(d2).p50, 2),
+        print(json.dumps({"decode_128_only": {"step_us_wall": round(w2 / args.steps * 1e6, 2),
+                                              "dispatch_us_p50": round(Statistics.create(d2).p50, 2),
                                               "combine_us_p50": round(Statistics.create(c2).p50, 2),
                                               "total_us_p50": round(Statistics.create(b2).p50, 2)}}))
         return 0
 
     case = C3
     wl = Workload(case, device, args.routings, ctx_flags)
-    wall_s, disp, comb, both = time_workload(wl, args.steps, args.warmup)
+    wall_s, disp, comb, both = time_workload(wl, args.steps, args.warmup, args.event_every)
     rows = wl.rows
     cpu_rd = wl.cpu_first
     wl.close()
@@ -275,15 +281,19 @@ def main() -> int:
     decode = None
     if not args.no_decode:
         wl2 = Workload(C2, device, args.routings, ctx_flags)
-        _, d2, c2, b2 = time_workload(wl2, max(args.steps, 200), args.warmup)
+        steps2 = max(args.steps, 200)
+        w2, d2, c2, b2 = time_workload(wl2, steps2, args.warmup, args.event_every)
         wl2.close()
         decode = {
             "workload": "DeepSeek-V3 decode: 128 tokens, hidden 7168, 256 experts / 8 logical ranks, top-8 uniform, 1% x50 outliers",
+            "step_us_wall": round(w2 / steps2 * 1e6, 2),
             "dispatch_us_p50": round(Statistics.create(d2).p50, 2),
             "combine_us_p50": round(Statistics.create(c2).p50, 2),
             "total_us_p50": round(Statistics.create(b2).p50, 2),
             "total_us_mean": round(Statistics.create(b2).mean, 2),
-            "note": "working set (26 MB) fits the 256 MB Infinity Cache and is not flushed between steps",
+            "note": "working set (26 MB) fits the 256 MB Infinity Cache and is not flushed between steps; "
+                    "step_us_wall is wall time over all steps, the p50 figures come from the steps that carry "
+                    "events (each event adds about 3 us)",
         }
 
     cpu = None
@@ -320,6 +330,8 @@ def main() -> int:
         },
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "prefill_4096": {
+            "step_us_wall": round(ms_per_step * 1e3, 2),
+            "steps_with_events": len(disp),
             "dispatch_us": {"p50": round(d_stats.p50, 2), "mean": round(d_stats.mean, 2)},
             "combine_us": {"p50": round(c_stats.p50, 2), "mean": round(c_stats.mean, 2)},
             "total_us": {"p50": round(b_stats.p50, 2), "mean": round(b_stats.mean, 2),
