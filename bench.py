@@ -42,7 +42,7 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 # HBM bytes per launch on the default workload, from hardware counters (FETCH_SIZE and WRITE_SIZE
 # passes, scaled by what the same counters read for a 512 MiB copy: x2.000 and x1.000).  The counter
 # runs and their commands are summarised in profiles/hbm_traffic_dsv3_prefill_4096_pack_and_combine.md.
-MEASURED_TRAFFIC_BYTES = {"combine_gather_kernel": 531_696_000, "dispatch_resolve_kernel": 303_576_000,
+MEASURED_TRAFFIC_BYTES = {"combine_gather_kernel": 531_696_000, "dispatch_resolve_kernel": 303_561_000,
                           "dispatch_push_kernel": 303_073_000}
 
 
@@ -117,10 +117,15 @@ class Workload:
             self.dispatch_args.append(self.ctx.pack_dispatch_args(d))
             self.combine_args.append(self.ctx.pack_combine_args(c))
 
-    def step(self, i: int, stream: int, events=None):
-        """One dispatch + combine; `events` = (start, middle, end) or None."""
+    def step(self, i: int, stream: int, events=None, kernel_events=None):
+        """One dispatch + combine.  `events` = (start, middle, end) recorded around the two calls;
+        `kernel_events` = (pack start, pack stop, gather start, gather stop), which the library
+        records at the start and end of the two bandwidth kernels themselves."""
         import torch
         j = i % len(self.routings)
+        if kernel_events is not None:
+            self.ctx.time_next_kernel(0, kernel_events[0].cuda_event, kernel_events[1].cuda_event)
+            self.ctx.time_next_kernel(1, kernel_events[2].cuda_event, kernel_events[3].cuda_event)
         if events is not None:
             events[0].record()
         self.ctx.dispatch(self.dispatch_args[j], True, stream)
@@ -134,33 +139,47 @@ class Workload:
         self.ctx.destroy()
 
 
-def time_workload(wl: Workload, steps: int, warmup: int, event_every: int = 8):
+def time_workload(wl: Workload, steps: int, warmup: int, event_every: int = 8, kernel_events: bool = True):
     """W untimed steps, then exactly K timed steps between two synchronisations.
 
-    Every `event_every`-th step of the timed region carries three events (before the dispatch, between
-    dispatch and combine, after the combine); the phase times come from those steps.  An event between
-    two launches costs about 3 us of idle GPU (measured: 146.8 us per 4096-token step without events,
-    152.5 us with two per step), which is why not every step carries them."""
+    Events are kept sparse, because they cost idle GPU time (measured on the 4096-token step: 146.8 us
+    per step without events, 152.5 us with one after each call; a launch that records its own start and
+    end costs about 8 us more).  Every `event_every`-th step carries three events around the two calls
+    (before the dispatch, between dispatch and combine, after the combine).  Every 2 * `event_every`-th
+    step, offset so that it is never one of those, has the library record events at the start and end
+    of the pack and the gather kernel themselves: those are the kernels' own durations.
+
+    Returns wall seconds and, in microseconds per sampled step: dispatch call, combine call, both,
+    pack kernel, gather kernel."""
     import torch
     stream = torch.cuda.current_stream(wl.device).cuda_stream
+    every = max(event_every, 1)
+    call_steps = [i for i in range(steps) if i % every == 0]
+    kernel_steps = [i for i in range(steps) if i % (2 * every) == every // 2 and i not in call_steps] \
+        if kernel_events else []
+    call_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for i in call_steps}
+    kern_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(4)] for i in kernel_steps}
+    for evs in kern_ev.values():         # an event gets its handle when it is first recorded
+        for ev in evs:
+            ev.record()
     for i in range(warmup):
         wl.step(i, stream)
     torch.cuda.synchronize(wl.device)
-    sampled = [i for i in range(steps) if i % max(event_every, 1) == 0]
-    events = {i: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for i in sampled}
-    torch.cuda.synchronize(wl.device)
     t0 = time.perf_counter()
     for i in range(steps):
-        wl.step(warmup + i, stream, events.get(i))
+        wl.step(warmup + i, stream, call_ev.get(i), kern_ev.get(i))
     torch.cuda.synchronize(wl.device)
     wall_s = time.perf_counter() - t0
     flags = wl.ctx.status(stream)
     if flags:
         raise RuntimeError(f"device error flags {flags}")
-    disp = [events[i][0].elapsed_time(events[i][1]) * 1e3 for i in sampled]   # microseconds
-    comb = [events[i][1].elapsed_time(events[i][2]) * 1e3 for i in sampled]
-    both = [events[i][0].elapsed_time(events[i][2]) * 1e3 for i in sampled]
-    return wall_s, disp, comb, both
+    us = lambda a, b: a.elapsed_time(b) * 1e3
+    disp = [us(call_ev[i][0], call_ev[i][1]) for i in call_steps]
+    comb = [us(call_ev[i][1], call_ev[i][2]) for i in call_steps]
+    both = [us(call_ev[i][0], call_ev[i][2]) for i in call_steps]
+    pack = [us(kern_ev[i][0], kern_ev[i][1]) for i in kernel_steps]
+    gather = [us(kern_ev[i][2], kern_ev[i][3]) for i in kernel_steps]
+    return wall_s, disp, comb, both, pack, gather
 
 
 def cpu_baseline(case, rd, reps: int):
@@ -238,9 +257,11 @@ def main() -> int:
     ctx_flags = 2 if args.separate_routing else 0   # A2A_FLAG_SEPARATE_ROUTING
     if args.decode_only:
         wl2 = Workload(C2, device, args.routings, ctx_flags)
-        w2, d2, c2, b2 = time_workload(wl2, args.steps, args.warmup, args.event_every)
+        w2, d2, c2, b2, p2, g2 = time_workload(wl2, args.steps, args.warmup, args.event_every)
         wl2.close()
         print(json.dumps({"decode_128_only": {"step_us_wall": round(w2 / args.steps * 1e6, 2),
+                                              "pack_kernel_us_mean": round(Statistics.create(p2).mean, 2),
+                                              "gather_kernel_us_mean": round(Statistics.create(g2).mean, 2),
                                               "dispatch_us_p50": round(Statistics.create(d2).p50, 2),
                                               "combine_us_p50": round(Statistics.create(c2).p50, 2),
                                               "total_us_p50": round(Statistics.create(b2).p50, 2)}}))
@@ -248,7 +269,10 @@ def main() -> int:
 
     case = C3
     wl = Workload(case, device, args.routings, ctx_flags)
-    wall_s, disp, comb, both = time_workload(wl, args.steps, args.warmup, args.event_every)
+    wall_s, disp, comb, both, pack, gather = time_workload(wl, args.steps, args.warmup, args.event_every)
+    # Phase statistics as the reference's benchmark reports them (events around each phase of EVERY
+    # iteration, benchmarks/bench_all_to_all.py:391-433), outside the timed region above.
+    _, disp_all, comb_all, both_all, _, _ = time_workload(wl, max(args.steps, 200), 0, 1, kernel_events=False)
     rows = wl.rows
     cpu_rd = wl.cpu_first
     wl.close()
@@ -257,6 +281,10 @@ def main() -> int:
     ms_per_step = wall_s / args.steps * 1e3
     value = (d_bytes + c_bytes) / (ms_per_step * 1e-3) / 1e9
     d_stats, c_stats, b_stats = Statistics.create(disp), Statistics.create(comb), Statistics.create(both)
+    p_stats, g_stats = Statistics.create(pack), Statistics.create(gather)
+
+    def stats_dict(xs):
+        return {k: round(v, 2) for k, v in Statistics.create(xs).as_dict().items()}
 
     def roof(bytes_, mean_us, kernel, note):
         achieved = bytes_ / (mean_us * 1e-6) / 1e9
@@ -265,35 +293,33 @@ def main() -> int:
                 "traffic": MEASURED_TRAFFIC_BYTES.get(kernel), "bytes_per_launch": bytes_,
                 "avg_us": round(mean_us, 2), "timing": note}
 
-    combine_roof = roof(c_bytes, c_stats.mean, "combine_gather_kernel",
-                        "events around a2a_combine, which is this one launch")
-    if args.separate_routing:
-        dispatch_roof = roof(d_bytes, d_stats.mean, "dispatch_push_kernel",
-                             "events around a2a_dispatch: route_hist + route_finalize + this kernel, so the "
-                             "kernel alone is faster than avg_us")
-    else:
-        dispatch_roof = roof(d_bytes, d_stats.mean, "dispatch_resolve_kernel",
-                             "events around a2a_dispatch: route_hist + this kernel, so the kernel alone is "
-                             "faster than avg_us")
-    dominant, other = ((combine_roof, dispatch_roof) if c_stats.mean >= d_stats.mean
+    note = ("events recorded by the launch itself at the start and end of this kernel (hipExtLaunchKernelGGL), "
+            f"on {len(gather)} of the {args.steps} timed steps")
+    combine_roof = roof(c_bytes, g_stats.mean, "combine_gather_kernel", note)
+    dispatch_roof = roof(d_bytes, p_stats.mean,
+                         "dispatch_push_kernel" if args.separate_routing else "dispatch_resolve_kernel", note)
+    dominant, other = ((combine_roof, dispatch_roof) if g_stats.mean >= p_stats.mean
                        else (dispatch_roof, combine_roof))
 
     decode = None
     if not args.no_decode:
         wl2 = Workload(C2, device, args.routings, ctx_flags)
         steps2 = max(args.steps, 200)
-        w2, d2, c2, b2 = time_workload(wl2, steps2, args.warmup, args.event_every)
+        w2, d2, c2, b2, p2, g2 = time_workload(wl2, steps2, args.warmup, args.event_every)
         wl2.close()
         decode = {
             "workload": "DeepSeek-V3 decode: 128 tokens, hidden 7168, 256 experts / 8 logical ranks, top-8 uniform, 1% x50 outliers",
             "step_us_wall": round(w2 / steps2 * 1e6, 2),
+            "pack_kernel_us_mean": round(Statistics.create(p2).mean, 2),
+            "gather_kernel_us_mean": round(Statistics.create(g2).mean, 2),
             "dispatch_us_p50": round(Statistics.create(d2).p50, 2),
             "combine_us_p50": round(Statistics.create(c2).p50, 2),
             "total_us_p50": round(Statistics.create(b2).p50, 2),
             "total_us_mean": round(Statistics.create(b2).mean, 2),
             "note": "working set (26 MB) fits the 256 MB Infinity Cache and is not flushed between steps; "
                     "step_us_wall is wall time over all steps, the p50 figures come from the steps that carry "
-                    "events (each event adds about 3 us)",
+                    "events around the calls (each event adds about 3 us), the kernel figures from events the "
+                    "launches record themselves",
         }
 
     cpu = None
@@ -336,7 +362,16 @@ def main() -> int:
             "combine_us": {"p50": round(c_stats.p50, 2), "mean": round(c_stats.mean, 2)},
             "total_us": {"p50": round(b_stats.p50, 2), "mean": round(b_stats.mean, 2),
                          "min": round(b_stats.min, 2), "p99": round(b_stats.p99, 2)},
+            "pack_kernel_us": {"p50": round(p_stats.p50, 2), "mean": round(p_stats.mean, 2)},
+            "gather_kernel_us": {"p50": round(g_stats.p50, 2), "mean": round(g_stats.mean, 2)},
             "algorithmic_bytes": {"dispatch": d_bytes, "combine": c_bytes},
+            "with_events_on_every_step": {
+                "note": "a second pass outside the timed region, events around each phase of every iteration as "
+                        "in the reference's benchmark; each event adds about 3 us",
+                "dispatch_us": stats_dict(disp_all),
+                "combine_us": stats_dict(comb_all),
+                "total_us": stats_dict(both_all),
+            },
         },
         "decode_128": decode,
         "roofline": dominant,

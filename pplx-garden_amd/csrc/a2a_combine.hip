@@ -285,28 +285,28 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
 
 template <typename T, typename U>
 static hipError_t launch_typed(const CombArgs &args, const Workspace &ws, uint32_t total_tokens,
-                               hipStream_t stream) {
+                               hipStream_t stream, KernelTiming timing) {
     constexpr int V = vec_elems<T>();
     const uint32_t chunks = args.hidden_dim / V;
     const uint32_t slabs = (chunks + kSlabChunks - 1) / kSlabChunks;
     const uint64_t units = (uint64_t)total_tokens * slabs;
     const uint32_t blocks = (uint32_t)((units + kCombineWaves - 1) / kCombineWaves);
     if (ws.topk == 8) {
-        hipLaunchKernelGGL((combine_gather_kernel<T, U, 8>), dim3(blocks), dim3(kCombineWaves * kWave), 0,
-                           stream, args, ws);
+        hipExtLaunchKernelGGL((combine_gather_kernel<T, U, 8>), dim3(blocks), dim3(kCombineWaves * kWave), 0,
+                              stream, timing.start, timing.stop, 0, args, ws);
     } else {
-        hipLaunchKernelGGL((combine_gather_kernel<T, U, 0>), dim3(blocks), dim3(kCombineWaves * kWave), 0,
-                           stream, args, ws);
+        hipExtLaunchKernelGGL((combine_gather_kernel<T, U, 0>), dim3(blocks), dim3(kCombineWaves * kWave), 0,
+                              stream, timing.start, timing.stop, 0, args, ws);
     }
     return hipGetLastError();
 }
 
 hipError_t launch_combine_gather(const CombArgs &args, const Workspace &ws, uint32_t in_dtype,
-                                 uint32_t out_dtype, uint32_t total_tokens, hipStream_t stream) {
+                                 uint32_t out_dtype, uint32_t total_tokens, hipStream_t stream, KernelTiming timing) {
     if (total_tokens == 0) return hipSuccess;
 #define A2A_COMBINE_CASE(IN_TAG, IN_T, OUT_TAG, OUT_T) \
     if (in_dtype == IN_TAG && out_dtype == OUT_TAG)    \
-        return launch_typed<IN_T, OUT_T>(args, ws, total_tokens, stream);
+        return launch_typed<IN_T, OUT_T>(args, ws, total_tokens, stream, timing);
     A2A_COMBINE_CASE(A2A_BF16, Bf16, A2A_BF16, Bf16)
     A2A_COMBINE_CASE(A2A_BF16, Bf16, A2A_F32, F32)
     A2A_COMBINE_CASE(A2A_BF16, Bf16, A2A_F16, F16)

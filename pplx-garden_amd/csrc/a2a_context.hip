@@ -36,6 +36,8 @@ struct a2a_ctx {
     uint32_t quantized = 0;        // mode of the last dispatch
 
     Staging staging;               // buffers and tables of the split calls
+
+    KernelTiming timing[2];        // one-shot events for the next pack / gather launch of a group call
 };
 
 namespace {
@@ -473,9 +475,11 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
     pa.hidden_dim_scale = c.hidden_dim_scale;
     pa.topk_magic = K > 1 ? (uint32_t)((0x100000000ull + K - 1) / K) : 0;
 
+    const KernelTiming pack_timing = ctx->timing[A2A_KERNEL_PACK];
+    ctx->timing[A2A_KERNEL_PACK] = KernelTiming();
     hipError_t e;
     if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && dispatch_small_fits(pa, ctx->ws, quantize != 0, tokens)) {
-        e = launch_dispatch_small(pa, fa, ctx->ws, quantize != 0, tokens, s);
+        e = launch_dispatch_small(pa, fa, ctx->ws, quantize != 0, tokens, s, pack_timing);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_small");
     } else if (c.flags & A2A_FLAG_SEPARATE_ROUTING) {
         if (fused_routing_pays(fa, G, blocks)) {
@@ -487,14 +491,14 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
             e = launch_finalize(fa, ctx->ws, s);
             if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
         }
-        e = launch_dispatch_push(pa, ctx->ws, quantize != 0, tokens, s);
+        e = launch_dispatch_push(pa, ctx->ws, quantize != 0, tokens, s, pack_timing);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_push");
     } else {
         // Two launches: chunk histograms that also add up the step's totals, then a pack whose
         // workgroups resolve their own rows from them.
         e = launch_route_accumulate(ra, ctx->ws, blocks, s);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist (accumulating)");
-        e = launch_dispatch_resolve(pa, fa, ctx->ws, quantize != 0, tokens, s);
+        e = launch_dispatch_resolve(pa, fa, ctx->ws, quantize != 0, tokens, s, pack_timing);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_resolve");
     }
 
@@ -558,9 +562,22 @@ int a2a_combine(a2a_ctx *ctx, const a2a_combine_args *args, uint32_t expert_y_dt
     ca.hidden_dim = c.hidden_dim;
     ca.accumulate = accumulate ? 1 : 0;
     DeviceGuard guard(c.device);
+    const KernelTiming gather_timing = ctx->timing[A2A_KERNEL_GATHER];
+    ctx->timing[A2A_KERNEL_GATHER] = KernelTiming();
     hipError_t e = launch_combine_gather(ca, ctx->ws, expert_y_dtype, c.out_dtype, tokens,
-                                         static_cast<hipStream_t>(stream));
+                                         static_cast<hipStream_t>(stream), gather_timing);
     if (e != hipSuccess) return hip_fail(ctx, e, "launch combine_gather");
+    return A2A_OK;
+}
+
+int a2a_ctx_time_next_kernel(a2a_ctx *ctx, uint32_t which, void *start_event, void *stop_event) {
+    if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (which != A2A_KERNEL_PACK && which != A2A_KERNEL_GATHER)
+        return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "unknown kernel %u", which);
+    if ((start_event == nullptr) != (stop_event == nullptr))
+        return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "pass both events or neither");
+    ctx->timing[which].start = static_cast<hipEvent_t>(start_event);
+    ctx->timing[which].stop = static_cast<hipEvent_t>(stop_event);
     return A2A_OK;
 }
 

@@ -595,15 +595,15 @@ __global__ __launch_bounds__(1024) void dispatch_resolve_kernel(const PushArgs a
 }
 
 hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool quantize,
-                                uint32_t total_tokens, hipStream_t stream) {
+                                uint32_t total_tokens, hipStream_t stream, KernelTiming timing) {
     if (total_tokens == 0) return hipSuccess;
     const uint32_t threads = push_threads(args, quantize);
     if (quantize) {
-        hipLaunchKernelGGL(dispatch_push_kernel<true>, dim3(total_tokens), dim3(threads), 0, stream,
-                           args, ws);
+        hipExtLaunchKernelGGL(dispatch_push_kernel<true>, dim3(total_tokens), dim3(threads), 0, stream,
+                              timing.start, timing.stop, 0, args, ws);
     } else {
-        hipLaunchKernelGGL(dispatch_push_kernel<false>, dim3(total_tokens), dim3(threads), 0,
-                           stream, args, ws);
+        hipExtLaunchKernelGGL(dispatch_push_kernel<false>, dim3(total_tokens), dim3(threads), 0, stream,
+                              timing.start, timing.stop, 0, args, ws);
     }
     return hipGetLastError();
 }
@@ -621,31 +621,35 @@ bool dispatch_small_fits(const PushArgs &args, const Workspace &ws, bool quantiz
 }
 
 hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
-                                 bool quantize, uint32_t total_tokens, hipStream_t stream) {
+                                 bool quantize, uint32_t total_tokens, hipStream_t stream, KernelTiming timing) {
     const uint32_t threads = push_threads(args, quantize);
     const uint32_t blocks = total_tokens + (fin.recv_mask != 0 ? ws.world : 0);
     if (blocks == 0) return hipSuccess;
     const size_t table_words = (((size_t)ws.num_groups + 3) * ws.num_experts + 1) & ~(size_t)1;
     const size_t lds = table_words * sizeof(uint32_t) + (size_t)total_tokens * sizeof(uint64_t);
     if (quantize) {
-        hipLaunchKernelGGL(dispatch_small_kernel<true>, dim3(blocks), dim3(threads), lds, stream, args, fin, ws);
+        hipExtLaunchKernelGGL(dispatch_small_kernel<true>, dim3(blocks), dim3(threads), lds, stream, timing.start,
+                              timing.stop, 0, args, fin, ws);
     } else {
-        hipLaunchKernelGGL(dispatch_small_kernel<false>, dim3(blocks), dim3(threads), lds, stream, args, fin, ws);
+        hipExtLaunchKernelGGL(dispatch_small_kernel<false>, dim3(blocks), dim3(threads), lds, stream, timing.start,
+                              timing.stop, 0, args, fin, ws);
     }
     return hipGetLastError();
 }
 
 hipError_t launch_dispatch_resolve(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
-                                   bool quantize, uint32_t total_tokens, hipStream_t stream) {
+                                   bool quantize, uint32_t total_tokens, hipStream_t stream, KernelTiming timing) {
     uint32_t threads = push_threads(args, quantize);
     if (threads < ws.experts_per_rank) {   // a receiver workgroup has one thread per local expert
         threads = (ws.experts_per_rank + kWave - 1) / kWave * kWave;
     }
     const uint32_t blocks = total_tokens + ws.world + ws.num_groups;
     if (quantize) {
-        hipLaunchKernelGGL(dispatch_resolve_kernel<true>, dim3(blocks), dim3(threads), 0, stream, args, fin, ws);
+        hipExtLaunchKernelGGL(dispatch_resolve_kernel<true>, dim3(blocks), dim3(threads), 0, stream, timing.start,
+                              timing.stop, 0, args, fin, ws);
     } else {
-        hipLaunchKernelGGL(dispatch_resolve_kernel<false>, dim3(blocks), dim3(threads), 0, stream, args, fin, ws);
+        hipExtLaunchKernelGGL(dispatch_resolve_kernel<false>, dim3(blocks), dim3(threads), 0, stream, timing.start,
+                              timing.stop, 0, args, fin, ws);
     }
     return hipGetLastError();
 }

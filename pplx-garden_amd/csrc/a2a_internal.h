@@ -4,6 +4,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include "a2a.h"
@@ -137,6 +138,13 @@ struct CombArgs {
     uint64_t staged_stride;
 };
 
+// Events a caller wants recorded when a kernel itself begins and ends (both
+// null: an ordinary launch).
+struct KernelTiming {
+    hipEvent_t start = nullptr;
+    hipEvent_t stop = nullptr;
+};
+
 // Launchers (defined next to their kernels); all return the hipError_t of the
 // launch.
 hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
@@ -147,12 +155,13 @@ hipError_t launch_route_accumulate(const RouteArgs &args, const Workspace &ws, u
 // Pack that resolves its rows from the chunk histograms and the step's totals, with the
 // receiver layout and the per-source tables computed by extra workgroups of the same launch.
 hipError_t launch_dispatch_resolve(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
-                                   bool quantize, uint32_t total_tokens, hipStream_t stream);
+                                   bool quantize, uint32_t total_tokens, hipStream_t stream,
+                                   KernelTiming timing = KernelTiming());
 hipError_t launch_finalize(const FinalizeArgs &args, const Workspace &ws, hipStream_t stream);
 hipError_t launch_route_fused(const RouteArgs &args, const FinalizeArgs &fin, const Workspace &ws,
                               hipStream_t stream);
 hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool quantize,
-                                uint32_t total_tokens, hipStream_t stream);
+                                uint32_t total_tokens, hipStream_t stream, KernelTiming timing = KernelTiming());
 // One-launch routing + pack for small steps: whether a step qualifies, and the launch.
 #ifndef A2A_SMALL_MAX_ENTRIES
 #define A2A_SMALL_MAX_ENTRIES 8192
@@ -162,9 +171,11 @@ hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool 
 #endif
 bool dispatch_small_fits(const PushArgs &args, const Workspace &ws, bool quantize, uint32_t total_tokens);
 hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
-                                 bool quantize, uint32_t total_tokens, hipStream_t stream);
+                                 bool quantize, uint32_t total_tokens, hipStream_t stream,
+                                 KernelTiming timing = KernelTiming());
 hipError_t launch_combine_gather(const CombArgs &args, const Workspace &ws, uint32_t in_dtype,
-                                 uint32_t out_dtype, uint32_t total_tokens, hipStream_t stream);
+                                 uint32_t out_dtype, uint32_t total_tokens, hipStream_t stream,
+                                 KernelTiming timing = KernelTiming());
 
 // Device-side: effective token count of a source (bound_m clamps num_tokens,
 // a2a_dispatch_send.cu:172).

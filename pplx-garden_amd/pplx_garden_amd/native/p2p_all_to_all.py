@@ -45,6 +45,8 @@ DEV_BAD_SLOT = 4
 
 FLAG_PREALLOC_STAGING = 1
 FLAG_SEPARATE_ROUTING = 2   # never take the one-launch paths of small steps
+KERNEL_PACK = 0
+KERNEL_GATHER = 1
 
 
 class A2AConfig(ctypes.Structure):
@@ -89,6 +91,7 @@ _SIGNATURES = {
     "a2a_ctx_destroy": (c_int, [c_void_p]),
     "a2a_ctx_status": (c_int, [c_void_p, c_void_p, POINTER(c_uint32)]),
     "a2a_ctx_read_table": (c_int, [c_void_p, c_uint32, c_uint32, POINTER(c_uint32), c_size_t, c_void_p]),
+    "a2a_ctx_time_next_kernel": (c_int, [c_void_p, c_uint32, c_void_p, c_void_p]),
     "a2a_dispatch_send": (c_int, [
         c_void_p, c_uint32, c_size_t, c_void_p, c_size_t, c_uint32, c_void_p, c_size_t, c_size_t,
         c_void_p, c_size_t, c_void_p, c_size_t, c_void_p, c_void_p]),
@@ -304,6 +307,13 @@ class AllToAllContext:
         buf = (c_uint32 * max(count, 1))()
         self._check(self._lib.a2a_ctx_read_table(self._handle, rank, which, buf, count, _ptr(stream)))
         return torch.tensor(list(buf[:count]), dtype=torch.int64)
+
+    def time_next_kernel(self, which: int, start_event: Optional[int], stop_event: Optional[int]) -> None:
+        """Have the next group dispatch (`KERNEL_PACK`) or combine (`KERNEL_GATHER`) record the two
+        events (raw `hipEvent_t` handles, e.g. `torch.cuda.Event.cuda_event`) at the start and end of
+        its bandwidth kernel itself."""
+        self._require_open()
+        self._check(self._lib.a2a_ctx_time_next_kernel(self._handle, which, _ptr(start_event), _ptr(stop_event)))
 
     def dispatch_token_stride(self) -> int:
         return int(self._lib.a2a_dispatch_token_stride(ctypes.byref(self._config)))

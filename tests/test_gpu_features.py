@@ -307,3 +307,62 @@ def test_calls_can_be_captured_in_a_hip_graph(case, sources):
     finally:
         for op in ops:
             op.destroy()
+
+
+def test_kernel_own_events():
+    """a2a_ctx_time_next_kernel: the pack and the gather of the next group calls record the caller's
+    events at their own start and end; the request is one-shot."""
+    case = C1
+    world = make_world(case, "all")
+    rows = rows_needed(case, world)
+    N, Le, H, Hs = case.world_size, case.experts_per_rank, case.hidden_dim, case.hidden_dim_scale
+    _, ops = make_ops(case, DEV)
+    try:
+        t = []
+        gen = torch.Generator().manual_seed(4)
+        for r, rd in enumerate(world):
+            t.append(dict(x=rd.x.to(DEV), idx=rd.indices_u32.to(DEV), w=rd.weights.to(DEV),
+                          n=torch.zeros(Le, dtype=torch.int32, device=DEV),
+                          ox=torch.zeros((rows, H), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn),
+                          os=torch.zeros((rows, Hs), dtype=torch.float32, device=DEV),
+                          y=torch.randn((rows, H), generator=gen).to(torch.bfloat16).to(DEV),
+                          o=torch.zeros((rd.x.shape[0], H), dtype=torch.bfloat16, device=DEV)))
+
+        def step():
+            for r in range(N):
+                ops[r].dispatch(out_expert_num_tokens=t[r]["n"], out_expert_x=t[r]["ox"], out_expert_x_scale=t[r]["os"],
+                                dp_x=t[r]["x"], dp_x_scale=None, indices=t[r]["idx"], weights=t[r]["w"])
+            for r in range(N):
+                ops[r].combine(out_tokens=t[r]["o"], indices=t[r]["idx"], weights=t[r]["w"], expert_y=t[r]["y"])
+
+        step()
+        torch.cuda.synchronize(DEV)
+        first = [a["o"].clone() for a in t]
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(6)]
+        for e in ev:
+            e.record()                       # gives the event its handle
+        torch.cuda.synchronize(DEV)
+        ctx = ops[0].context
+        ctx.time_next_kernel(native.KERNEL_PACK, ev[0].cuda_event, ev[1].cuda_event)
+        ctx.time_next_kernel(native.KERNEL_GATHER, ev[2].cuda_event, ev[3].cuda_event)
+        ev[4].record()
+        step()
+        ev[5].record()
+        torch.cuda.synchronize(DEV)
+        pack_ms, gather_ms, both_ms = ev[0].elapsed_time(ev[1]), ev[2].elapsed_time(ev[3]), ev[4].elapsed_time(ev[5])
+        assert 0.0 < pack_ms < both_ms and 0.0 < gather_ms < both_ms
+        assert ev[1].elapsed_time(ev[2]) >= 0.0          # the pack ends before the gather begins
+        for a, want in zip(t, first):
+            assert torch.equal(a["o"].view(torch.int16), want.view(torch.int16))
+        # one-shot: a further step leaves the events alone
+        step()
+        torch.cuda.synchronize(DEV)
+        assert ev[0].elapsed_time(ev[1]) == pack_ms and ev[2].elapsed_time(ev[3]) == gather_ms
+        with pytest.raises(RuntimeError, match="both events or neither"):
+            ctx.time_next_kernel(native.KERNEL_PACK, ev[0].cuda_event, None)
+        with pytest.raises(RuntimeError, match="unknown kernel"):
+            ctx.time_next_kernel(7, None, None)
+        assert ctx.status() == 0
+    finally:
+        for op in ops:
+            op.destroy()
