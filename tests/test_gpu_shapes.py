@@ -24,6 +24,8 @@ SHAPES = [
     Case("world_32", 64, 256, 64, 32, 4, 7008, expert_padding=8, node_size=8),
     Case("world_1", 100, 512, 7, 1, 3, 7009, expert_padding=16),
     Case("several_chunks", 700, 256, 24, 4, 8, 7010, routing="zipf", zipf_s=1.5),   # 5600 entries: 6 chunks
+    Case("many_chunks", 600, 128, 64, 2, 64, 7012),                        # 38 400 entries of one source: 38 chunks
+    Case("wide_ranks", 900, 128, 90, 2, 8, 7013, expert_padding=4),        # Le = 45 experts per rank, two-launch dispatch
 ]
 
 
