@@ -182,8 +182,10 @@ def time_workload(wl: Workload, steps: int, warmup: int, event_every: int = 8, k
     return wall_s, disp, comb, both, pack, gather
 
 
-def cpu_baseline(case, rd, reps: int):
-    """The oracle's C restatement on the same batch, one thread; best of `reps`."""
+def cpu_baseline(case, rd, reps: int, threads: int = 1):
+    """The oracle's C restatement on the same batch; best of `reps`.  Returns seconds per step and the
+    seconds of its routing part (histogram, ranks, receiver layout: what the reference does on one host
+    thread, a2a_worker.rs:526-703)."""
     import numpy as np
     from a2a_cases import bf16_codes
     from a2a_harness import rows_needed
@@ -201,15 +203,21 @@ def cpu_baseline(case, rd, reps: int):
     idx = [w.indices.numpy() for w in world]
     xs = [bf16_codes(w.x) for w in world]
     ws = [w.weights.numpy() for w in world]
-    best = None
-    for _ in range(reps):
-        t0 = time.perf_counter()
-        cw.route_all(idx)
-        cw.dispatch(xs)
-        cw.combine(ws)
-        dt = time.perf_counter() - t0
-        best = dt if best is None else min(best, dt)
-    return best
+    best = route_best = None
+    c_oracle.set_threads(threads)
+    try:
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            cw.route_all(idx)
+            t1 = time.perf_counter()
+            cw.dispatch(xs)
+            cw.combine(ws)
+            dt = time.perf_counter() - t0
+            best = dt if best is None else min(best, dt)
+            route_best = t1 - t0 if route_best is None else min(route_best, t1 - t0)
+    finally:
+        c_oracle.set_threads(1)
+    return best, route_best
 
 
 def main() -> int:
@@ -322,15 +330,23 @@ def main() -> int:
                     "launches record themselves",
         }
 
-    cpu = None
+    cpu = cpu_more = None
     if args.cpu_reps > 0:
-        dt = cpu_baseline(case, cpu_rd, args.cpu_reps)
+        dt, route_dt = cpu_baseline(case, cpu_rd, args.cpu_reps)
         cpu = {
             "value": round((d_bytes + c_bytes) / dt / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
             "us_per_step": round(dt * 1e6, 1),
             "sample": f"the full {case.num_tokens}-token batch (routing pass, quantising dispatch, combine), "
                       f"best of {args.cpu_reps} runs of the oracle's C restatement, one thread of "
                       f"{os.cpu_count()} host cores",
+        }
+        cores = min(16, os.cpu_count() or 1)
+        dt_all, _ = cpu_baseline(case, cpu_rd, args.cpu_reps, threads=cores)
+        cpu_more = {
+            "routing_only_us_one_thread": round(route_dt * 1e6, 1),
+            "all_cores": {"value": round((d_bytes + c_bytes) / dt_all / 1e9, 3), "unit": "GB/s", "cores": cores,
+                          "us_per_step": round(dt_all * 1e6, 1),
+                          "note": "same code, tokens split over OpenMP threads; routing stays on one thread"},
         }
 
     line = {
@@ -377,6 +393,7 @@ def main() -> int:
         "roofline": dominant,
         "roofline_other": other,
         "cpu_baseline": cpu,
+        "cpu_baseline_more": cpu_more,
     }
     print(json.dumps(line, ensure_ascii=False))
     return 0

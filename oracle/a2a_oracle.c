@@ -3,7 +3,8 @@
  * it is the checker of the parity tests and the timed CPU baseline of the
  * benchmark, never part of the shipped library.
  *
- * Scalar, single-threaded, written from the algorithm of the reference (cited
+ * Scalar code, one thread unless oracle_set_threads asks for more (tokens are
+ * then split over OpenMP threads), written from the algorithm of the reference (cited
  * per function, paths relative to the reference checkout).  Choices where the
  * reference leaves something open are the same as in a2a_oracle.py: stable
  * (token, k) order inside an expert, and the bf16 -> fp8 e4m3 quantiser defined
@@ -11,9 +12,15 @@
  * uses arithmetic, so that the two pin each other.
  */
 #include <math.h>
+#include <omp.h>
 #include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
+
+/* Threads used by oracle_dispatch_rank and oracle_combine_rank (tokens are split
+ * over them; results do not depend on the number).  1 = the scalar port. */
+static int g_threads = 1;
+void oracle_set_threads(int n) { g_threads = n > 1 ? n : 1; }
 
 static inline float bf16_to_f32(uint16_t v) {
     uint32_t b = (uint32_t)v << 16;
@@ -163,13 +170,12 @@ void oracle_quantize_row(const uint16_t *x, uint32_t H, uint8_t *q, float *scale
  * out_x[r] / out_scale[r] are the receivers' buffers (row strides H and Hs).
  * `qrow` / `srow` are scratch of H bytes / Hs floats.
  */
-void oracle_dispatch_rank(const uint16_t *x, size_t x_stride_elems, const int32_t *indices,
-                          size_t indices_stride, uint32_t num_tokens, uint32_t H, uint32_t K,
-                          uint32_t Le, const uint32_t *token_offset, const uint32_t *base_g,
-                          uint8_t *const *out_x, float *const *out_scale, uint8_t *qrow,
-                          float *srow) {
+static void dispatch_tokens(const uint16_t *x, size_t x_stride_elems, const int32_t *indices,
+                            size_t indices_stride, uint32_t t0, uint32_t t1, uint32_t H, uint32_t K,
+                            uint32_t Le, const uint32_t *token_offset, const uint32_t *base_g,
+                            uint8_t *const *out_x, float *const *out_scale, uint8_t *qrow, float *srow) {
     const uint32_t Hs = H / 128;
-    for (uint32_t t = 0; t < num_tokens; ++t) {
+    for (uint32_t t = t0; t < t1; ++t) {
         oracle_quantize_row(x + (size_t)t * x_stride_elems, H, qrow, srow);
         for (uint32_t k = 0; k < K; ++k) {
             const uint32_t e = (uint32_t)indices[(size_t)t * indices_stride + k];
@@ -181,18 +187,45 @@ void oracle_dispatch_rank(const uint16_t *x, size_t x_stride_elems, const int32_
     }
 }
 
+void oracle_dispatch_rank(const uint16_t *x, size_t x_stride_elems, const int32_t *indices,
+                          size_t indices_stride, uint32_t num_tokens, uint32_t H, uint32_t K,
+                          uint32_t Le, const uint32_t *token_offset, const uint32_t *base_g,
+                          uint8_t *const *out_x, float *const *out_scale, uint8_t *qrow,
+                          float *srow) {
+    if (g_threads <= 1) {
+        dispatch_tokens(x, x_stride_elems, indices, indices_stride, 0, num_tokens, H, K, Le, token_offset, base_g,
+                        out_x, out_scale, qrow, srow);
+        return;
+    }
+    /* tokens are independent: split them over the threads, each with scratch of its own */
+#pragma omp parallel num_threads(g_threads)
+    {
+        uint8_t *q = (uint8_t *)malloc(H);
+        float *sc = (float *)malloc((size_t)(H / 128 + 1) * sizeof(float));
+        const uint32_t n = (uint32_t)omp_get_num_threads(), i = (uint32_t)omp_get_thread_num();
+        const uint32_t per = (num_tokens + n - 1) / n;
+        const uint32_t t0 = i * per < num_tokens ? i * per : num_tokens;
+        const uint32_t t1 = t0 + per < num_tokens ? t0 + per : num_tokens;
+        if (q != NULL && sc != NULL)
+            dispatch_tokens(x, x_stride_elems, indices, indices_stride, t0, t1, H, K, Le, token_offset, base_g,
+                            out_x, out_scale, q, sc);
+        free(q);
+        free(sc);
+    }
+}
+
 /*
  * combine for one source rank: out[t] = (accumulate ? out[t] : 0) + sum_k
  * w[t,k] * y(t,k), one fused multiply-add per k in float, k ascending, one
  * rounding to bf16 (a2a_combine_recv.cu:131-146, combine_utils.cuh:108-114).
  * expert_y[r] are the receivers' bf16 rows (row stride H).
  */
-void oracle_combine_rank(uint16_t *out, size_t out_stride_elems, const int32_t *indices,
-                         size_t indices_stride, const float *weights, size_t weights_stride,
-                         uint32_t num_tokens, uint32_t H, uint32_t K, uint32_t Le,
-                         const uint32_t *token_offset, const uint32_t *base_g,
-                         const uint16_t *const *expert_y, int accumulate, float *acc) {
-    for (uint32_t t = 0; t < num_tokens; ++t) {
+static void combine_tokens(uint16_t *out, size_t out_stride_elems, const int32_t *indices,
+                           size_t indices_stride, const float *weights, size_t weights_stride,
+                           uint32_t t0, uint32_t t1, uint32_t H, uint32_t K, uint32_t Le,
+                           const uint32_t *token_offset, const uint32_t *base_g,
+                           const uint16_t *const *expert_y, int accumulate, float *acc) {
+    for (uint32_t t = t0; t < t1; ++t) {
         uint16_t *o = out + (size_t)t * out_stride_elems;
         for (uint32_t h = 0; h < H; ++h) acc[h] = accumulate ? bf16_to_f32(o[h]) : 0.0f;
         for (uint32_t k = 0; k < K; ++k) {
@@ -203,6 +236,30 @@ void oracle_combine_rank(uint16_t *out, size_t out_stride_elems, const int32_t *
             for (uint32_t h = 0; h < H; ++h) acc[h] = fmaf(w, bf16_to_f32(y[h]), acc[h]);
         }
         for (uint32_t h = 0; h < H; ++h) o[h] = f32_to_bf16(acc[h]);
+    }
+}
+
+void oracle_combine_rank(uint16_t *out, size_t out_stride_elems, const int32_t *indices,
+                         size_t indices_stride, const float *weights, size_t weights_stride,
+                         uint32_t num_tokens, uint32_t H, uint32_t K, uint32_t Le,
+                         const uint32_t *token_offset, const uint32_t *base_g,
+                         const uint16_t *const *expert_y, int accumulate, float *acc) {
+    if (g_threads <= 1) {
+        combine_tokens(out, out_stride_elems, indices, indices_stride, weights, weights_stride, 0, num_tokens, H, K,
+                       Le, token_offset, base_g, expert_y, accumulate, acc);
+        return;
+    }
+#pragma omp parallel num_threads(g_threads)
+    {
+        float *a = (float *)malloc((size_t)H * sizeof(float));
+        const uint32_t n = (uint32_t)omp_get_num_threads(), i = (uint32_t)omp_get_thread_num();
+        const uint32_t per = (num_tokens + n - 1) / n;
+        const uint32_t t0 = i * per < num_tokens ? i * per : num_tokens;
+        const uint32_t t1 = t0 + per < num_tokens ? t0 + per : num_tokens;
+        if (a != NULL)
+            combine_tokens(out, out_stride_elems, indices, indices_stride, weights, weights_stride, t0, t1, H, K, Le,
+                           token_offset, base_g, expert_y, accumulate, a);
+        free(a);
     }
 }
 

@@ -32,6 +32,8 @@ def lib() -> ctypes.CDLL:
         l.oracle_combine_rank.argtypes = [c_void_p, c_size_t, c_void_p, c_size_t, c_void_p, c_size_t, c_uint32,
                                           c_uint32, c_uint32, c_uint32, c_void_p, c_void_p, c_void_p, c_int, c_void_p]
         l.oracle_act_rows.argtypes = [c_void_p, c_void_p, c_size_t, c_uint32, c_void_p]
+        l.oracle_set_threads.argtypes = [ctypes.c_int]
+        l.oracle_set_threads.restype = None
         _lib = l
     return _lib
 
@@ -81,8 +83,13 @@ def quantize(x_codes: np.ndarray):
     return q, s
 
 
+def set_threads(n: int) -> None:
+    """Threads the C oracle splits the tokens of a dispatch or combine over (1 = the scalar port)."""
+    lib().oracle_set_threads(int(n))
+
+
 class CWorld:
-    """dispatch + combine of a whole group with the C oracle (single thread)."""
+    """dispatch + combine of a whole group with the C oracle (one thread unless set_threads says more)."""
 
     def __init__(self, num_experts, world_size, node_size, expert_padding, hidden_dim, topk, rows):
         self.E, self.N, self.node, self.pad = num_experts, world_size, node_size, expert_padding

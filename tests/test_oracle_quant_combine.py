@@ -137,3 +137,34 @@ def test_combine_accumulate_and_bound_m():
     a = oracle.bf16_to_f32(accum[1]).astype(np.float64)
     p = oracle.bf16_to_f32(plain[1]).astype(np.float64) + oracle.bf16_to_f32(prev[1]).astype(np.float64)
     np.testing.assert_allclose(a, p, rtol=2 ** -6, atol=2 ** -6)
+
+
+def test_c_oracle_with_threads_equals_scalar():
+    """The C oracle splits tokens over threads for the all-cores CPU baseline; tokens are independent,
+    so the bytes must not depend on the number of threads."""
+    import c_oracle
+    from a2a_cases import C0, bf16_codes, make_world
+    from a2a_harness import rows_needed
+    case = C0
+    world = make_world(case, "ragged")
+    rows = rows_needed(case, world)
+    results = []
+    for threads in (1, 3, 8):
+        c_oracle.set_threads(threads)
+        try:
+            cw = c_oracle.CWorld(case.num_experts, case.world_size, case.world_size, case.expert_padding,
+                                 case.hidden_dim, case.topk, rows)
+            cw.route_all([rd.indices.numpy() for rd in world])
+            cw.dispatch([bf16_codes(rd.x) for rd in world])
+            cw.act()
+            outs = cw.combine([rd.weights.numpy() for rd in world])
+            results.append(([a.copy() for a in cw.out_x], [a.copy() for a in cw.out_s], outs))
+        finally:
+            c_oracle.set_threads(1)
+    for other in results[1:]:
+        for a, b in zip(results[0][0], other[0]):
+            np.testing.assert_array_equal(a, b)
+        for a, b in zip(results[0][1], other[1]):
+            np.testing.assert_array_equal(a.view(np.uint32), b.view(np.uint32))
+        for a, b in zip(results[0][2], other[2]):
+            np.testing.assert_array_equal(a, b)
