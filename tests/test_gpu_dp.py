@@ -16,6 +16,9 @@ CONFIGS = [
     RefConfig("dp4_one_node", 8, 4, 40, 16, 128, None, 3, F32, F32, None),
     RefConfig("dp2_fp8_scales", 4, 2, 96, 32, 1024, 8, 8, FP8, BF16, F32, node_size=2),
     RefConfig("dp8_single_group", 8, 8, 33, 24, 256, None, 6, BF16, BF16, None),
+    # large enough for the two-launch dispatch (4 groups x 700 tokens x 8 = 22 400 entries)
+    RefConfig("dp2_two_launch", 8, 2, 700, 32, 256, None, 8, BF16, BF16, None, expert_padding=4, node_size=4),
+    RefConfig("dp4_two_launch_fp8", 8, 4, 1300, 48, 512, 4, 8, FP8, BF16, F32, node_size=8),
 ]
 
 
