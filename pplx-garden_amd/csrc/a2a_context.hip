@@ -308,6 +308,8 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
     const size_t o_chunk_counts = carve((size_t)N * ws.nb_max * E * sizeof(uint32_t));
     const size_t o_totals = carve(2 * ((size_t)ws.num_groups + 1) * E * sizeof(uint32_t));
     const size_t o_turn = carve(2 * sizeof(uint32_t));
+    const size_t o_send_totals = carve(2 * ((size_t)E + N) * sizeof(uint32_t));
+    const size_t o_send_turn = carve(2 * sizeof(uint32_t));
     ctx->arena_bytes = off;
     e = hipMalloc(&ctx->arena, ctx->arena_bytes);
     if (e != hipSuccess) {
@@ -338,6 +340,8 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
     ws.chunk_counts = reinterpret_cast<uint32_t *>(base + o_chunk_counts);
     ws.totals = reinterpret_cast<uint32_t *>(base + o_totals);
     ws.turn = reinterpret_cast<uint32_t *>(base + o_turn);
+    ws.send_totals = reinterpret_cast<uint32_t *>(base + o_send_totals);
+    ws.send_turn = reinterpret_cast<uint32_t *>(base + o_send_turn);
     {
         // i-th source each receiver lays out, and which sources come before which: fixed for the
         // life of the context
@@ -700,17 +704,26 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
         fa.fold_mask = 1u << group;
         fa.valid_mask = ctx->sent_mask | (1u << group);
         fa.recv_mask = 0;
-        if (fused_routing_pays(fa, c.world_size / c.dp_size, nb)) {
-            e = launch_route_fused(ra, fa, ctx->ws, s);
-            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
+        if (T != 0 && !(c.flags & A2A_FLAG_SEPARATE_ROUTING)) {
+            // two launches: chunk histograms that also add up the sender's totals, then a staging
+            // launch whose workgroups resolve their own positions from them
+            e = launch_route_accumulate(ra, ctx->ws, nb, s, true);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist (accumulating, send)");
+            e = launch_stage_send_resolve(sa, ctx->ws, ctx->staging, quantize != 0, s);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send_resolve");
         } else {
-            e = launch_route(ra, ctx->ws, nb, s);
-            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
-            e = launch_finalize(fa, ctx->ws, s);
-            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+            if (fused_routing_pays(fa, c.world_size / c.dp_size, nb)) {
+                e = launch_route_fused(ra, fa, ctx->ws, s);
+                if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
+            } else {
+                e = launch_route(ra, ctx->ws, nb, s);
+                if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
+                e = launch_finalize(fa, ctx->ws, s);
+                if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+            }
+            e = launch_stage_send(sa, ctx->ws, ctx->staging, quantize != 0, s);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send");
         }
-        e = launch_stage_send(sa, ctx->ws, ctx->staging, quantize != 0, s);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send");
     }
 
     ctx->sent_mask |= 1u << group;

@@ -39,6 +39,9 @@ struct Workspace {
                                //                accumulated by the routing launch of large group steps; two copies
                                //                used in turn
     uint32_t *turn;            // [2]            [0] copy the next routing launch fills, [1] copy the current step uses
+    uint32_t *send_totals;     // [2][E + N]     the same for the send of a split call: counts of ONE source per expert,
+                               //                then per owning rank; two copies used in turn
+    uint32_t *send_turn;       // [2]            as `turn`, for send_totals
     uint32_t max_tk;           // max_num_tokens * K
     uint32_t nb_max;           // ceil(max_tk / kRouteBlock)
     uint32_t world;            // N logical ranks (receivers)
@@ -149,9 +152,10 @@ struct KernelTiming {
 // launch.
 hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
                         hipStream_t stream);
-// The same, and every chunk adds its counts to the step's totals (large group steps).
+// The same, and every chunk adds its counts to the step's totals (large group steps), or to
+// the totals of the one source of a split send (`for_send`).
 hipError_t launch_route_accumulate(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
-                                   hipStream_t stream);
+                                   hipStream_t stream, bool for_send = false);
 // Pack that resolves its rows from the chunk histograms and the step's totals, with the
 // receiver layout and the per-source tables computed by extra workgroups of the same launch.
 hipError_t launch_dispatch_resolve(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,

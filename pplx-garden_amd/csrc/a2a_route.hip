@@ -208,26 +208,31 @@ __device__ uint32_t rank_chunk(const RouteSrc &src, const Workspace &ws, uint32_
 
 }  // namespace
 
-// ACCUM: the launch also adds every chunk's counts to the step's totals (per
-// source and expert, and per expert), which the pack of a large group step
-// resolves its rows from.  The totals exist twice and are used in turn, so that
-// this launch can clear the copy of the NEXT step while it fills its own:
-// turn[0] says which copy to fill (flipped by the pack launch that follows),
-// turn[1] tells that pack which copy this launch filled.  All of it lives on
-// the device, so a recorded sequence of launches can be replayed.
-template <bool ACCUM>
+// MODE 1 (group steps): the launch also adds every chunk's counts to the step's
+// totals (per source and expert, and per expert), which the pack of a large
+// group step resolves its rows from.  MODE 2 (the send of a split call, one
+// source per launch): to that source's totals per expert and per owning rank,
+// which the staging launch resolves its positions from.  The totals exist twice
+// and are used in turn, so that this launch can clear the copy of the NEXT step
+// while it fills its own: turn[0] says which copy to fill (flipped by the launch
+// that follows and consumes them), turn[1] tells that launch which copy this
+// one filled.  All of it lives on the device, so a recorded sequence of launches
+// can be replayed.
+template <int MODE>
 __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs args,
                                                                  const Workspace ws) {
     __shared__ uint16_t wave_hist[kRouteWaves][A2A_MAX_EXPERTS];
     const uint32_t G = ws.num_groups, E = ws.num_experts;
-    const uint32_t words = (G + 1) * E;
+    const uint32_t words = MODE == 2 ? E + ws.world : (G + 1) * E;
+    uint32_t *totals = MODE == 2 ? ws.send_totals : ws.totals;
+    uint32_t *turn = MODE == 2 ? ws.send_turn : ws.turn;
     uint32_t fill = 0;
-    if constexpr (ACCUM) {
-        fill = ws.turn[0] & 1u;
+    if constexpr (MODE != 0) {
+        fill = turn[0] & 1u;
         if (blockIdx.x == 0) {
-            uint32_t *next = ws.totals + (size_t)(fill ^ 1u) * words;
+            uint32_t *next = totals + (size_t)(fill ^ 1u) * words;
             for (uint32_t i = threadIdx.x; i < words; i += kRouteBlock) next[i] = 0;
-            if (threadIdx.x == 0) ws.turn[1] = fill;
+            if (threadIdx.x == 0) turn[1] = fill;
         }
         if (blockIdx.x >= args.block_start[G]) return;   // a step without entries: only the duties above
     }
@@ -236,16 +241,33 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
     while (g + 1 < G && blockIdx.x >= args.block_start[g + 1]) ++g;
     const uint32_t chunk = blockIdx.x - args.block_start[g];
     const uint32_t count = rank_chunk(args.src[g], ws, g, chunk, wave_hist);
+    uint32_t *mine = totals + (size_t)fill * words;
     if (threadIdx.x < E) {
-        if constexpr (!ACCUM) ws.block_hist[((size_t)g * ws.nb_max + chunk) * E + threadIdx.x] = count;
-        if constexpr (ACCUM) {
-            // the pack reads all chunks of ONE expert, and all sources of one expert: keep those together
+        if constexpr (MODE == 0) {
+            ws.block_hist[((size_t)g * ws.nb_max + chunk) * E + threadIdx.x] = count;
+        } else {
+            // the consumer reads all chunks of ONE expert, and all sources of one expert: keep those together
             ws.chunk_counts[((size_t)g * E + threadIdx.x) * ws.nb_max + chunk] = count;
             if (count != 0) {
-                uint32_t *mine = ws.totals + (size_t)fill * words;
-                atomicAdd(&mine[threadIdx.x * G + g], count);
-                atomicAdd(&mine[G * E + threadIdx.x], count);
+                if constexpr (MODE == 1) {
+                    atomicAdd(&mine[threadIdx.x * G + g], count);
+                    atomicAdd(&mine[G * E + threadIdx.x], count);
+                } else {
+                    atomicAdd(&mine[threadIdx.x], count);
+                }
             }
+        }
+    }
+    if constexpr (MODE == 2) {
+        // Per owning rank: the experts of a rank are added up in LDS first, so that one atomic per
+        // rank and chunk reaches memory (one per expert would pile hundreds onto a few addresses).
+        __shared__ uint32_t rank_sum[kMaxWorld];
+        if (threadIdx.x < ws.world) rank_sum[threadIdx.x] = 0;
+        __syncthreads();
+        if (threadIdx.x < E && count != 0) atomicAdd(&rank_sum[owner_of_expert(ws, threadIdx.x)], count);
+        __syncthreads();
+        if (threadIdx.x < ws.world && rank_sum[threadIdx.x] != 0) {
+            atomicAdd(&mine[E + threadIdx.x], rank_sum[threadIdx.x]);
         }
     }
 }
@@ -401,15 +423,19 @@ __global__ __launch_bounds__(kRouteBlock) void route_finalize_kernel(const Final
 hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
                         hipStream_t stream) {
     if (total_blocks == 0) return hipSuccess;
-    hipLaunchKernelGGL(route_hist_kernel<false>, dim3(total_blocks), dim3(kRouteBlock), 0, stream, args, ws);
+    hipLaunchKernelGGL(route_hist_kernel<0>, dim3(total_blocks), dim3(kRouteBlock), 0, stream, args, ws);
     return hipGetLastError();
 }
 
 hipError_t launch_route_accumulate(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
-                                   hipStream_t stream) {
+                                   hipStream_t stream, bool for_send) {
     // at least one workgroup: the launch also hands over the totals between steps
-    hipLaunchKernelGGL(route_hist_kernel<true>, dim3(total_blocks != 0 ? total_blocks : 1), dim3(kRouteBlock), 0,
-                       stream, args, ws);
+    const dim3 grid(total_blocks != 0 ? total_blocks : 1);
+    if (for_send) {
+        hipLaunchKernelGGL(route_hist_kernel<2>, grid, dim3(kRouteBlock), 0, stream, args, ws);
+    } else {
+        hipLaunchKernelGGL(route_hist_kernel<1>, grid, dim3(kRouteBlock), 0, stream, args, ws);
+    }
     return hipGetLastError();
 }
 

@@ -87,6 +87,9 @@ hipError_t launch_stage_send(const StageSendArgs &args, const Workspace &ws, con
 bool stage_send_small_fits(const StageSendArgs &args, const Workspace &ws);
 hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                                    bool quantize, hipStream_t stream);
+// The send of a large step after launch_route_accumulate(..., for_send = true).
+hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace &ws, const Staging &st,
+                                     bool quantize, hipStream_t stream);
 hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st,
                              hipStream_t stream);
 hipError_t launch_combine_send(const CombineSendArgs &args, const Workspace &ws, const Staging &st,

@@ -191,6 +191,105 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
     stage_row<QUANT>(args, st, g, token);
 }
 
+// The send of a large step, after a routing launch that left the chunk counts,
+// the in-chunk rank of every entry and the sender's totals per expert and per
+// owning rank.  No launch in between scans anything: wavefront 0 of a token
+// workgroup finds the position of each of its K copies in the sender's
+// expert-sorted order itself, eight lanes per route, from three short sums
+// (copies of the same expert in earlier chunks; copies for the ranks before
+// the expert's owner; copies for the owner's experts before it), while the
+// other wavefronts stage the row.  Workgroup 0 is not a token: it publishes the
+// sender's counts and their scan (a2a_dispatch_send.cu:199-204,236-242) and
+// hands the totals over to the next send.
+template <bool QUANT>
+__global__ __launch_bounds__(1024) void stage_send_resolve_kernel(const StageSendArgs args, const Workspace ws,
+                                                                  const Staging st) {
+    __shared__ uint32_t scratch[kRouteWaves];
+    __shared__ uint32_t s_carry;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const uint32_t E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
+    const uint32_t g = args.rank / ws.dp_size;
+    const uint32_t use = ws.send_turn[1] & 1u;
+    const uint32_t *per_expert = ws.send_totals + (size_t)use * (E + ws.world);   // [E]
+    const uint32_t *per_rank = per_expert + E;                                     // [N]
+
+    if (blockIdx.x == 0) {
+        uint32_t carry = 0;
+        for (uint32_t e0 = 0; e0 < E; e0 += blockDim.x) {
+            const uint32_t e = e0 + tid;
+            const uint32_t c = e < E ? per_expert[e] : 0;
+            const uint32_t incl = carry + block_inclusive_scan(c, scratch);
+            if (e < E) {
+                ws.num_routed[g * E + e] = c;
+                ws.expert_offsets[g * E + e] = incl;
+            }
+            if (e0 + blockDim.x < E) {   // uniform: another round follows
+                if (tid == blockDim.x - 1) s_carry = incl;
+                __syncthreads();
+                carry = s_carry;
+            }
+        }
+        if (tid == 0) ws.send_turn[0] = use ^ 1u;
+        return;
+    }
+
+    const uint32_t token = blockIdx.x - 1;
+    const PushSrc &src = args.src;
+    if (token >= effective_tokens(src.bound_m, src.num_tokens)) return;
+
+    if (wave == 0) {
+        const uint32_t *counts = ws.chunk_counts + (size_t)g * E * ws.nb_max;   // [E][nb_max]
+        const uint32_t part = lane & 7, route = lane >> 3;
+        for (uint32_t k0 = 0; k0 < K; k0 += 8) {
+            const uint32_t k = k0 + route;
+            const bool in = k < K;
+            const uint32_t kk = in ? k : 0;   // a lane without a route reads route 0 and is dropped below
+            const uint32_t id = (uint32_t)src.indices[(size_t)token * src.indices_stride + kk];
+            const uint32_t local = ws.local_rank[(size_t)g * ws.max_tk + token * K + kk];
+            const bool live = in && id < E;
+            const uint32_t e = live ? id : 0;
+            const uint32_t upto = live ? (token * K + k) / kRouteBlock : 0;   // chunk of this entry
+            const uint32_t r = owner_of_expert(ws, e);
+            const uint32_t le = live ? e - r * Le : 0;
+            const uint32_t ranks_before = live ? r : 0;
+            // four terms of each sum per lane without a branch (clamped index, masked value)
+            uint32_t v_chunk[4], v_rank[4], v_expert[4];
+#pragma unroll
+            for (uint32_t i = 0; i < 4; ++i) {
+                const uint32_t n = part + 8 * i;
+                v_chunk[i] = counts[(size_t)e * ws.nb_max + (n < upto ? n : 0)];
+                v_rank[i] = per_rank[n < ranks_before ? n : 0];
+                v_expert[i] = per_expert[r * Le + (n < le ? n : 0)];
+            }
+            uint32_t earlier = 0, excl = 0;
+#pragma unroll
+            for (uint32_t i = 0; i < 4; ++i) {
+                const uint32_t n = part + 8 * i;
+                earlier += n < upto ? v_chunk[i] : 0;
+                excl += n < ranks_before ? v_rank[i] : 0;
+                excl += n < le ? v_expert[i] : 0;
+            }
+            // longer sums (more than 32 chunks, more than 32 experts in a rank)
+            for (uint32_t c = 32 + part; c < upto; c += 8) earlier += counts[(size_t)e * ws.nb_max + c];
+            for (uint32_t q = 32 + part; q < le; q += 8) excl += per_expert[r * Le + q];
+            earlier = group8_sum(earlier);
+            excl = group8_sum(excl);
+            if (part == 0 && in) {
+                uint32_t toff = 0;
+                if (live) {
+                    toff = earlier + local;
+                    // position of the copy (a2a_dispatch_send.cu:54)
+                    st.pos_token[(size_t)g * ws.max_tk + excl + toff] = token;
+                }
+                ws.token_offset[(size_t)g * ws.max_tk + token * K + k] = toff;
+            }
+        }
+    }
+    stage_row<QUANT>(args, st, g, token);
+}
+
 // A team of `team` threads (one or more whole wavefronts) copies a row of
 // `num_chunks` 16-byte pieces: eight loads per thread in flight, non-temporal
 // both ways (rows are read once and written once).
@@ -551,6 +650,18 @@ hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &w
     } else {
         hipLaunchKernelGGL(stage_send_small_kernel<false>, dim3(args.src.num_tokens), dim3(threads), lds, stream,
                            args, ws, st);
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace &ws, const Staging &st,
+                                     bool quantize, hipStream_t stream) {
+    const uint32_t threads = block_for_chunks(quantize ? args.hidden_dim / 16 : args.row_bytes / 16);
+    const uint32_t blocks = args.src.num_tokens + 1;
+    if (quantize) {
+        hipLaunchKernelGGL(stage_send_resolve_kernel<true>, dim3(blocks), dim3(threads), 0, stream, args, ws, st);
+    } else {
+        hipLaunchKernelGGL(stage_send_resolve_kernel<false>, dim3(blocks), dim3(threads), 0, stream, args, ws, st);
     }
     return hipGetLastError();
 }
