@@ -183,3 +183,41 @@ def test_context_creation_fails_loudly_without_a_gpu():
             hidden_dim=128, hidden_dim_scale=None, in_elemsize=2, out_elemsize=2, out_dtype=torch.bfloat16,
             scale_elemsize=None, max_num_tokens=4, max_recv_tokens=16, max_private_tokens=0, num_experts=4,
             expert_padding=1, num_experts_per_token=2, dp_size=1, node_size=2, world_size=2, device=0)
+
+
+def test_header_is_plain_c_and_links_against_the_library(tmp_path):
+    """include/a2a.h must be usable from C (no C++ or torch types): compile a caller with gcc -std=c99
+    and g++, link it against the built library and let it read the version and the two stride
+    helpers (no GPU work)."""
+    import shutil
+    import subprocess
+    repo = Path(__file__).resolve().parent.parent
+    lib = native.library_path()
+    src = tmp_path / "caller.c"
+    src.write_text("""
+#include <stdio.h>
+#include <string.h>
+#include "a2a.h"
+int main(void) {
+    a2a_config cfg;
+    memset(&cfg, 0, sizeof cfg);
+    cfg.struct_size = sizeof cfg; cfg.hidden_dim = 7168; cfg.hidden_dim_scale = 56; cfg.in_elemsize = 1;
+    cfg.out_elemsize = 2; cfg.out_dtype = A2A_BF16; cfg.scale_elemsize = 4;
+    a2a_dispatch_args d; a2a_combine_args c; (void)d; (void)c;
+    printf("%s %zu %zu %d\\n", a2a_version(), a2a_dispatch_token_stride(&cfg), a2a_combine_token_stride(&cfg),
+           (int)A2A_FLAG_SEPARATE_ROUTING);
+    return 0;
+}
+""")
+    for compiler, std in (("gcc", "-std=c99"), ("g++", "-std=c++11")):
+        if shutil.which(compiler) is None:
+            pytest.skip(f"{compiler} not installed")
+        exe = tmp_path / f"caller_{compiler}"
+        unit = src if compiler == "gcc" else tmp_path / "caller.cpp"
+        if compiler == "g++":
+            unit.write_text(src.read_text())
+        subprocess.run([compiler, std, "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", str(repo / "include"), str(unit),
+                        "-o", str(exe), "-L", str(lib.parent), "-la2a_mi355", f"-Wl,-rpath,{lib.parent}",
+                        "-Wl,--allow-shlib-undefined"], check=True)
+        out = subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()
+        assert out == ["0.1", "7408", "14336", "2"], out
