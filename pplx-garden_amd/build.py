@@ -3,7 +3,9 @@
     python pplx-garden_amd/build.py
 
 Compiles every file under csrc/ with hipcc into
-pplx_garden_amd/lib/liba2a_mi355.so.  hipcc cross-compiles without a GPU.
+pplx_garden_amd/lib/liba2a_mi355.so, and examples/selftest.cpp (a C++ caller of
+the C ABI) into pplx_garden_amd/lib/a2a_selftest.  hipcc cross-compiles without
+a GPU.
 """
 
 from __future__ import annotations
@@ -35,6 +37,10 @@ HIPCC_FLAGS = [
 
 def library_path() -> Path:
     return OUT_DIR / LIB_NAME
+
+
+def selftest_path() -> Path:
+    return OUT_DIR / "a2a_selftest"
 
 
 def build(verbose: bool = True) -> Path:
@@ -70,6 +76,12 @@ def build(verbose: bool = True) -> Path:
     if verbose:
         print(" ".join(link), flush=True)
     subprocess.run(link, check=True)
+    # A caller of the C ABI with nothing but the HIP runtime around it (no Python, no torch).
+    selftest = [hipcc, "-O2", "-std=c++17", "-I", str(REPO / "include"), str(ROOT / "examples" / "selftest.cpp"),
+                "-o", str(selftest_path()), "-L", str(OUT_DIR), "-la2a_mi355", "-Wl,-rpath,$ORIGIN"]
+    if verbose:
+        print(" ".join(selftest), flush=True)
+    subprocess.run(selftest, check=True)
     return library_path()
 
 

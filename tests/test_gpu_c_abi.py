@@ -1,0 +1,24 @@
+"""The C ABI driven by a C++ program with nothing but the HIP runtime around it (no Python, no torch):
+one step through the group calls and one through the split calls, checked on the host by the program
+itself (expert counts against a host histogram, the reference's round-trip identity)."""
+
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+def test_cpp_caller_of_the_c_abi():
+    repo = Path(__file__).resolve().parent.parent
+    sys.path.insert(0, str(repo / "pplx-garden_amd"))
+    exe = repo / "pplx-garden_amd" / "pplx_garden_amd" / "lib" / "a2a_selftest"
+    assert exe.exists(), "run pplx-garden_amd/build.py first"
+    print("running", exe, flush=True)
+    done = subprocess.run([str(exe)], capture_output=True, text=True, timeout=100)
+    print(done.stdout, done.stderr, flush=True)
+    assert done.returncode == 0, done.stderr
+    assert "selftest passed" in done.stdout
+    assert "group calls" in done.stdout and "split calls" in done.stdout
