@@ -15,8 +15,8 @@ reference's benchmark (benchmarks/bench_all_to_all.py:382-389).
 
 Prints one JSON line.  `value` is algorithmic bytes per step over the wall time
 of the timed region; per-phase times come from events recorded on the stream
-the kernels run on, around every eighth step of the same region (an event
-between two launches idles the GPU for about 3 us, so they are kept sparse).  The 128-token decode shape is timed too and reported in
+the kernels run on, around about 25 steps of the same region (an event between
+two launches idles the GPU for about 3 us, so they are kept sparse).  The 128-token decode shape is timed too and reported in
 the same line.  The CPU baseline is the oracle's C restatement, single thread,
 on the same workload.
 """
@@ -223,11 +223,12 @@ def cpu_baseline(case, rd, reps: int, threads: int = 1):
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--routings", type=int, default=4, help="distinct routings cycled over the steps")
-    ap.add_argument("--event-every", type=int, default=8,
-                    help="every how many timed steps carry the three events the phase times come from")
+    ap.add_argument("--event-every", type=int, default=0,
+                    help="every how many timed steps carry the three events the phase times come from "
+                         "(0 = about 25 such steps, at least 8 apart)")
     ap.add_argument("--cpu-reps", type=int, default=3, help="repetitions of the CPU baseline (0 = skip)")
     ap.add_argument("--no-decode", action="store_true", help="skip the 128-token shape")
     ap.add_argument("--decode-only", action="store_true",
@@ -263,6 +264,8 @@ def main() -> int:
         del src, dst
 
     ctx_flags = 2 if args.separate_routing else 0   # A2A_FLAG_SEPARATE_ROUTING
+    if args.event_every <= 0:
+        args.event_every = max(8, args.steps // 25)
     if args.decode_only:
         wl2 = Workload(C2, device, args.routings, ctx_flags)
         w2, d2, c2, b2, p2, g2 = time_workload(wl2, args.steps, args.warmup, args.event_every)
