@@ -155,8 +155,11 @@ def time_workload(wl: Workload, steps: int, warmup: int, event_every: int = 8, k
     stream = torch.cuda.current_stream(wl.device).cuda_stream
     every = max(event_every, 1)
     call_steps = [i for i in range(steps) if i % every == 0]
-    kernel_steps = [i for i in range(steps) if i % (2 * every) == every // 2 and i not in call_steps] \
-        if kernel_events else []
+    kernel_steps = []
+    if kernel_events:
+        kernel_steps = [i for i in range(steps) if i % (2 * every) == every // 2 and i not in call_steps]
+        if not kernel_steps and steps > 0:      # a very short run: share a step rather than have no sample
+            kernel_steps = [min(1, steps - 1)]
     call_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for i in call_steps}
     kern_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(4)] for i in kernel_steps}
     for evs in kern_ev.values():         # an event gets its handle when it is first recorded
