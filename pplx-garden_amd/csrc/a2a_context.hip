@@ -102,10 +102,6 @@ int check_config(const a2a_config &c) {
     if (c.num_experts_per_token == 0 || c.num_experts_per_token > A2A_MAX_EXPERTS_PER_TOKEN)
         return fail(nullptr, A2A_ERR_UNSUPPORTED, "num_experts_per_token %u not in [1, %d]",
                     c.num_experts_per_token, A2A_MAX_EXPERTS_PER_TOKEN);
-    if (((size_t)c.world_size + 1) * c.num_experts + 32 > 16384)
-        return fail(nullptr, A2A_ERR_UNSUPPORTED,
-                    "world_size * num_experts = %u is too large for the layout kernel",
-                    c.world_size * c.num_experts);
     if (c.expert_padding == 0)
         return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "expert_padding must be at least 1");
     if (c.hidden_dim == 0 || (c.in_elemsize != 1 && c.in_elemsize != 2 && c.in_elemsize != 4))

@@ -26,6 +26,7 @@ SHAPES = [
     Case("several_chunks", 700, 256, 24, 4, 8, 7010, routing="zipf", zipf_s=1.5),   # 5600 entries: 6 chunks
     Case("many_chunks", 600, 128, 64, 2, 64, 7012),                        # 38 400 entries of one source: 38 chunks
     Case("wide_ranks", 900, 128, 90, 2, 8, 7013, expert_padding=4),        # Le = 45 experts per rank, two-launch dispatch
+    Case("largest_group", 400, 128, 1024, 32, 6, 7014, expert_padding=128, node_size=16),   # 32 ranks x 1024 experts
 ]
 
 
