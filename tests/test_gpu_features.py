@@ -57,8 +57,8 @@ def test_quantiser_on_every_bf16_value_and_many_scales():
 
 
 @pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
-def test_bound_m_limits_the_tokens(split):
-    case = C0
+@pytest.mark.parametrize("case", [C0, scaled(C0, 1200)], ids=["one_launch", "two_launch"])
+def test_bound_m_limits_the_tokens(case, split):
     world = make_world(case, "all")
     bounds = [case.num_tokens, 0, 17, 1]
     rows = rows_needed(case, world)
