@@ -214,6 +214,53 @@ def test_errors_are_reported_not_faulted():
             op.destroy()
 
 
+@pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
+def test_device_errors_in_the_two_launch_paths(split):
+    """The same two device-side errors (an expert id out of range, receive buffers that are too small)
+    on a step large enough for the two-launch dispatch and send: flagged, not faulted, and the context
+    keeps working afterwards."""
+    case = scaled(C0, 1500)
+    world = make_world(case, "one")
+    N, Le, H, Hs = case.world_size, case.experts_per_rank, case.hidden_dim, case.hidden_dim_scale
+    _, ops = make_ops(case, DEV)
+    try:
+        ctx = ops[0].context
+        rd = world[0]
+        bad = rd.indices.clone()
+        bad[1234, 2] = case.num_experts + 1
+        phases = [dict(do_send=True, do_recv=False), dict(do_send=False, do_recv=True)] if split else [dict()]
+
+        def run(indices, rows):
+            t = [dict(n=torch.zeros(Le, dtype=torch.int32, device=DEV),
+                      ox=torch.full((rows, H), SENTINEL, dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn),
+                      os=torch.zeros((rows, Hs), dtype=torch.float32, device=DEV)) for _ in range(N)]
+            x, w = rd.x.to(DEV), rd.weights.to(DEV)
+            for ph in phases:
+                for r in range(N):
+                    ops[r].dispatch(out_expert_num_tokens=t[r]["n"], out_expert_x=t[r]["ox"],
+                                    out_expert_x_scale=t[r]["os"], dp_x=x if r == 0 else x[:0], dp_x_scale=None,
+                                    indices=(indices if r == 0 else indices[:0]).view(torch.uint32).to(DEV),
+                                    weights=w if r == 0 else w[:0], **ph)
+            return t
+
+        run(bad, 16)
+        flags = ctx.status()
+        assert flags & native.DEV_BAD_EXPERT_ID and flags & native.DEV_RECV_OVERFLOW
+        assert ctx.status() == 0
+        # a clean step on the same context afterwards
+        rows = rows_needed(case, world)
+        t = run(rd.indices, rows)
+        assert ctx.status() == 0
+        want = run_oracle(case, world, rows)
+        for r in range(N):
+            np.testing.assert_array_equal(t[r]["n"].cpu().numpy(), want.num_tokens[r])
+            wr = want.written[r]
+            np.testing.assert_array_equal(t[r]["ox"].view(torch.uint8).cpu().numpy()[wr], want.x[r][wr])
+    finally:
+        for op in ops:
+            op.destroy()
+
+
 def test_operator_asserts_like_the_reference():
     case = C0
     _, ops = make_ops(case, DEV)
