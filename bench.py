@@ -239,6 +239,8 @@ def main() -> int:
     ap.add_argument("--separate-routing", action="store_true",
                     help="create the context with A2A_FLAG_SEPARATE_ROUTING (routing kernels, then the pack): "
                          "for comparisons with the default paths")
+    ap.add_argument("--context-flags", type=int, default=None,
+                    help="create the context with these A2A_FLAG_* bits (for comparisons between paths)")
     ap.add_argument("--probe-copy", action="store_true",
                     help="also run plain device-to-device copies of 512 MiB (torch's copy kernel): the "
                          "known-size kernel that hardware byte counters are scaled by")
@@ -267,6 +269,8 @@ def main() -> int:
         del src, dst
 
     ctx_flags = 2 if args.separate_routing else 0   # A2A_FLAG_SEPARATE_ROUTING
+    if args.context_flags is not None:
+        ctx_flags = args.context_flags
     if args.event_every <= 0:
         args.event_every = max(8, args.steps // 25)
     if args.decode_only:
