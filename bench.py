@@ -119,13 +119,15 @@ class Workload:
 
     def step(self, i: int, stream: int, events=None, kernel_events=None):
         """One dispatch + combine.  `events` = (start, middle, end) recorded around the two calls;
-        `kernel_events` = (pack start, pack stop, gather start, gather stop), which the library
-        records at the start and end of the two bandwidth kernels themselves."""
+        `kernel_events` = (pack start, pack stop, gather start, gather stop, route start, route stop),
+        which the library records at the start and end of those kernels themselves (the last pair only
+        in a step whose dispatch has a routing launch of its own)."""
         import torch
         j = i % len(self.routings)
         if kernel_events is not None:
             self.ctx.time_next_kernel(0, kernel_events[0].cuda_event, kernel_events[1].cuda_event)
             self.ctx.time_next_kernel(1, kernel_events[2].cuda_event, kernel_events[3].cuda_event)
+            self.ctx.time_next_kernel(2, kernel_events[4].cuda_event, kernel_events[5].cuda_event)
         if events is not None:
             events[0].record()
         self.ctx.dispatch(self.dispatch_args[j], True, stream)
@@ -147,10 +149,12 @@ def time_workload(wl: Workload, steps: int, warmup: int, event_every: int = 8, k
     end costs about 8 us more).  Every `event_every`-th step carries three events around the two calls
     (before the dispatch, between dispatch and combine, after the combine).  Every 2 * `event_every`-th
     step, offset so that it is never one of those, has the library record events at the start and end
-    of the pack and the gather kernel themselves: those are the kernels' own durations.
+    of the pack, the gather and (where the step has one) the routing kernel themselves: those are the
+    kernels' own durations.
 
     Returns wall seconds and, in microseconds per sampled step: dispatch call, combine call, both,
-    pack kernel, gather kernel."""
+    pack kernel, gather kernel, routing kernel (empty when the dispatch counts its routing inside the
+    pack)."""
     import torch
     stream = torch.cuda.current_stream(wl.device).cuda_stream
     every = max(event_every, 1)
@@ -161,7 +165,7 @@ def time_workload(wl: Workload, steps: int, warmup: int, event_every: int = 8, k
         if not kernel_steps and steps > 0:      # a very short run: share a step rather than have no sample
             kernel_steps = [min(1, steps - 1)]
     call_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for i in call_steps}
-    kern_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(4)] for i in kernel_steps}
+    kern_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(6)] for i in kernel_steps}
     for evs in kern_ev.values():         # an event gets its handle when it is first recorded
         for ev in evs:
             ev.record()
@@ -182,7 +186,11 @@ def time_workload(wl: Workload, steps: int, warmup: int, event_every: int = 8, k
     both = [us(call_ev[i][0], call_ev[i][2]) for i in call_steps]
     pack = [us(kern_ev[i][0], kern_ev[i][1]) for i in kernel_steps]
     gather = [us(kern_ev[i][2], kern_ev[i][3]) for i in kernel_steps]
-    return wall_s, disp, comb, both, pack, gather
+    # a routing launch that ran in this step started shortly before the pack; events that no launch
+    # recorded still hold the time of their first recording, long before
+    route = [us(kern_ev[i][4], kern_ev[i][5]) for i in kernel_steps
+             if 0.0 <= us(kern_ev[i][4], kern_ev[i][0]) < 500.0]
+    return wall_s, disp, comb, both, pack, gather, route
 
 
 def cpu_baseline(case, rd, reps: int, threads: int = 1):
@@ -275,7 +283,7 @@ def main() -> int:
         args.event_every = max(8, args.steps // 25)
     if args.decode_only:
         wl2 = Workload(C2, device, args.routings, ctx_flags)
-        w2, d2, c2, b2, p2, g2 = time_workload(wl2, args.steps, args.warmup, args.event_every)
+        w2, d2, c2, b2, p2, g2, _ = time_workload(wl2, args.steps, args.warmup, args.event_every)
         wl2.close()
         print(json.dumps({"decode_128_only": {"step_us_wall": round(w2 / args.steps * 1e6, 2),
                                               "pack_kernel_us_mean": round(Statistics.create(p2).mean, 2),
@@ -287,10 +295,10 @@ def main() -> int:
 
     case = C3
     wl = Workload(case, device, args.routings, ctx_flags)
-    wall_s, disp, comb, both, pack, gather = time_workload(wl, args.steps, args.warmup, args.event_every)
+    wall_s, disp, comb, both, pack, gather, route = time_workload(wl, args.steps, args.warmup, args.event_every)
     # Phase statistics as the reference's benchmark reports them (events around each phase of EVERY
     # iteration, benchmarks/bench_all_to_all.py:391-433), outside the timed region above.
-    _, disp_all, comb_all, both_all, _, _ = time_workload(wl, max(args.steps, 200), 0, 1, kernel_events=False)
+    _, disp_all, comb_all, both_all, _, _, _ = time_workload(wl, max(args.steps, 200), 0, 1, kernel_events=False)
     rows = wl.rows
     cpu_rd = wl.cpu_first
     wl.close()
@@ -323,7 +331,7 @@ def main() -> int:
     if not args.no_decode:
         wl2 = Workload(C2, device, args.routings, ctx_flags)
         steps2 = max(args.steps, 200)
-        w2, d2, c2, b2, p2, g2 = time_workload(wl2, steps2, args.warmup, args.event_every)
+        w2, d2, c2, b2, p2, g2, _ = time_workload(wl2, steps2, args.warmup, args.event_every)
         wl2.close()
         decode = {
             "workload": "DeepSeek-V3 decode: 128 tokens, hidden 7168, 256 experts / 8 logical ranks, top-8 uniform, 1% x50 outliers",
@@ -390,6 +398,8 @@ def main() -> int:
                          "min": round(b_stats.min, 2), "p99": round(b_stats.p99, 2)},
             "pack_kernel_us": {"p50": round(p_stats.p50, 2), "mean": round(p_stats.mean, 2)},
             "gather_kernel_us": {"p50": round(g_stats.p50, 2), "mean": round(g_stats.mean, 2)},
+            "route_kernel_us": ({"p50": round(Statistics.create(route).p50, 2),
+                                 "mean": round(Statistics.create(route).mean, 2)} if route else None),
             "algorithmic_bytes": {"dispatch": d_bytes, "combine": c_bytes},
             "with_events_on_every_step": {
                 "note": "a second pass outside the timed region, events around each phase of every iteration as "

@@ -37,7 +37,7 @@ struct a2a_ctx {
 
     Staging staging;               // buffers and tables of the split calls
 
-    KernelTiming timing[2];        // one-shot events for the next pack / gather launch of a group call
+    KernelTiming timing[3];        // one-shot events for the next pack / gather / routing launch of a group call
 };
 
 namespace {
@@ -476,7 +476,9 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
     pa.topk_magic = K > 1 ? (uint32_t)((0x100000000ull + K - 1) / K) : 0;
 
     const KernelTiming pack_timing = ctx->timing[A2A_KERNEL_PACK];
+    const KernelTiming route_timing = ctx->timing[A2A_KERNEL_ROUTE];
     ctx->timing[A2A_KERNEL_PACK] = KernelTiming();
+    ctx->timing[A2A_KERNEL_ROUTE] = KernelTiming();
     hipError_t e;
     if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && dispatch_small_fits(pa, ctx->ws, quantize != 0, tokens)) {
         e = launch_dispatch_small(pa, fa, ctx->ws, quantize != 0, tokens, s, pack_timing);
@@ -496,7 +498,7 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
     } else {
         // Two launches: chunk histograms that also add up the step's totals, then a pack whose
         // workgroups resolve their own rows from them.
-        e = launch_route_accumulate(ra, ctx->ws, blocks, s);
+        e = launch_route_accumulate(ra, ctx->ws, blocks, s, false, route_timing);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist (accumulating)");
         e = launch_dispatch_resolve(pa, fa, ctx->ws, quantize != 0, tokens, s, pack_timing);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_resolve");
@@ -572,7 +574,7 @@ int a2a_combine(a2a_ctx *ctx, const a2a_combine_args *args, uint32_t expert_y_dt
 
 int a2a_ctx_time_next_kernel(a2a_ctx *ctx, uint32_t which, void *start_event, void *stop_event) {
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
-    if (which != A2A_KERNEL_PACK && which != A2A_KERNEL_GATHER)
+    if (which != A2A_KERNEL_PACK && which != A2A_KERNEL_GATHER && which != A2A_KERNEL_ROUTE)
         return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "unknown kernel %u", which);
     if ((start_event == nullptr) != (stop_event == nullptr))
         return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "pass both events or neither");

@@ -155,7 +155,8 @@ hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t tot
 // The same, and every chunk adds its counts to the step's totals (large group steps), or to
 // the totals of the one source of a split send (`for_send`).
 hipError_t launch_route_accumulate(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
-                                   hipStream_t stream, bool for_send = false);
+                                   hipStream_t stream, bool for_send = false,
+                                   KernelTiming timing = KernelTiming());
 // Pack that resolves its rows from the chunk histograms and the step's totals, with the
 // receiver layout and the per-source tables computed by extra workgroups of the same launch.
 hipError_t launch_dispatch_resolve(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,

@@ -428,13 +428,14 @@ hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t tot
 }
 
 hipError_t launch_route_accumulate(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
-                                   hipStream_t stream, bool for_send) {
+                                   hipStream_t stream, bool for_send, KernelTiming timing) {
     // at least one workgroup: the launch also hands over the totals between steps
     const dim3 grid(total_blocks != 0 ? total_blocks : 1);
     if (for_send) {
         hipLaunchKernelGGL(route_hist_kernel<2>, grid, dim3(kRouteBlock), 0, stream, args, ws);
     } else {
-        hipLaunchKernelGGL(route_hist_kernel<1>, grid, dim3(kRouteBlock), 0, stream, args, ws);
+        hipExtLaunchKernelGGL(route_hist_kernel<1>, grid, dim3(kRouteBlock), 0, stream, timing.start, timing.stop,
+                              0, args, ws);
     }
     return hipGetLastError();
 }

@@ -47,6 +47,7 @@ FLAG_PREALLOC_STAGING = 1
 FLAG_SEPARATE_ROUTING = 2   # never take the one-launch paths of small steps
 KERNEL_PACK = 0
 KERNEL_GATHER = 1
+KERNEL_ROUTE = 2
 
 
 class A2AConfig(ctypes.Structure):
@@ -309,9 +310,10 @@ class AllToAllContext:
         return torch.tensor(list(buf[:count]), dtype=torch.int64)
 
     def time_next_kernel(self, which: int, start_event: Optional[int], stop_event: Optional[int]) -> None:
-        """Have the next group dispatch (`KERNEL_PACK`) or combine (`KERNEL_GATHER`) record the two
-        events (raw `hipEvent_t` handles, e.g. `torch.cuda.Event.cuda_event`) at the start and end of
-        its bandwidth kernel itself."""
+        """Have the next group dispatch (`KERNEL_PACK`, `KERNEL_ROUTE`) or combine (`KERNEL_GATHER`)
+        record the two events (raw `hipEvent_t` handles, e.g. `torch.cuda.Event.cuda_event`) at the
+        start and end of that kernel itself.  `KERNEL_ROUTE` is the routing launch before the pack of a
+        large step; a step without such a launch leaves those events alone."""
         self._require_open()
         self._check(self._lib.a2a_ctx_time_next_kernel(self._handle, which, _ptr(start_event), _ptr(stop_event)))
 

@@ -8,7 +8,8 @@ import torch
 
 import a2a_oracle as oracle
 from a2a_cases import C0, C1, bf16_codes, make_world, scaled
-from a2a_harness import SENTINEL, make_ops, rows_needed, run_oracle
+from a2a_harness import (SENTINEL, assert_combine_close, assert_dispatch_equal, make_ops, rows_needed, run_gpu,
+                         run_oracle)
 from a2a_transport import RefConfig, make_ref_rank, oracle_combine, oracle_dispatch, rows_for
 from a2a_transport import make_ops as make_transport_ops
 from pplx_garden_amd.native import p2p_all_to_all as native
@@ -410,6 +411,50 @@ def test_kernel_own_events():
         with pytest.raises(RuntimeError, match="unknown kernel"):
             ctx.time_next_kernel(7, None, None)
         assert ctx.status() == 0
+    finally:
+        for op in ops:
+            op.destroy()
+
+
+def test_routing_kernel_own_events():
+    """A large group step has a routing launch of its own before the pack: A2A_KERNEL_ROUTE times it,
+    and it ends before the pack begins."""
+    case = scaled(C1, 1500)     # 8 x 1500 tokens x 8 entries: far beyond the one-launch step
+    world = make_world(case, "all")
+    rows = rows_needed(case, world)
+    want = run_oracle(case, world, rows)
+    _, ops = make_ops(case, DEV)
+    try:
+        ev = [torch.cuda.Event(enable_timing=True) for _ in range(4)]
+        for e in ev:
+            e.record()
+        torch.cuda.synchronize(DEV)
+        ctx = ops[0].context
+        ctx.time_next_kernel(native.KERNEL_ROUTE, ev[0].cuda_event, ev[1].cuda_event)
+        ctx.time_next_kernel(native.KERNEL_PACK, ev[2].cuda_event, ev[3].cuda_event)
+        got = run_gpu(case, world, rows, DEV, ops=ops)
+        torch.cuda.synchronize(DEV)
+        route_ms, pack_ms = ev[0].elapsed_time(ev[1]), ev[2].elapsed_time(ev[3])
+        print(f"route {route_ms * 1e3:.1f} us, pack {pack_ms * 1e3:.1f} us", flush=True)
+        assert 0.0 < route_ms < 1.0 and 0.0 < pack_ms
+        assert ev[1].elapsed_time(ev[2]) >= 0.0          # the routing ends before the pack begins
+        assert_dispatch_equal(case, got, want)
+        assert_combine_close(case, got, want)
+    finally:
+        for op in ops:
+            op.destroy()
+    # a small step counts its routing inside the pack: the request is consumed, nothing is recorded
+    case = C0
+    world = make_world(case, "all")
+    rows = rows_needed(case, world)
+    _, ops = make_ops(case, DEV)
+    try:
+        before = ev[3].elapsed_time(ev[0])
+        ops[0].context.time_next_kernel(native.KERNEL_ROUTE, ev[0].cuda_event, ev[1].cuda_event)
+        run_gpu(case, world, rows, DEV, ops=ops)
+        run_gpu(case, world, rows, DEV, ops=ops)
+        torch.cuda.synchronize(DEV)
+        assert ev[3].elapsed_time(ev[0]) == before
     finally:
         for op in ops:
             op.destroy()
