@@ -3,9 +3,10 @@
     python pplx-garden_amd/build.py
 
 Compiles every file under csrc/ with hipcc into
-pplx_garden_amd/lib/liba2a_mi355.so, and examples/selftest.cpp (a C++ caller of
-the C ABI) into pplx_garden_amd/lib/a2a_selftest.  hipcc cross-compiles without
-a GPU.
+pplx_garden_amd/lib/liba2a_mi355.so, examples/selftest.cpp (a C++ caller of
+the C ABI) into pplx_garden_amd/lib/a2a_selftest and examples/ceilings.hip (what
+the memory system sustains for the step's access shapes, without the library)
+into pplx_garden_amd/lib/a2a_ceilings.  hipcc cross-compiles without a GPU.
 """
 
 from __future__ import annotations
@@ -41,6 +42,10 @@ def library_path() -> Path:
 
 def selftest_path() -> Path:
     return OUT_DIR / "a2a_selftest"
+
+
+def ceilings_path() -> Path:
+    return OUT_DIR / "a2a_ceilings"
 
 
 def build(verbose: bool = True) -> Path:
@@ -82,6 +87,17 @@ def build(verbose: bool = True) -> Path:
     if verbose:
         print(" ".join(selftest), flush=True)
     subprocess.run(selftest, check=True)
+    # The yardstick of the roofline figures: plain kernels of the step's access shapes.
+    ceilings = [hipcc, "--offload-arch=gfx950", "-O3", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+                "-packed-fp32-ops", str(ROOT / "examples" / "ceilings.hip"), "-o", str(ceilings_path())]
+    if verbose:
+        print(" ".join(ceilings), flush=True)
+    out = subprocess.run(ceilings, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    lines = [l for l in out.stdout.splitlines() if "packed-fp32-ops" not in l and l.strip()]
+    if lines and verbose:
+        print("\n".join(lines), flush=True)
+    if out.returncode != 0:
+        raise RuntimeError("hipcc failed on ceilings.hip")
     return library_path()
 
 

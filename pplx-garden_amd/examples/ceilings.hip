@@ -1,0 +1,234 @@
+// What the memory system of this GPU sustains for the access shapes of the
+// DeepSeek-V3 prefill step (4096 tokens, hidden 7168, top-8), with none of the
+// library's routing in the way: the yardstick the pack and the gather kernels
+// are measured against.
+//
+//   sweep      read-only, write-only and copy over 512 MiB
+//   push       one workgroup of 448 threads per token: 32 bytes in per lane,
+//              16 bytes out to each of 8 rows of 7168 bytes (the pack's shape);
+//              rows are a random permutation of a dense buffer
+//   gather     one wavefront per token and 1 KiB piece: 16 bytes from each of
+//              8 rows of 14336 bytes, summed, 16 bytes out (the combine's shape)
+//
+// What ran before matters, because it decides what the caches hold when the
+// timed kernel starts: after a kernel that mostly reads (clean lines) the push
+// is a fifth faster than after one that wrote 600 MiB (dirty lines to evict
+// first).  So every timed launch follows a stated predecessor: the push follows
+// the gather and the gather the push, as dispatch and combine alternate in a
+// model; the sweeps follow a 600 MiB read.  The payload is random unless a
+// line says otherwise: all-zero rows are written measurably faster, so constant
+// data flatters a write-bound kernel.
+//
+// Usage: a2a_ceilings            (prints microseconds and GB/s, median of 20)
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <numeric>
+#include <random>
+#include <vector>
+
+#define CHECK(call)                                                                                \
+    do {                                                                                           \
+        hipError_t err_ = (call);                                                                  \
+        if (err_ != hipSuccess) {                                                                  \
+            std::fprintf(stderr, "%s failed: %s (%s:%d)\n", #call, hipGetErrorString(err_), __FILE__, \
+                         __LINE__);                                                                \
+            std::exit(1);                                                                          \
+        }                                                                                          \
+    } while (0)
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr uint32_t kTokens = 4096, kTopk = 8, kHidden = 7168;
+constexpr uint32_t kRows = kTokens * kTopk;
+constexpr size_t kInRow = (size_t)kHidden * 2;    // bf16 token / expert output row
+constexpr size_t kOutRow = kHidden;               // fp8 dispatched row
+
+__global__ void read_sweep(const u32x4 *__restrict__ in, u32x4 *out, size_t n, uint32_t never) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    u32x4 acc = {0, 0, 0, 0};
+    for (; i < n; i += stride) acc += __builtin_nontemporal_load(in + i);
+    if (acc[0] == never) out[0] = acc;   // keeps the loads alive, never taken
+}
+
+__global__ void write_sweep(u32x4 *out, size_t n, uint32_t seed) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        const uint32_t v = (uint32_t)i * 2654435761u + seed;
+        out[i] = u32x4{v, v ^ 0x9E3779B9u, v * 3u, v + 7u};
+    }
+}
+
+__global__ void copy_sweep(const u32x4 *__restrict__ in, u32x4 *__restrict__ out, size_t n) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) out[i] = __builtin_nontemporal_load(in + i);
+}
+
+// The pack without routing or arithmetic: the xor of two 16-byte halves stands
+// for the quantised chunk (random in, random out; equal halves give zeros).
+__global__ __launch_bounds__(448) void push(const uint8_t *__restrict__ x, uint8_t *__restrict__ out,
+                                            const uint32_t *__restrict__ slots) {
+    const uint32_t t = blockIdx.x, c = threadIdx.x;
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(x + (size_t)t * kInRow + (size_t)c * 32);
+    const u32x4 a = __builtin_nontemporal_load(p), b = __builtin_nontemporal_load(p + 1);
+    const u32x4 q = a ^ b;
+#pragma unroll
+    for (uint32_t k = 0; k < kTopk; ++k) {
+        *reinterpret_cast<u32x4 *>(out + (size_t)slots[t * kTopk + k] * kOutRow + (size_t)c * 16) = q;
+    }
+}
+
+// The combine without routing or arithmetic.  STORE = false predicates the
+// output off (one value in 2^32 would store), leaving the reads alone.
+template <bool STORE>
+__global__ __launch_bounds__(64) void gather(const uint8_t *__restrict__ y, uint8_t *__restrict__ out,
+                                             const uint32_t *__restrict__ slots, uint32_t never) {
+    const uint32_t t = blockIdx.x / 14, piece = blockIdx.x % 14;
+    const uint32_t c = piece * 64 + threadIdx.x;
+    u32x4 v[kTopk];
+#pragma unroll
+    for (uint32_t k = 0; k < kTopk; ++k) {
+        v[k] = __builtin_nontemporal_load(
+            reinterpret_cast<const u32x4 *>(y + (size_t)slots[t * kTopk + k] * kInRow + (size_t)c * 16));
+    }
+    u32x4 acc = v[0];
+#pragma unroll
+    for (uint32_t k = 1; k < kTopk; ++k) acc += v[k];
+    u32x4 *o = reinterpret_cast<u32x4 *>(out + (size_t)t * kInRow + (size_t)c * 16);
+    if (STORE) {
+        __builtin_nontemporal_store(acc, o);
+    } else if (acc[0] == never) {
+        *o = acc;
+    }
+}
+
+struct Timer {
+    hipStream_t stream;
+    hipEvent_t start, stop;
+
+    // Median over `reps` of: predecessor (untimed), then the timed launch.
+    template <typename Before, typename Launch>
+    float median_us(Before before, Launch launch, int reps = 20) {
+        std::vector<float> us;
+        for (int i = 0; i < reps + 4; ++i) {
+            before();
+            CHECK(hipEventRecord(start, stream));
+            launch();
+            CHECK(hipEventRecord(stop, stream));
+            CHECK(hipEventSynchronize(stop));
+            float ms = 0.0f;
+            CHECK(hipEventElapsedTime(&ms, start, stop));
+            if (i >= 4) us.push_back(ms * 1e3f);
+        }
+        CHECK(hipGetLastError());
+        std::sort(us.begin(), us.end());
+        return us[us.size() / 2];
+    }
+};
+
+void report(const char *name, float us, double bytes) {
+    std::printf("%-52s %7.1f us  %6.0f GB/s\n", name, us, bytes / (us * 1e-6) / 1e9);
+    std::fflush(stdout);
+}
+
+void fill_random(void *device, size_t bytes, uint32_t seed) {
+    std::vector<uint32_t> host(bytes / 4);
+    uint32_t z = seed;
+    for (auto &w : host) {
+        z = z * 1664525u + 1013904223u;
+        w = z ^ (z >> 15);
+    }
+    CHECK(hipMemcpy(device, host.data(), bytes, hipMemcpyHostToDevice));
+}
+
+}  // namespace
+
+int main() {
+    Timer timer;
+    CHECK(hipStreamCreate(&timer.stream));
+    CHECK(hipEventCreate(&timer.start));
+    CHECK(hipEventCreate(&timer.stop));
+    hipStream_t s = timer.stream;
+
+    std::vector<uint32_t> slots(kRows);
+    std::iota(slots.begin(), slots.end(), 0u);
+    std::mt19937 rng(1);
+    std::shuffle(slots.begin(), slots.end(), rng);
+    uint32_t *d_slots;
+    CHECK(hipMalloc(&d_slots, kRows * sizeof(uint32_t)));
+    CHECK(hipMemcpy(d_slots, slots.data(), kRows * sizeof(uint32_t), hipMemcpyHostToDevice));
+
+    uint8_t *x, *x_const, *dispatched, *y, *combined, *big_a, *big_b;
+    const size_t sweep_bytes = (size_t)512 << 20;
+    CHECK(hipMalloc(&x, kTokens * kInRow));
+    CHECK(hipMalloc(&x_const, kTokens * kInRow));
+    CHECK(hipMalloc(&dispatched, kRows * kOutRow));
+    CHECK(hipMalloc(&y, kRows * kInRow));
+    CHECK(hipMalloc(&combined, kTokens * kInRow));
+    CHECK(hipMalloc(&big_a, sweep_bytes));
+    CHECK(hipMalloc(&big_b, sweep_bytes));
+    fill_random(x, kTokens * kInRow, 11);
+    CHECK(hipMemset(x_const, 0x3c, kTokens * kInRow));
+    fill_random(y, kRows * kInRow, 12);
+    fill_random(big_a, sweep_bytes, 13);
+
+    uint8_t *other;
+    const size_t other_bytes = (size_t)600 << 20;
+    CHECK(hipMalloc(&other, other_bytes));
+    fill_random(other, other_bytes, 14);
+
+    const size_t n16 = sweep_bytes / 16;
+    auto read_other = [&] {
+        hipLaunchKernelGGL(read_sweep, dim3(2048), dim3(256), 0, s, (const u32x4 *)other, (u32x4 *)big_b,
+                           other_bytes / 16, 0x12345u);
+    };
+    auto fill_other = [&] {
+        hipLaunchKernelGGL(write_sweep, dim3(512), dim3(256), 0, s, (u32x4 *)other, other_bytes / 16, 3u);
+    };
+    auto run_push = [&] { hipLaunchKernelGGL(push, dim3(kTokens), dim3(448), 0, s, x, dispatched, d_slots); };
+    auto run_push_zero = [&] { hipLaunchKernelGGL(push, dim3(kTokens), dim3(448), 0, s, x_const, dispatched, d_slots); };
+    auto run_gather = [&] {
+        hipLaunchKernelGGL(gather<true>, dim3(kTokens * 14), dim3(64), 0, s, y, combined, d_slots, 0x12345u);
+    };
+    auto run_gather_reads = [&] {
+        hipLaunchKernelGGL(gather<false>, dim3(kTokens * 14), dim3(64), 0, s, y, combined, d_slots, 0x12345u);
+    };
+
+    std::printf("after a 600 MiB read:\n");
+    report("  read-only sweep, 512 MiB",
+           timer.median_us(read_other, [&] { hipLaunchKernelGGL(read_sweep, dim3(2048), dim3(256), 0, s, (const u32x4 *)big_a, (u32x4 *)big_b, n16, 0x12345u); }),
+           (double)sweep_bytes);
+    report("  write-only sweep, 512 MiB, 512 workgroups",
+           timer.median_us(read_other, [&] { hipLaunchKernelGGL(write_sweep, dim3(512), dim3(256), 0, s, (u32x4 *)big_b, n16, 5u); }),
+           (double)sweep_bytes);
+    report("  write-only sweep, 512 MiB, 4096 workgroups",
+           timer.median_us(read_other, [&] { hipLaunchKernelGGL(write_sweep, dim3(4096), dim3(256), 0, s, (u32x4 *)big_b, n16, 5u); }),
+           (double)sweep_bytes);
+    report("  copy, 512 MiB read + 512 MiB written",
+           timer.median_us(read_other, [&] { hipLaunchKernelGGL(copy_sweep, dim3(2048), dim3(256), 0, s, (const u32x4 *)big_a, (u32x4 *)big_b, n16); }),
+           2.0 * sweep_bytes);
+
+    const double push_bytes = (double)kTokens * (kInRow + kTopk * kOutRow);
+    const double gather_reads = (double)kTokens * kTopk * kInRow;
+    const double gather_bytes = gather_reads + (double)kTokens * kInRow;
+    std::printf("push and gather in turn, as dispatch and combine alternate:\n");
+    report("  push (pack's shape), random payload", timer.median_us(run_gather, run_push), push_bytes);
+    report("  push (pack's shape), all-zero rows written", timer.median_us(run_gather, run_push_zero), push_bytes);
+    report("  gather (combine's shape)", timer.median_us(run_push, run_gather), gather_bytes);
+    report("  gather, reads only (output predicated off)", timer.median_us(run_push, run_gather_reads), gather_reads);
+    std::printf("after a 600 MiB fill (dirty caches):\n");
+    report("  push (pack's shape), random payload", timer.median_us(fill_other, run_push), push_bytes);
+    report("  gather (combine's shape)", timer.median_us(fill_other, run_gather), gather_bytes);
+    report("  the gather's output alone, 56 MiB striped fill",
+           timer.median_us(fill_other, [&] { hipLaunchKernelGGL(write_sweep, dim3(512), dim3(256), 0, s, (u32x4 *)combined, kTokens * kInRow / 16, 9u); }),
+           (double)kTokens * kInRow);
+    return 0;
+}

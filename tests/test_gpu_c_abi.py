@@ -22,3 +22,19 @@ def test_cpp_caller_of_the_c_abi():
     assert done.returncode == 0, done.stderr
     assert "selftest passed" in done.stdout
     assert "group calls" in done.stdout and "split calls" in done.stdout
+
+
+def test_memory_ceilings_program_runs():
+    """The yardstick of the roofline figures (plain kernels of the step's access shapes) runs and reports
+    every line; its numbers are read by people, not asserted here."""
+    repo = Path(__file__).resolve().parent.parent
+    exe = repo / "pplx-garden_amd" / "pplx_garden_amd" / "lib" / "a2a_ceilings"
+    assert exe.exists(), "run pplx-garden_amd/build.py first"
+    print("running", exe, flush=True)
+    done = subprocess.run([str(exe)], capture_output=True, text=True, timeout=100)
+    print(done.stdout, done.stderr, flush=True)
+    assert done.returncode == 0, done.stderr
+    lines = [l for l in done.stdout.splitlines() if "GB/s" in l]
+    assert len(lines) == 11
+    assert any("push (pack's shape), random payload" in l for l in lines)
+    assert any("gather (combine's shape)" in l for l in lines)
