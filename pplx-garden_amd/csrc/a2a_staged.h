@@ -45,6 +45,7 @@ struct StageSendArgs {
     uint32_t hidden_dim;
     uint32_t hidden_dim_scale;
     uint32_t topk_magic;      // ceil(2^32 / K) (0 for K = 1), for entry -> token without a division
+    uint32_t resolver_wave;   // resolving send: wavefront that resolves the routes (set by the launcher)
 };
 
 struct StageRecvArgs {

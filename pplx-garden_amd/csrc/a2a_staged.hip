@@ -19,8 +19,10 @@ size_t align_up_sz(size_t n, size_t a) { return (n + a - 1) / a * a; }
 
 // Stages the row of `token` (payload, then scales).  Whole workgroup.
 template <bool QUANT>
-__device__ __forceinline__ void stage_row(const StageSendArgs &args, const Staging &st, uint32_t g, uint32_t token) {
+__device__ __forceinline__ void stage_row(const StageSendArgs &args, const Staging &st, uint32_t g, uint32_t token,
+                                          uint32_t staging_threads) {
     const uint32_t tid = threadIdx.x;
+    if (tid >= staging_threads) return;
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
     const PushSrc &src = args.src;
@@ -30,7 +32,7 @@ __device__ __forceinline__ void stage_row(const StageSendArgs &args, const Stagi
 
     if constexpr (QUANT) {
         const uint32_t num_chunks = args.hidden_dim / 16;
-        for (uint32_t base = wave * kWave; base < num_chunks; base += blockDim.x) {
+        for (uint32_t base = wave * kWave; base < num_chunks; base += staging_threads) {
             const uint32_t c = base + lane;
             const bool active = c < num_chunks;
             u32x4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
@@ -48,13 +50,13 @@ __device__ __forceinline__ void stage_row(const StageSendArgs &args, const Stagi
         }
     } else {
         const uint32_t num_chunks = args.row_bytes / 16;
-        for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
+        for (uint32_t c = tid; c < num_chunks; c += staging_threads) {
             reinterpret_cast<u32x4 *>(row)[c] =
                 __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
         }
         if (src.x_scale != nullptr) {
             const float *xs = src.x_scale + (size_t)token * src.xs_stride_token;
-            for (uint32_t j = tid; j < args.hidden_dim_scale; j += blockDim.x) {
+            for (uint32_t j = tid; j < args.hidden_dim_scale; j += staging_threads) {
                 row_scale[j] = xs[(size_t)j * src.xs_stride_elem];
             }
         }
@@ -87,7 +89,7 @@ __global__ __launch_bounds__(1024) void stage_send_kernel(const StageSendArgs ar
         }
         ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
     }
-    stage_row<QUANT>(args, st, g, token);
+    stage_row<QUANT>(args, st, g, token, blockDim.x);
 }
 
 // The send of a small step in ONE launch (the reference's dispatch-send kernel
@@ -188,7 +190,7 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
             ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
         }
     }
-    stage_row<QUANT>(args, st, g, token);
+    stage_row<QUANT>(args, st, g, token, blockDim.x);
 }
 
 // The send of a large step, after a routing launch that left the chunk counts,
@@ -239,7 +241,10 @@ __global__ __launch_bounds__(1024) void stage_send_resolve_kernel(const StageSen
     const PushSrc &src = args.src;
     if (token >= effective_tokens(src.bound_m, src.num_tokens)) return;
 
-    if (wave == 0) {
+    // With a wavefront to spare the last one resolves and stages nothing, so that no wavefront
+    // has both chains of memory trips to walk; otherwise wavefront 0 does both.
+    const uint32_t staging_threads = args.resolver_wave != 0 ? args.resolver_wave * kWave : blockDim.x;
+    if (wave == args.resolver_wave) {
         const uint32_t *counts = ws.chunk_counts + (size_t)g * E * ws.nb_max;   // [E][nb_max]
         const uint32_t part = lane & 7, route = lane >> 3;
         for (uint32_t k0 = 0; k0 < K; k0 += 8) {
@@ -287,7 +292,7 @@ __global__ __launch_bounds__(1024) void stage_send_resolve_kernel(const StageSen
             }
         }
     }
-    stage_row<QUANT>(args, st, g, token);
+    stage_row<QUANT>(args, st, g, token, staging_threads);
 }
 
 // A team of `team` threads (one or more whole wavefronts) copies a row of
@@ -656,12 +661,18 @@ hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &w
 
 hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                                      bool quantize, hipStream_t stream) {
-    const uint32_t threads = block_for_chunks(quantize ? args.hidden_dim / 16 : args.row_bytes / 16);
+    uint32_t threads = block_for_chunks(quantize ? args.hidden_dim / 16 : args.row_bytes / 16);
     const uint32_t blocks = args.src.num_tokens + 1;
+    StageSendArgs a = args;
+    a.resolver_wave = 0;
+    if (threads + kWave <= 1024) {   // a wavefront of its own for the routes (measured: 27.3 against 28.5 us)
+        a.resolver_wave = threads / kWave;
+        threads += kWave;
+    }
     if (quantize) {
-        hipLaunchKernelGGL(stage_send_resolve_kernel<true>, dim3(blocks), dim3(threads), 0, stream, args, ws, st);
+        hipLaunchKernelGGL(stage_send_resolve_kernel<true>, dim3(blocks), dim3(threads), 0, stream, a, ws, st);
     } else {
-        hipLaunchKernelGGL(stage_send_resolve_kernel<false>, dim3(blocks), dim3(threads), 0, stream, args, ws, st);
+        hipLaunchKernelGGL(stage_send_resolve_kernel<false>, dim3(blocks), dim3(threads), 0, stream, a, ws, st);
     }
     return hipGetLastError();
 }
