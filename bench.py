@@ -119,7 +119,7 @@ class Workload:
 
     def step(self, i: int, stream: int, events=None, kernel_events=None):
         """One dispatch + combine.  `events` = (start, middle, end) recorded around the two calls;
-        `kernel_events` = (pack start, pack stop, gather start, gather stop, route start, route stop),
+        `kernel_events` = (pack start, pack stop, gather start, gather stop[, route start, route stop]),
         which the library records at the start and end of those kernels themselves (the last pair only
         in a step whose dispatch has a routing launch of its own)."""
         import torch
@@ -127,7 +127,8 @@ class Workload:
         if kernel_events is not None:
             self.ctx.time_next_kernel(0, kernel_events[0].cuda_event, kernel_events[1].cuda_event)
             self.ctx.time_next_kernel(1, kernel_events[2].cuda_event, kernel_events[3].cuda_event)
-            self.ctx.time_next_kernel(2, kernel_events[4].cuda_event, kernel_events[5].cuda_event)
+            if len(kernel_events) >= 6:
+                self.ctx.time_next_kernel(2, kernel_events[4].cuda_event, kernel_events[5].cuda_event)
         if events is not None:
             events[0].record()
         self.ctx.dispatch(self.dispatch_args[j], True, stream)
@@ -141,31 +142,32 @@ class Workload:
         self.ctx.destroy()
 
 
-def time_workload(wl: Workload, steps: int, warmup: int, event_every: int = 8, kernel_events: bool = True):
+def time_workload(wl: Workload, steps: int, warmup: int, kernel_every: int = 32, call_every: int = 0,
+                  route_events: bool = False):
     """W untimed steps, then exactly K timed steps between two synchronisations.
 
-    Events are kept sparse, because they cost idle GPU time (measured on the 4096-token step: 146.8 us
-    per step without events, 152.5 us with one after each call; a launch that records its own start and
-    end costs about 8 us more).  Every `event_every`-th step carries three events around the two calls
-    (before the dispatch, between dispatch and combine, after the combine).  Every 2 * `event_every`-th
-    step, offset so that it is never one of those, has the library record events at the start and end
-    of the pack, the gather and (where the step has one) the routing kernel themselves: those are the
-    kernels' own durations.
+    Events cost idle GPU time (measured on the 4096-token step: 146.8 us per step without events,
+    152.5 us with one after each call; a launch that records its own start and end costs about 3 us
+    more), so the timed region carries them sparsely.  Every `kernel_every`-th step has the library record
+    events at the start and end of the pack and the gather kernel themselves: the kernels' own durations
+    (with `route_events` also of the routing launch, where the step has one).  Every `call_every`-th
+    step (0 = none), never one of those, carries three events around the two calls (before the dispatch,
+    between dispatch and combine, after the combine).
 
     Returns wall seconds and, in microseconds per sampled step: dispatch call, combine call, both,
-    pack kernel, gather kernel, routing kernel (empty when the dispatch counts its routing inside the
-    pack)."""
+    pack kernel, gather kernel, routing kernel (empty without `route_events`, or when the dispatch
+    counts its routing inside the pack)."""
     import torch
     stream = torch.cuda.current_stream(wl.device).cuda_stream
-    every = max(event_every, 1)
-    call_steps = [i for i in range(steps) if i % every == 0]
     kernel_steps = []
-    if kernel_events:
-        kernel_steps = [i for i in range(steps) if i % (2 * every) == every // 2 and i not in call_steps]
-        if not kernel_steps and steps > 0:      # a very short run: share a step rather than have no sample
-            kernel_steps = [min(1, steps - 1)]
+    if kernel_every > 0:
+        kernel_steps = [i for i in range(steps) if i % kernel_every == kernel_every // 2]
+        if not kernel_steps and steps > 0:      # a very short run still gets a sample
+            kernel_steps = [steps // 2]
+    call_steps = [i for i in range(steps) if call_every > 0 and i % call_every == 0 and i not in kernel_steps]
     call_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for i in call_steps}
-    kern_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(6)] for i in kernel_steps}
+    kern_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(6 if route_events else 4)]
+               for i in kernel_steps}
     for evs in kern_ev.values():         # an event gets its handle when it is first recorded
         for ev in evs:
             ev.record()
@@ -186,10 +188,12 @@ def time_workload(wl: Workload, steps: int, warmup: int, event_every: int = 8, k
     both = [us(call_ev[i][0], call_ev[i][2]) for i in call_steps]
     pack = [us(kern_ev[i][0], kern_ev[i][1]) for i in kernel_steps]
     gather = [us(kern_ev[i][2], kern_ev[i][3]) for i in kernel_steps]
-    # a routing launch that ran in this step started shortly before the pack; events that no launch
-    # recorded still hold the time of their first recording, long before
-    route = [us(kern_ev[i][4], kern_ev[i][5]) for i in kernel_steps
-             if 0.0 <= us(kern_ev[i][4], kern_ev[i][0]) < 500.0]
+    route = []
+    if route_events:
+        # a routing launch that ran in this step started shortly before the pack; events that no launch
+        # recorded still hold the time of their first recording, long before
+        route = [us(kern_ev[i][4], kern_ev[i][5]) for i in kernel_steps
+                 if 0.0 <= us(kern_ev[i][4], kern_ev[i][0]) < 500.0]
     return wall_s, disp, comb, both, pack, gather, route
 
 
@@ -237,9 +241,9 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--routings", type=int, default=4, help="distinct routings cycled over the steps")
-    ap.add_argument("--event-every", type=int, default=0,
-                    help="every how many timed steps carry the three events the phase times come from "
-                         "(0 = about 25 such steps, at least 8 apart)")
+    ap.add_argument("--kernel-every", type=int, default=0,
+                    help="every how many timed steps have the pack and the gather kernel record their own "
+                         "start and end (0 = about 12 such steps, at least 16 apart)")
     ap.add_argument("--cpu-reps", type=int, default=3, help="repetitions of the CPU baseline (0 = skip)")
     ap.add_argument("--no-decode", action="store_true", help="skip the 128-token shape")
     ap.add_argument("--decode-only", action="store_true",
@@ -279,11 +283,12 @@ def main() -> int:
     ctx_flags = 2 if args.separate_routing else 0   # A2A_FLAG_SEPARATE_ROUTING
     if args.context_flags is not None:
         ctx_flags = args.context_flags
-    if args.event_every <= 0:
-        args.event_every = max(8, args.steps // 25)
+    if args.kernel_every <= 0:
+        args.kernel_every = max(16, args.steps // 12)
     if args.decode_only:
         wl2 = Workload(C2, device, args.routings, ctx_flags)
-        w2, d2, c2, b2, p2, g2, _ = time_workload(wl2, args.steps, args.warmup, args.event_every)
+        w2, _, _, _, p2, g2, _ = time_workload(wl2, args.steps, args.warmup, args.kernel_every)
+        _, d2, c2, b2, _, _, _ = time_workload(wl2, max(args.steps, 200), 0, 0, call_every=1)
         wl2.close()
         print(json.dumps({"decode_128_only": {"step_us_wall": round(w2 / args.steps * 1e6, 2),
                                               "pack_kernel_us_mean": round(Statistics.create(p2).mean, 2),
@@ -295,10 +300,12 @@ def main() -> int:
 
     case = C3
     wl = Workload(case, device, args.routings, ctx_flags)
-    wall_s, disp, comb, both, pack, gather, route = time_workload(wl, args.steps, args.warmup, args.event_every)
+    wall_s, _, _, _, pack, gather, _ = time_workload(wl, args.steps, args.warmup, args.kernel_every)
     # Phase statistics as the reference's benchmark reports them (events around each phase of EVERY
-    # iteration, benchmarks/bench_all_to_all.py:391-433), outside the timed region above.
-    _, disp_all, comb_all, both_all, _, _, _ = time_workload(wl, max(args.steps, 200), 0, 1, kernel_events=False)
+    # iteration, benchmarks/bench_all_to_all.py:391-433), outside the timed region above; every fourth
+    # step times the routing launch by its own events instead.
+    _, disp, comb, both, _, _, route = time_workload(wl, max(args.steps, 200), 0, 4, call_every=1,
+                                                     route_events=True)
     rows = wl.rows
     cpu_rd = wl.cpu_first
     wl.close()
@@ -306,7 +313,6 @@ def main() -> int:
     d_bytes, c_bytes = algorithmic_bytes(case.num_tokens, case.hidden_dim, case.topk)
     ms_per_step = wall_s / args.steps * 1e3
     value = (d_bytes + c_bytes) / (ms_per_step * 1e-3) / 1e9
-    d_stats, c_stats, b_stats = Statistics.create(disp), Statistics.create(comb), Statistics.create(both)
     p_stats, g_stats = Statistics.create(pack), Statistics.create(gather)
 
     def stats_dict(xs):
@@ -331,7 +337,8 @@ def main() -> int:
     if not args.no_decode:
         wl2 = Workload(C2, device, args.routings, ctx_flags)
         steps2 = max(args.steps, 200)
-        w2, d2, c2, b2, p2, g2, _ = time_workload(wl2, steps2, args.warmup, args.event_every)
+        w2, _, _, _, p2, g2, _ = time_workload(wl2, steps2, args.warmup, args.kernel_every)
+        _, d2, c2, b2, _, _, _ = time_workload(wl2, steps2, 0, 0, call_every=1)
         wl2.close()
         decode = {
             "workload": "DeepSeek-V3 decode: 128 tokens, hidden 7168, 256 experts / 8 logical ranks, top-8 uniform, 1% x50 outliers",
@@ -343,9 +350,9 @@ def main() -> int:
             "total_us_p50": round(Statistics.create(b2).p50, 2),
             "total_us_mean": round(Statistics.create(b2).mean, 2),
             "note": "working set (26 MB) fits the 256 MB Infinity Cache and is not flushed between steps; "
-                    "step_us_wall is wall time over all steps, the p50 figures come from the steps that carry "
-                    "events around the calls (each event adds about 3 us), the kernel figures from events the "
-                    "launches record themselves",
+                    "step_us_wall is wall time over the timed steps, the kernel figures come from events the "
+                    "launches record themselves on a few of those steps, the p50 figures from a second pass "
+                    "with events around the calls of every step (each event adds about 3 us)",
         }
 
     cpu = cpu_more = None
@@ -391,22 +398,19 @@ def main() -> int:
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "prefill_4096": {
             "step_us_wall": round(ms_per_step * 1e3, 2),
-            "steps_with_events": len(disp),
-            "dispatch_us": {"p50": round(d_stats.p50, 2), "mean": round(d_stats.mean, 2)},
-            "combine_us": {"p50": round(c_stats.p50, 2), "mean": round(c_stats.mean, 2)},
-            "total_us": {"p50": round(b_stats.p50, 2), "mean": round(b_stats.mean, 2),
-                         "min": round(b_stats.min, 2), "p99": round(b_stats.p99, 2)},
+            "timed_steps_with_kernel_events": len(gather),
             "pack_kernel_us": {"p50": round(p_stats.p50, 2), "mean": round(p_stats.mean, 2)},
             "gather_kernel_us": {"p50": round(g_stats.p50, 2), "mean": round(g_stats.mean, 2)},
-            "route_kernel_us": ({"p50": round(Statistics.create(route).p50, 2),
-                                 "mean": round(Statistics.create(route).mean, 2)} if route else None),
             "algorithmic_bytes": {"dispatch": d_bytes, "combine": c_bytes},
             "with_events_on_every_step": {
                 "note": "a second pass outside the timed region, events around each phase of every iteration as "
-                        "in the reference's benchmark; each event adds about 3 us",
-                "dispatch_us": stats_dict(disp_all),
-                "combine_us": stats_dict(comb_all),
-                "total_us": stats_dict(both_all),
+                        "in the reference's benchmark (each event adds about 3 us); every fourth step has the "
+                        "routing launch record its own start and end instead",
+                "dispatch_us": stats_dict(disp),
+                "combine_us": stats_dict(comb),
+                "total_us": stats_dict(both),
+                "route_kernel_us": ({"p50": round(Statistics.create(route).p50, 2),
+                                     "mean": round(Statistics.create(route).mean, 2)} if route else None),
             },
         },
         "decode_128": decode,
