@@ -238,8 +238,8 @@ def cpu_baseline(case, rd, reps: int, threads: int = 1):
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=400)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=1000)
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--routings", type=int, default=4, help="distinct routings cycled over the steps")
     ap.add_argument("--kernel-every", type=int, default=0,
                     help="every how many timed steps have the pack and the gather kernel record their own "
