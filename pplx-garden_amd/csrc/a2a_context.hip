@@ -125,6 +125,8 @@ int check_config(const a2a_config &c) {
                     c.scale_elemsize);
     if (c.max_num_tokens == 0)
         return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "max_num_tokens must be at least 1");
+    if (c.flags & ~(uint32_t)(A2A_FLAG_PREALLOC_STAGING | A2A_FLAG_SEPARATE_ROUTING))
+        return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "unknown bits in flags: 0x%x", c.flags);
     if ((uint64_t)c.max_num_tokens * c.num_experts_per_token > 0x7FFFFFFFull)
         return fail(nullptr, A2A_ERR_UNSUPPORTED, "max_num_tokens * num_experts_per_token too large");
     return A2A_OK;

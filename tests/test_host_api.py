@@ -71,6 +71,7 @@ def _config(**over):
     (dict(out_dtype=14, out_elemsize=8), -3, "out_dtype"),
     (dict(hidden_dim_scale=4, scale_elemsize=2), -3, "scale"),
     (dict(max_num_tokens=0), -1, "max_num_tokens"),
+    (dict(flags=8), -1, "flags"),
 ])
 def test_bad_configurations_are_rejected_with_a_message(over, code, needle):
     lib = native.load_library()
