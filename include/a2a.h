@@ -227,6 +227,34 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
                  void *stream);
 
 /*
+ * a2a_dispatch without a context and without any allocation.  No counterpart in
+ * the reference; it is for callers that cannot allocate device memory where they
+ * run a step: code under HIP graph capture, serving loops and harnesses that
+ * forbid hipMalloc.  Same arguments and same results as a2a_dispatch on a context
+ * created from `config` (its `flags` must be 0), but the routing tables of the
+ * step live in a fixed array of A2A_STATIC_SCRATCH_BYTES inside the library
+ * (every GPU the library is used on holds one copy until the process ends) and
+ * the call neither allocates nor frees nor copies: it enqueues one small kernel
+ * that prepares the tables, then the launches of a2a_dispatch.
+ *   - The tables are sized for THIS step (largest `num_tokens` among the ranks);
+ *     a step whose tables exceed the array is refused with
+ *     A2A_ERR_TOO_MANY_TOKENS and a message that names the sizes.  The DeepSeek-V3
+ *     prefill step with all 8 ranks sending 4096 tokens needs 3.4 MB.
+ *   - All calls on one GPU share the array: calls whose kernels could overlap
+ *     (different streams, no ordering between them) race.  Calls on one stream,
+ *     or ordered by events, are fine; each call clears what it needs cleared.
+ *   - `device_flags`: optional DEVICE pointer to one uint32 that the kernels OR
+ *     the A2A_DEV_* bits into (the caller clears it); with NULL bad input is
+ *     dropped silently as described at those bits.
+ *   - The routing of the step stays inside the library: a2a_combine needs a
+ *     context and the a2a_dispatch that goes with it.
+ * Error text: a2a_last_error(NULL) on the calling thread.
+ */
+#define A2A_STATIC_SCRATCH_BYTES (8u << 20)
+int a2a_dispatch_static(const a2a_config *config, const a2a_dispatch_args *args,
+                        uint32_t quantize, uint32_t *device_flags, void *stream);
+
+/*
  * combine() of all ranks in one call (p2p_all_to_all.py:442-517 with do_send
  * and do_recv); uses the routing of the last a2a_dispatch.  expert_y rows are
  * read in place: no staging copy.

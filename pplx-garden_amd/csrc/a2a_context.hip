@@ -11,6 +11,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -39,6 +40,13 @@ struct a2a_ctx {
 
     KernelTiming timing[3];        // one-shot events for the next pack / gather / routing launch of a group call
 };
+
+// Device memory of a2a_dispatch_static: the routing tables of ONE step, in a
+// file-scope array instead of an allocation.  Every GPU the library runs on
+// holds its own copy at its own address until the process ends.  In host code
+// this name only stands for the symbol: the address kernels get is the one
+// hipGetSymbolAddress returns with that GPU current (static_scratch_of).
+static __device__ __align__(256) unsigned char scratch[A2A_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -140,9 +148,8 @@ int check_rank(a2a_ctx *ctx, uint32_t rank) {
 }
 
 // Arguments of the send half that do not depend on who receives.
-int check_send(a2a_ctx *ctx, uint32_t rank, uint64_t num_tokens, const void *x, uint64_t x_stride,
-               uint32_t quantize, const float *xs, const int32_t *indices) {
-    const a2a_config &c = ctx->cfg;
+int check_send(a2a_ctx *ctx, const a2a_config &c, uint32_t rank, uint64_t num_tokens, const void *x,
+               uint64_t x_stride, uint32_t quantize, const float *xs, const int32_t *indices) {
     if (num_tokens > c.max_num_tokens)
         return fail(ctx, A2A_ERR_TOO_MANY_TOKENS, "Number of tokens exceeds maximum allowed (rank %u: %llu > %u)",
                     rank, (unsigned long long)num_tokens, c.max_num_tokens);
@@ -175,9 +182,8 @@ int check_send(a2a_ctx *ctx, uint32_t rank, uint64_t num_tokens, const void *x, 
     return A2A_OK;
 }
 
-int check_recv(a2a_ctx *ctx, uint32_t rank, const void *out_x, uint64_t out_stride,
+int check_recv(a2a_ctx *ctx, const a2a_config &c, uint32_t rank, const void *out_x, uint64_t out_stride,
                const float *out_scale) {
-    const a2a_config &c = ctx->cfg;
     if (out_x == nullptr) return A2A_OK;  // a rank may decline to receive
     if (!aligned16(out_x) || out_stride % 16 != 0)
         return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: out_x rows must be 16-byte aligned", rank);
@@ -226,8 +232,225 @@ bool fused_routing_pays(const FinalizeArgs &fa, uint32_t world, uint32_t total_b
     return total_blocks <= 4 * A2A_FUSED_MAX_CHUNKS;
 }
 
-uint32_t all_ranks(const a2a_ctx *ctx) {
-    return ctx->cfg.world_size >= 32 ? 0xFFFFFFFFu : ((1u << ctx->cfg.world_size) - 1);
+// Dimensions of the device workspace for steps of at most `max_tokens` tokens per
+// rank, and its tables carved out of `base` (256-byte aligned each).  With a null
+// `base` only the dimensions are filled in.  Returns the bytes the tables take.
+size_t carve_workspace(const a2a_config &c, uint32_t max_tokens, uint8_t *base, Workspace &ws) {
+    const uint32_t N = c.world_size, E = c.num_experts, K = c.num_experts_per_token;
+    ws.max_tk = (max_tokens != 0 ? max_tokens : 1) * K;
+    ws.nb_max = ceil_div_u32(ws.max_tk, kRouteBlock);
+    ws.world = N;
+    ws.num_groups = N / c.dp_size;
+    ws.dp_size = c.dp_size;
+    ws.num_experts = E;
+    ws.topk = K;
+    ws.experts_per_rank = ceil_div_u32(E, N);
+    ws.node_size = c.node_size;
+    ws.expert_padding = c.expert_padding;
+    ws.le_magic = ws.experts_per_rank > 1 ? 0xFFFFFFFFu / ws.experts_per_rank + 1 : 0;
+
+    size_t off = 0;
+    auto carve = [&off](size_t bytes) {
+        const size_t at = off;
+        off = align_up(off + bytes, 256);
+        return at;
+    };
+    const size_t o_local = carve((size_t)N * ws.max_tk * sizeof(uint16_t));
+    const size_t o_hist = carve((size_t)N * ws.nb_max * E * sizeof(uint32_t));
+    const size_t o_block = carve((size_t)N * ws.nb_max * E * sizeof(uint32_t));
+    const size_t o_routed = carve((size_t)N * E * sizeof(uint32_t));
+    const size_t o_offsets = carve((size_t)N * E * sizeof(uint32_t));
+    const size_t o_base = carve((size_t)N * E * sizeof(uint32_t));
+    const size_t o_tpe = carve((size_t)E * sizeof(uint32_t));
+    const size_t o_poff = carve((size_t)E * sizeof(uint32_t));
+    const size_t o_slot = carve((size_t)N * ws.max_tk * sizeof(uint32_t));
+    const size_t o_toff = carve((size_t)N * ws.max_tk * sizeof(uint32_t));
+    const size_t o_err = carve(sizeof(uint32_t));
+    const size_t o_order = carve((size_t)N * kMaxWorld);
+    const size_t o_before = carve((size_t)N * ws.num_groups * sizeof(uint32_t));
+    const size_t o_chunk_counts = carve((size_t)N * ws.nb_max * E * sizeof(uint32_t));
+    const size_t o_totals = carve(2 * ((size_t)ws.num_groups + 1) * E * sizeof(uint32_t));
+    const size_t o_turn = carve(2 * sizeof(uint32_t));
+    const size_t o_send_totals = carve(2 * ((size_t)E + N) * sizeof(uint32_t));
+    const size_t o_send_turn = carve(2 * sizeof(uint32_t));
+    if (base != nullptr) {
+        ws.local_rank = reinterpret_cast<uint16_t *>(base + o_local);
+        ws.block_hist = reinterpret_cast<uint32_t *>(base + o_hist);
+        ws.block_prefix = reinterpret_cast<uint32_t *>(base + o_block);
+        ws.num_routed = reinterpret_cast<uint32_t *>(base + o_routed);
+        ws.expert_offsets = reinterpret_cast<uint32_t *>(base + o_offsets);
+        ws.slot_base = reinterpret_cast<uint32_t *>(base + o_base);
+        ws.tokens_per_expert = reinterpret_cast<uint32_t *>(base + o_tpe);
+        ws.padded_offset = reinterpret_cast<uint32_t *>(base + o_poff);
+        ws.route_slot = reinterpret_cast<uint32_t *>(base + o_slot);
+        ws.token_offset = reinterpret_cast<uint32_t *>(base + o_toff);
+        ws.err = reinterpret_cast<uint32_t *>(base + o_err);
+        ws.order = reinterpret_cast<const uint32_t *>(base + o_order);
+        ws.laid_before = reinterpret_cast<const uint32_t *>(base + o_before);
+        ws.chunk_counts = reinterpret_cast<uint32_t *>(base + o_chunk_counts);
+        ws.totals = reinterpret_cast<uint32_t *>(base + o_totals);
+        ws.turn = reinterpret_cast<uint32_t *>(base + o_turn);
+        ws.send_totals = reinterpret_cast<uint32_t *>(base + o_send_totals);
+        ws.send_turn = reinterpret_cast<uint32_t *>(base + o_send_turn);
+    }
+    return off;
+}
+
+// The group dispatch on the tables of `ws`: argument checks, then the launches.  `ctx` only
+// receives error texts and may be null (then they go where a2a_last_error(NULL) finds them).
+// `num_tokens_out[g]`, if not null, gets the tokens of every source.
+int dispatch_group(a2a_ctx *ctx, const a2a_config &c, const Workspace &ws, const a2a_dispatch_args *args,
+                   uint32_t quantize, hipStream_t s, KernelTiming pack_timing, KernelTiming route_timing,
+                   uint32_t *num_tokens_out) {
+    const uint32_t N = c.world_size, K = c.num_experts_per_token;
+    for (uint32_t r = 0; r < N; ++r) {
+        const a2a_dispatch_args &a = args[r];
+        if (int rc = check_send(ctx, c, r, a.num_tokens, a.x_ptr, a.x_stride, quantize, a.x_scale_ptr, a.indices))
+            return rc;
+        if (int rc = check_recv(ctx, c, r, a.out_x, a.out_x_stride, a.out_x_scale)) return rc;
+    }
+
+    RouteArgs ra;
+    FinalizeArgs fa;
+    PushArgs pa;
+    memset(&ra, 0, sizeof ra);
+    memset(&fa, 0, sizeof fa);
+    memset(&pa, 0, sizeof pa);
+    const uint32_t D = c.dp_size, G = N / D;
+    uint32_t blocks = 0, tokens = 0;
+    // Sources: one per dp group (its members hold the same tokens; the first member's are read).
+    for (uint32_t g = 0; g < G; ++g) {
+        const a2a_dispatch_args &a = args[g * D];
+        for (uint32_t m = 1; m < D; ++m) {
+            if (args[g * D + m].num_tokens != a.num_tokens)
+                return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "ranks %u and %u share a dp group but pass %llu and %llu tokens",
+                            g * D, g * D + m, (unsigned long long)a.num_tokens,
+                            (unsigned long long)args[g * D + m].num_tokens);
+        }
+        const uint32_t T = (uint32_t)a.num_tokens;
+        ra.src[g] = RouteSrc{a.indices, a.bound_m, (uint32_t)a.indices_stride, T};
+        ra.block_start[g] = blocks;
+        fa.num_blocks[g] = ceil_div_u32((uint64_t)T * K, kRouteBlock);
+        blocks += fa.num_blocks[g];
+        PushSrc &ps = pa.src[g];
+        ps.x = static_cast<const uint8_t *>(a.x_ptr);
+        ps.x_scale = a.x_scale_ptr;
+        ps.indices = a.indices;
+        ps.bound_m = a.bound_m;
+        ps.x_stride = a.x_stride;
+        ps.xs_stride_elem = (uint32_t)a.x_scale_stride_elem;
+        ps.xs_stride_token = (uint32_t)a.x_scale_stride_token;
+        ps.indices_stride = (uint32_t)a.indices_stride;
+        ps.num_tokens = T;
+        pa.token_start[g] = tokens;
+        tokens += T;
+        if (num_tokens_out != nullptr) num_tokens_out[g] = T;
+    }
+    for (uint32_t g = G; g <= (uint32_t)kMaxWorld; ++g) {
+        ra.block_start[g] = blocks;
+        pa.token_start[g] = tokens;
+    }
+    // Receivers: every rank.
+    for (uint32_t r = 0; r < N; ++r) {
+        const a2a_dispatch_args &a = args[r];
+        fa.out_num_tokens[r] = a.out_num_tokens;
+        fa.out_rows[r] = a.out_x != nullptr ? (uint32_t)(a.out_x_rows > 0xFFFFFFFFull ? 0xFFFFFFFFull : a.out_x_rows)
+                                            : 0xFFFFFFFFu;
+        PushDst &pd = pa.dst[r];
+        pd.out_x = static_cast<uint8_t *>(a.out_x);
+        pd.out_scale = a.out_x_scale;
+        pd.out_stride = a.out_x_stride;
+        pd.os_stride_elem = (uint32_t)a.out_x_scale_stride_elem;
+        pd.os_stride_token = (uint32_t)a.out_x_scale_stride_token;
+        pd.out_rows = fa.out_rows[r];
+    }
+    fa.fold_mask = fa.valid_mask = G >= 32 ? 0xFFFFFFFFu : ((1u << G) - 1);
+    fa.recv_mask = N >= 32 ? 0xFFFFFFFFu : ((1u << N) - 1);
+    pa.row_bytes = (uint32_t)row_bytes_of(c);
+    pa.hidden_dim = c.hidden_dim;
+    pa.hidden_dim_scale = c.hidden_dim_scale;
+    pa.topk_magic = K > 1 ? (uint32_t)((0x100000000ull + K - 1) / K) : 0;
+
+    hipError_t e;
+    if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && dispatch_small_fits(pa, ws, quantize != 0, tokens)) {
+        e = launch_dispatch_small(pa, fa, ws, quantize != 0, tokens, s, pack_timing);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_small");
+    } else if (c.flags & A2A_FLAG_SEPARATE_ROUTING) {
+        if (fused_routing_pays(fa, G, blocks)) {
+            e = launch_route_fused(ra, fa, ws, s);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
+        } else {
+            e = launch_route(ra, ws, blocks, s);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
+            e = launch_finalize(fa, ws, s);
+            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
+        }
+        e = launch_dispatch_push(pa, ws, quantize != 0, tokens, s, pack_timing);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_push");
+    } else {
+        // Two launches: chunk histograms that also add up the step's totals, then a pack whose
+        // workgroups resolve their own rows from them.
+        e = launch_route_accumulate(ra, ws, blocks, s, false, route_timing);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist (accumulating)");
+        e = launch_dispatch_resolve(pa, fa, ws, quantize != 0, tokens, s, pack_timing);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_resolve");
+    }
+    return A2A_OK;
+}
+
+
+// Address of `scratch` on device `dev` (which must be current), looked up once
+// per device.
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+uint8_t *g_scratch_ptr[kMaxDevices] = {};
+
+hipError_t static_scratch_of(int dev, uint8_t **out) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return e;
+        g_scratch_ptr[dev] = static_cast<uint8_t *>(ptr);
+    }
+    *out = g_scratch_ptr[dev];
+    return hipSuccess;
+}
+
+// What a step on tables that hold another step's leftovers needs before its
+// first launch: both copies of the step totals and the word that says whose turn
+// it is start at zero, and the two tables that a context uploads once at create
+// (the order in which every receiver lays out its sources, and which sources
+// come before which) are computed here.  `clear_err`: the error word is the
+// library's own (the caller gave none), so nobody reads it; keep it tidy.
+__global__ __launch_bounds__(1024) void static_prepare_kernel(const Workspace ws, uint32_t clear_err) {
+    const uint32_t N = ws.world, G = ws.num_groups, E = ws.num_experts;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t words = 2 * (G + 1) * E;
+    for (uint32_t i = blockIdx.x * blockDim.x + tid; i < words; i += gridDim.x * blockDim.x) ws.totals[i] = 0;
+    if (blockIdx.x != 0) return;
+    if (tid < 2) ws.turn[tid] = 0;
+    if (clear_err != 0 && tid == 0) *ws.err = 0;
+    uint32_t *order = const_cast<uint32_t *>(ws.order);
+    for (uint32_t w = tid; w < N * (kMaxWorld / 4); w += blockDim.x) {
+        const uint32_t r = w / (kMaxWorld / 4), i0 = (w % (kMaxWorld / 4)) * 4;
+        uint32_t word = 0;
+        for (uint32_t j = 0; j < 4; ++j) {
+            if (i0 + j < G) word |= source_order(r, i0 + j, N, ws.node_size, ws.dp_size) << (8 * j);
+        }
+        order[w] = word;
+    }
+    uint32_t *before = const_cast<uint32_t *>(ws.laid_before);
+    for (uint32_t w = tid; w < N * G; w += blockDim.x) {
+        const uint32_t r = w / G, g = w % G;
+        uint32_t seen = 0;
+        for (uint32_t i = 0; i < G; ++i) {
+            const uint32_t s = source_order(r, i, N, ws.node_size, ws.dp_size);
+            if (s == g) break;
+            seen |= 1u << s;
+        }
+        before[w] = seen;
+    }
 }
 
 }  // namespace
@@ -269,46 +492,9 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
     if (ctx == nullptr) return fail(nullptr, A2A_ERR_OUT_OF_MEMORY, "out of host memory");
     ctx->cfg = *config;
 
-    const uint32_t N = config->world_size, E = config->num_experts, K = config->num_experts_per_token;
+    const uint32_t N = config->world_size;
     Workspace &ws = ctx->ws;
-    ws.max_tk = config->max_num_tokens * K;
-    ws.nb_max = ceil_div_u32(ws.max_tk, kRouteBlock);
-    ws.world = N;
-    ws.num_groups = N / config->dp_size;
-    ws.dp_size = config->dp_size;
-    ws.num_experts = E;
-    ws.topk = K;
-    ws.experts_per_rank = ceil_div_u32(E, N);
-    ws.node_size = config->node_size;
-    ws.expert_padding = config->expert_padding;
-    ws.le_magic = ws.experts_per_rank > 1 ? 0xFFFFFFFFu / ws.experts_per_rank + 1 : 0;
-
-    // One allocation, carved into 256-byte aligned tables.
-    size_t off = 0;
-    auto carve = [&off](size_t bytes) {
-        const size_t at = off;
-        off = align_up(off + bytes, 256);
-        return at;
-    };
-    const size_t o_local = carve((size_t)N * ws.max_tk * sizeof(uint16_t));
-    const size_t o_hist = carve((size_t)N * ws.nb_max * E * sizeof(uint32_t));
-    const size_t o_block = carve((size_t)N * ws.nb_max * E * sizeof(uint32_t));
-    const size_t o_routed = carve((size_t)N * E * sizeof(uint32_t));
-    const size_t o_offsets = carve((size_t)N * E * sizeof(uint32_t));
-    const size_t o_base = carve((size_t)N * E * sizeof(uint32_t));
-    const size_t o_tpe = carve((size_t)E * sizeof(uint32_t));
-    const size_t o_poff = carve((size_t)E * sizeof(uint32_t));
-    const size_t o_slot = carve((size_t)N * ws.max_tk * sizeof(uint32_t));
-    const size_t o_toff = carve((size_t)N * ws.max_tk * sizeof(uint32_t));
-    const size_t o_err = carve(sizeof(uint32_t));
-    const size_t o_order = carve((size_t)N * kMaxWorld);
-    const size_t o_before = carve((size_t)N * ws.num_groups * sizeof(uint32_t));
-    const size_t o_chunk_counts = carve((size_t)N * ws.nb_max * E * sizeof(uint32_t));
-    const size_t o_totals = carve(2 * ((size_t)ws.num_groups + 1) * E * sizeof(uint32_t));
-    const size_t o_turn = carve(2 * sizeof(uint32_t));
-    const size_t o_send_totals = carve(2 * ((size_t)E + N) * sizeof(uint32_t));
-    const size_t o_send_turn = carve(2 * sizeof(uint32_t));
-    ctx->arena_bytes = off;
+    ctx->arena_bytes = carve_workspace(*config, config->max_num_tokens, nullptr, ws);
     e = hipMalloc(&ctx->arena, ctx->arena_bytes);
     if (e != hipSuccess) {
         delete ctx;
@@ -322,24 +508,7 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
         return hip_fail(nullptr, e, "hipMemset(workspace)");
     }
     uint8_t *base = static_cast<uint8_t *>(ctx->arena);
-    ws.local_rank = reinterpret_cast<uint16_t *>(base + o_local);
-    ws.block_hist = reinterpret_cast<uint32_t *>(base + o_hist);
-    ws.block_prefix = reinterpret_cast<uint32_t *>(base + o_block);
-    ws.num_routed = reinterpret_cast<uint32_t *>(base + o_routed);
-    ws.expert_offsets = reinterpret_cast<uint32_t *>(base + o_offsets);
-    ws.slot_base = reinterpret_cast<uint32_t *>(base + o_base);
-    ws.tokens_per_expert = reinterpret_cast<uint32_t *>(base + o_tpe);
-    ws.padded_offset = reinterpret_cast<uint32_t *>(base + o_poff);
-    ws.route_slot = reinterpret_cast<uint32_t *>(base + o_slot);
-    ws.token_offset = reinterpret_cast<uint32_t *>(base + o_toff);
-    ws.err = reinterpret_cast<uint32_t *>(base + o_err);
-    ws.order = reinterpret_cast<const uint32_t *>(base + o_order);
-    ws.laid_before = reinterpret_cast<const uint32_t *>(base + o_before);
-    ws.chunk_counts = reinterpret_cast<uint32_t *>(base + o_chunk_counts);
-    ws.totals = reinterpret_cast<uint32_t *>(base + o_totals);
-    ws.turn = reinterpret_cast<uint32_t *>(base + o_turn);
-    ws.send_totals = reinterpret_cast<uint32_t *>(base + o_send_totals);
-    ws.send_turn = reinterpret_cast<uint32_t *>(base + o_send_turn);
+    carve_workspace(*config, config->max_num_tokens, base, ws);
     {
         // i-th source each receiver lays out, and which sources come before which: fixed for the
         // life of the context
@@ -354,9 +523,10 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx) {
                 seen |= 1u << g;
             }
         }
-        e = hipMemcpy(base + o_order, table, (size_t)N * kMaxWorld, hipMemcpyHostToDevice);
+        e = hipMemcpy(const_cast<uint32_t *>(ws.order), table, (size_t)N * kMaxWorld, hipMemcpyHostToDevice);
         if (e == hipSuccess)
-            e = hipMemcpy(base + o_before, before, (size_t)N * ws.num_groups * sizeof(uint32_t), hipMemcpyHostToDevice);
+            e = hipMemcpy(const_cast<uint32_t *>(ws.laid_before), before, (size_t)N * ws.num_groups * sizeof(uint32_t),
+                          hipMemcpyHostToDevice);
         if (e != hipSuccess) {
             (void)hipFree(ctx->arena);
             delete ctx;
@@ -405,112 +575,61 @@ int a2a_ctx_status(a2a_ctx *ctx, void *stream, uint32_t *flags) {
 int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize, void *stream) {
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
     if (args == nullptr) return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "null args");
-    const a2a_config &c = ctx->cfg;
-    const uint32_t N = c.world_size, K = c.num_experts_per_token;
-    for (uint32_t r = 0; r < N; ++r) {
-        const a2a_dispatch_args &a = args[r];
-        if (int rc = check_send(ctx, r, a.num_tokens, a.x_ptr, a.x_stride, quantize, a.x_scale_ptr, a.indices))
-            return rc;
-        if (int rc = check_recv(ctx, r, a.out_x, a.out_x_stride, a.out_x_scale)) return rc;
-    }
-    DeviceGuard guard(c.device);
-    hipStream_t s = static_cast<hipStream_t>(stream);
-
-    RouteArgs ra;
-    FinalizeArgs fa;
-    PushArgs pa;
-    memset(&ra, 0, sizeof ra);
-    memset(&fa, 0, sizeof fa);
-    memset(&pa, 0, sizeof pa);
-    const uint32_t D = c.dp_size, G = N / D;
-    uint32_t blocks = 0, tokens = 0;
-    // Sources: one per dp group (its members hold the same tokens; the first member's are read).
-    for (uint32_t g = 0; g < G; ++g) {
-        const a2a_dispatch_args &a = args[g * D];
-        for (uint32_t m = 1; m < D; ++m) {
-            if (args[g * D + m].num_tokens != a.num_tokens)
-                return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "ranks %u and %u share a dp group but pass %llu and %llu tokens",
-                            g * D, g * D + m, (unsigned long long)a.num_tokens,
-                            (unsigned long long)args[g * D + m].num_tokens);
-        }
-        const uint32_t T = (uint32_t)a.num_tokens;
-        ra.src[g] = RouteSrc{a.indices, a.bound_m, (uint32_t)a.indices_stride, T};
-        ra.block_start[g] = blocks;
-        fa.num_blocks[g] = ceil_div_u32((uint64_t)T * K, kRouteBlock);
-        blocks += fa.num_blocks[g];
-        PushSrc &ps = pa.src[g];
-        ps.x = static_cast<const uint8_t *>(a.x_ptr);
-        ps.x_scale = a.x_scale_ptr;
-        ps.indices = a.indices;
-        ps.bound_m = a.bound_m;
-        ps.x_stride = a.x_stride;
-        ps.xs_stride_elem = (uint32_t)a.x_scale_stride_elem;
-        ps.xs_stride_token = (uint32_t)a.x_scale_stride_token;
-        ps.indices_stride = (uint32_t)a.indices_stride;
-        ps.num_tokens = T;
-        pa.token_start[g] = tokens;
-        tokens += T;
-        ctx->num_tokens[g] = T;
-    }
-    for (uint32_t g = G; g <= (uint32_t)kMaxWorld; ++g) {
-        ra.block_start[g] = blocks;
-        pa.token_start[g] = tokens;
-    }
-    // Receivers: every rank.
-    for (uint32_t r = 0; r < N; ++r) {
-        const a2a_dispatch_args &a = args[r];
-        fa.out_num_tokens[r] = a.out_num_tokens;
-        fa.out_rows[r] = a.out_x != nullptr ? (uint32_t)(a.out_x_rows > 0xFFFFFFFFull ? 0xFFFFFFFFull : a.out_x_rows)
-                                            : 0xFFFFFFFFu;
-        PushDst &pd = pa.dst[r];
-        pd.out_x = static_cast<uint8_t *>(a.out_x);
-        pd.out_scale = a.out_x_scale;
-        pd.out_stride = a.out_x_stride;
-        pd.os_stride_elem = (uint32_t)a.out_x_scale_stride_elem;
-        pd.os_stride_token = (uint32_t)a.out_x_scale_stride_token;
-        pd.out_rows = fa.out_rows[r];
-    }
-    fa.fold_mask = fa.valid_mask = G >= 32 ? 0xFFFFFFFFu : ((1u << G) - 1);
-    fa.recv_mask = all_ranks(ctx);
-    pa.row_bytes = (uint32_t)row_bytes_of(c);
-    pa.hidden_dim = c.hidden_dim;
-    pa.hidden_dim_scale = c.hidden_dim_scale;
-    pa.topk_magic = K > 1 ? (uint32_t)((0x100000000ull + K - 1) / K) : 0;
-
+    DeviceGuard guard(ctx->cfg.device);
     const KernelTiming pack_timing = ctx->timing[A2A_KERNEL_PACK];
     const KernelTiming route_timing = ctx->timing[A2A_KERNEL_ROUTE];
     ctx->timing[A2A_KERNEL_PACK] = KernelTiming();
     ctx->timing[A2A_KERNEL_ROUTE] = KernelTiming();
-    hipError_t e;
-    if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && dispatch_small_fits(pa, ctx->ws, quantize != 0, tokens)) {
-        e = launch_dispatch_small(pa, fa, ctx->ws, quantize != 0, tokens, s, pack_timing);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_small");
-    } else if (c.flags & A2A_FLAG_SEPARATE_ROUTING) {
-        if (fused_routing_pays(fa, G, blocks)) {
-            e = launch_route_fused(ra, fa, ctx->ws, s);
-            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_fused");
-        } else {
-            e = launch_route(ra, ctx->ws, blocks, s);
-            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist");
-            e = launch_finalize(fa, ctx->ws, s);
-            if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
-        }
-        e = launch_dispatch_push(pa, ctx->ws, quantize != 0, tokens, s, pack_timing);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_push");
-    } else {
-        // Two launches: chunk histograms that also add up the step's totals, then a pack whose
-        // workgroups resolve their own rows from them.
-        e = launch_route_accumulate(ra, ctx->ws, blocks, s, false, route_timing);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist (accumulating)");
-        e = launch_dispatch_resolve(pa, fa, ctx->ws, quantize != 0, tokens, s, pack_timing);
-        if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_resolve");
-    }
-
+    if (int rc = dispatch_group(ctx, ctx->cfg, ctx->ws, args, quantize, static_cast<hipStream_t>(stream), pack_timing,
+                                route_timing, ctx->num_tokens))
+        return rc;
     ctx->group_routing = true;
     ctx->step_open = false;
     ctx->sent_mask = 0;
     ctx->quantized = quantize;
     return A2A_OK;
+}
+
+int a2a_dispatch_static(const a2a_config *config, const a2a_dispatch_args *args, uint32_t quantize,
+                        uint32_t *device_flags, void *stream) {
+    if (config == nullptr || args == nullptr) return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "null argument");
+    if (int rc = check_config(*config)) return rc;
+    const a2a_config &c = *config;
+    if (c.flags != 0)
+        return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "a2a_dispatch_static takes no flags (got 0x%x)", c.flags);
+    if (c.device < 0 || c.device >= kMaxDevices)
+        return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "device %d not in [0, %d)", c.device, kMaxDevices);
+    // The tables are sized for this step: the largest source decides.
+    uint64_t max_tokens = 0;
+    for (uint32_t r = 0; r < c.world_size; ++r) {
+        if (args[r].num_tokens > max_tokens) max_tokens = args[r].num_tokens;
+    }
+    if (max_tokens > c.max_num_tokens)
+        return fail(nullptr, A2A_ERR_TOO_MANY_TOKENS, "Number of tokens exceeds maximum allowed (%llu > %u)",
+                    (unsigned long long)max_tokens, c.max_num_tokens);
+    Workspace ws;
+    memset(&ws, 0, sizeof ws);
+    const size_t need = carve_workspace(c, (uint32_t)max_tokens, nullptr, ws);
+    if (need > (size_t)A2A_STATIC_SCRATCH_BYTES)
+        return fail(nullptr, A2A_ERR_TOO_MANY_TOKENS,
+                    "a step of %u ranks x %llu tokens x %u routes over %u experts needs %zu bytes of routing tables; "
+                    "a2a_dispatch_static has %zu (use a2a_ctx_create and a2a_dispatch for larger steps)",
+                    c.world_size, (unsigned long long)max_tokens, c.num_experts_per_token, c.num_experts, need,
+                    (size_t)A2A_STATIC_SCRATCH_BYTES);
+    DeviceGuard guard(c.device);
+    if (!guard.ok) return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "cannot select device %d", c.device);
+    uint8_t *base = nullptr;
+    hipError_t e = static_scratch_of(c.device, &base);
+    if (e != hipSuccess) return hip_fail(nullptr, e, "hipGetSymbolAddress(scratch)");
+    carve_workspace(c, (uint32_t)max_tokens, base, ws);
+    if (device_flags != nullptr) ws.err = device_flags;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const uint32_t words = 2 * (ws.num_groups + 1) * ws.num_experts;
+    const uint32_t blocks = words > 8 * 1024 ? 8 : 1;
+    hipLaunchKernelGGL(static_prepare_kernel, dim3(blocks), dim3(1024), 0, s, ws, device_flags == nullptr ? 1u : 0u);
+    e = hipGetLastError();
+    if (e != hipSuccess) return hip_fail(nullptr, e, "launch static_prepare");
+    return dispatch_group(nullptr, c, ws, args, quantize, s, KernelTiming(), KernelTiming(), nullptr);
 }
 
 int a2a_combine(a2a_ctx *ctx, const a2a_combine_args *args, uint32_t expert_y_dtype,
@@ -647,7 +766,8 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     (void)weights_stride;
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
     if (int rc = check_rank(ctx, rank)) return rc;
-    if (int rc = check_send(ctx, rank, num_tokens, x_ptr, x_stride, quantize, x_scale_ptr, indices)) return rc;
+    if (int rc = check_send(ctx, ctx->cfg, rank, num_tokens, x_ptr, x_stride, quantize, x_scale_ptr, indices))
+        return rc;
     const a2a_config &c = ctx->cfg;
     DeviceGuard guard(c.device);
     if (!ctx->staging.allocated) {
@@ -741,7 +861,7 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
     if (int rc = check_rank(ctx, rank)) return rc;
     if (!ctx->step_open || ctx->sent_mask == 0)
         return fail(ctx, A2A_ERR_BAD_ORDER, "a2a_dispatch_recv before any a2a_dispatch_send of the step");
-    if (int rc = check_recv(ctx, rank, out_x, out_x_stride, out_x_scale)) return rc;
+    if (int rc = check_recv(ctx, ctx->cfg, rank, out_x, out_x_stride, out_x_scale)) return rc;
     const a2a_config &c = ctx->cfg;
     DeviceGuard guard(c.device);
     hipStream_t s = static_cast<hipStream_t>(stream);

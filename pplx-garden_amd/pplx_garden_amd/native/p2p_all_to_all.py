@@ -105,6 +105,7 @@ _SIGNATURES = {
         c_void_p, c_size_t, c_void_p, c_uint32, c_void_p]),
     "a2a_dispatch": (c_int, [c_void_p, POINTER(A2ADispatchArgs), c_uint32, c_void_p]),
     "a2a_combine": (c_int, [c_void_p, POINTER(A2ACombineArgs), c_uint32, c_uint32, c_void_p]),
+    "a2a_dispatch_static": (c_int, [POINTER(A2AConfig), POINTER(A2ADispatchArgs), c_uint32, c_void_p, c_void_p]),
 }
 
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
@@ -140,6 +141,24 @@ def _ptr(value: Optional[int]) -> Optional[int]:
 
 def _num(value: Optional[int]) -> int:
     return 0 if value is None else int(value)
+
+
+STATIC_SCRATCH_BYTES = 8 << 20
+
+
+def dispatch_static(config: A2AConfig, per_rank: Sequence[A2ADispatchArgs], quantize: bool,
+                    device_flags_ptr: Optional[int], stream: int) -> None:
+    """`a2a_dispatch_static`: the group dispatch without a context and without any allocation (the
+    routing tables of the step live in a fixed array inside the library).  `per_rank` holds one
+    A2ADispatchArgs per rank of `config.world_size`; `device_flags_ptr` is an optional device pointer
+    to one uint32 that collects the DEV_* bits."""
+    lib = load_library()
+    if len(per_rank) != config.world_size:
+        raise RuntimeError(f"expected arguments of {config.world_size} ranks, got {len(per_rank)}")
+    arr = per_rank if isinstance(per_rank, ctypes.Array) else (A2ADispatchArgs * config.world_size)(*per_rank)
+    rc = lib.a2a_dispatch_static(ctypes.byref(config), arr, int(quantize), _ptr(device_flags_ptr), _ptr(stream))
+    if rc != 0:
+        raise RuntimeError(lib.a2a_last_error(None).decode() or f"a2a_dispatch_static failed ({rc})")
 
 
 class AllToAllContext:

@@ -92,6 +92,28 @@ def test_null_arguments_do_not_crash():
     assert lib.a2a_ctx_status(None, None, None) == -1
 
 
+def test_static_dispatch_refuses_what_its_fixed_tables_cannot_hold():
+    """The checks of a2a_dispatch_static run before its first HIP call, so they can be exercised
+    without a GPU: a step beyond the fixed array, flags, and more tokens than max_num_tokens."""
+    lib = native.load_library()
+    big = _config(world_size=32, node_size=32, num_experts=1024, num_experts_per_token=8, max_num_tokens=8192,
+                  hidden_dim=7168, in_elemsize=1, hidden_dim_scale=56, scale_elemsize=4)
+    args = (native.A2ADispatchArgs * 32)()
+    for a in args:
+        a.num_tokens = 8192
+    assert lib.a2a_dispatch_static(ctypes.byref(big), args, 1, None, None) == -2
+    msg = lib.a2a_last_error(None).decode()
+    assert "bytes of routing tables" in msg and str(native.STATIC_SCRATCH_BYTES) in msg
+    assert lib.a2a_dispatch_static(ctypes.byref(_config(flags=2)), args, 0, None, None) == -1
+    assert "flags" in lib.a2a_last_error(None).decode()
+    small = _config()
+    args[0].num_tokens = 17
+    assert lib.a2a_dispatch_static(ctypes.byref(small), args, 0, None, None) == -2
+    assert lib.a2a_dispatch_static(None, None, 0, None, None) == -1
+    header_bytes = re.search(r"#define A2A_STATIC_SCRATCH_BYTES \((\d+)u << (\d+)\)", HEADER)
+    assert int(header_bytes.group(1)) << int(header_bytes.group(2)) == native.STATIC_SCRATCH_BYTES
+
+
 def test_strides_match_the_oracle():
     lib = native.load_library()
     for H, ie, Hs, se, oe in [(7168, 1, 56, 4, 2), (2048, 1, 16, 4, 2), (128, 4, 0, 0, 4), (16, 2, 0, 0, 2),
