@@ -8,7 +8,7 @@ from pathlib import Path
 
 import numpy as np
 
-_PATH = Path(__file__).resolve().parent.parent / "oracle" / "liba2a_oracle.so"
+_PATH = Path(__file__).resolve().parent / "liba2a_oracle.so"
 _lib = None
 
 

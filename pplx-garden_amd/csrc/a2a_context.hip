@@ -898,6 +898,15 @@ int a2a_combine_send(a2a_ctx *ctx, uint32_t rank, const void *expert_y, size_t e
     if (expert_y == nullptr || !aligned16(expert_y) || expert_y_stride % 16 != 0)
         return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: expert_y rows must be non-null and 16-byte aligned", rank);
     const a2a_config &c = ctx->cfg;
+    // The call copies whole staging rows of hidden_dim * out_elemsize bytes and is not told the type
+    // of expert_y (neither is the reference's, a2a_combine_send.cu:261): rows that are closer
+    // together than that hold narrower elements, and copying them would read past the last row.
+    if (expert_y_rows > 1 && expert_y_stride < (size_t)c.hidden_dim * c.out_elemsize)
+        return fail(ctx, A2A_ERR_UNSUPPORTED,
+                    "rank %u: expert_y rows are %zu bytes apart but a staged combine row holds %zu "
+                    "(hidden_dim x %u-byte elements of out_dtype): the split calls need expert_y in a type "
+                    "as wide as out_dtype",
+                    rank, expert_y_stride, (size_t)c.hidden_dim * c.out_elemsize, c.out_elemsize);
     DeviceGuard guard(c.device);
     CombineSendArgs cs;
     memset(&cs, 0, sizeof cs);

@@ -92,24 +92,10 @@ class P2PAllToAll(AllToAllKernel):
         num_dp_groups = world_size // self._dp_size
         self._num_local_experts = ceil_div(num_experts, world_size)
 
-        # Buffer sizing (p2p_all_to_all.py:94-114).
-        avg_tokens_per_expert = int(
-            ceil_div(max_num_tokens * num_experts_per_token, num_experts) * 1.2)
-        if max_private_tokens is None:
-            max_private_tokens = avg_tokens_per_expert * self._num_local_experts
-        assert max_private_tokens >= 0
-        num_tokens = max_num_tokens * num_dp_groups
-        max_recv_tokens = max_private_tokens * num_dp_groups + round_up(
-            max(
-                min(
-                    num_tokens * num_experts_per_token
-                    + self._num_local_experts * (expert_padding - 1),
-                    num_tokens * self._num_local_experts,
-                ),
-                self._num_local_experts * expert_padding,
-            ),
-            expert_padding,
-        )
+        max_private_tokens, max_recv_tokens = self.receive_capacity(
+            max_num_tokens=max_num_tokens, num_experts=num_experts, expert_padding=expert_padding,
+            num_experts_per_token=num_experts_per_token, world_size=world_size, dp_size=self._dp_size,
+            max_private_tokens=max_private_tokens)
         self.max_recv_tokens = max_recv_tokens
         self.max_private_tokens = max_private_tokens
 
@@ -153,6 +139,26 @@ class P2PAllToAll(AllToAllKernel):
         self._all_to_all = global_group.world.acquire_context(self._key, make_context)
 
     # ------------------------------------------------------------------
+
+    @staticmethod
+    def receive_capacity(*, max_num_tokens: int, num_experts: int, expert_padding: int,
+                         num_experts_per_token: int, world_size: int, dp_size: int = 1,
+                         max_private_tokens: Optional[int] = None):
+        """(max_private_tokens, max_recv_tokens): rows of a rank's receive region as the reference
+        sizes them (p2p_all_to_all.py:94-114).  Every dp group gets a private region (by default 1.2
+        times the average load of the rank's experts); on top of that come the rows all groups share:
+        every copy of every group's tokens could land here, but no more than one per (token, local
+        expert), and never less than one padded block per local expert."""
+        groups = world_size // dp_size
+        local_experts = ceil_div(num_experts, world_size)
+        if max_private_tokens is None:
+            average = int(ceil_div(max_num_tokens * num_experts_per_token, num_experts) * 1.2)
+            max_private_tokens = average * local_experts
+        assert max_private_tokens >= 0
+        tokens = max_num_tokens * groups
+        every_copy = tokens * num_experts_per_token + local_experts * (expert_padding - 1)
+        shared = max(min(every_copy, tokens * local_experts), local_experts * expert_padding)
+        return max_private_tokens, max_private_tokens * groups + round_up(shared, expert_padding)
 
     @property
     def num_local_experts(self) -> int:
@@ -375,6 +381,13 @@ class P2PAllToAll(AllToAllKernel):
                         "every rank must call combine() with the same expert_y dtype and accumulate")
                 self._all_to_all.combine([a for a, _, _, _ in posted], dtypes.pop(), accs.pop(), stream)
             return
+
+        if expert_y.dtype.itemsize != self._out_dtype.itemsize:
+            # combine-send copies staging rows sized for out_dtype without knowing the type of
+            # expert_y (as the reference's does, a2a_combine_send.cu:261); narrower rows would be over-read
+            raise RuntimeError(
+                f"split combine needs expert_y ({expert_y.dtype}) with the element size of out_dtype "
+                f"({self._out_dtype}); call combine() with do_send and do_recv for mixed types")
 
         if do_send:
             self._all_to_all.combine_send(

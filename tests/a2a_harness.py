@@ -9,7 +9,7 @@ import numpy as np
 import torch
 
 import a2a_oracle as oracle
-from a2a_cases import Case, RankData, bf16_codes
+from a2a_cases import Case, RankData, bf16_codes, rows_needed  # noqa: F401
 
 SENTINEL = 0xA5
 
@@ -20,18 +20,6 @@ class WorldResult:
     x: List[np.ndarray]               # per rank [rows, H] uint8 (fp8 codes)
     x_scale: List[np.ndarray]         # per rank [rows, Hs] float32
     out_tokens: List[np.ndarray]      # per rank [T, H] bf16 codes (uint16)
-
-
-def rows_needed(case: Case, world: Sequence[RankData]) -> int:
-    """Rows a receive buffer needs so that no rank overflows (with padding)."""
-    Le = case.experts_per_rank
-    counts = np.zeros(case.num_experts, dtype=np.int64)
-    for rd in world:
-        counts += np.bincount(rd.indices.numpy().reshape(-1), minlength=case.num_experts)
-    pad = case.expert_padding
-    padded = (counts + pad - 1) // pad * pad
-    per_rank = [padded[r * Le:(r + 1) * Le].sum() for r in range(case.world_size)]
-    return int(max(max(per_rank), 1))
 
 
 def act_numpy(q: np.ndarray, scale: np.ndarray) -> np.ndarray:

@@ -5,7 +5,7 @@ from pathlib import Path
 import pytest
 
 REPO = Path(__file__).resolve().parent.parent
-for p in (REPO, REPO / "pplx-garden_amd", REPO / "oracle", REPO / "tests"):
+for p in (REPO, REPO / "pplx-garden_amd", REPO / "pplx-garden_amd" / "benchmarks", REPO / "oracle", REPO / "tests"):
     if str(p) not in sys.path:
         sys.path.insert(0, str(p))
 

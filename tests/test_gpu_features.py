@@ -7,7 +7,7 @@ import pytest
 import torch
 
 import a2a_oracle as oracle
-from a2a_cases import C0, C1, bf16_codes, make_world, scaled
+from a2a_cases import C0, C1, C2, bf16_codes, make_world, scaled
 from a2a_harness import (SENTINEL, assert_combine_close, assert_dispatch_equal, make_ops, rows_needed, run_gpu,
                          run_oracle)
 from a2a_transport import RefConfig, make_ref_rank, oracle_combine, oracle_dispatch, rows_for
@@ -113,6 +113,37 @@ def test_bound_m_limits_the_tokens(case, split):
             op.destroy()
 
 
+def _check_split_combine_refuses_narrow_rows(in_dtype, out_dtype):
+    """combine-send copies staging rows sized for out_dtype and is not told the type of expert_y:
+    narrower rows are refused before any launch, by the operator and by the C ABI."""
+    cfg = RefConfig("types", 4, 1, 48, 16, 256, None, 4, torch.bfloat16, out_dtype, None)
+    world = [make_ref_rank(cfg, r) for r in range(4)]
+    rows = rows_for(cfg, world)
+    ops = make_transport_ops(cfg, DEV)
+    try:
+        t = []
+        for r, rd in enumerate(world):
+            t.append(dict(x=rd.dp_x.to(DEV), idx=rd.indices.view(torch.uint32).to(DEV), w=rd.weights.to(DEV),
+                          n=torch.zeros(4, dtype=torch.int32, device=DEV),
+                          ox=torch.zeros((rows, cfg.hidden_dim), dtype=torch.bfloat16, device=DEV),
+                          y=torch.zeros((rows, cfg.hidden_dim), dtype=in_dtype, device=DEV),
+                          o=torch.zeros((cfg.max_num_tokens, cfg.hidden_dim), dtype=out_dtype, device=DEV)))
+        for ph in (dict(do_send=True, do_recv=False), dict(do_send=False, do_recv=True)):
+            for r in range(4):
+                ops[r].dispatch(out_expert_num_tokens=t[r]["n"], out_expert_x=t[r]["ox"], out_expert_x_scale=None,
+                                dp_x=t[r]["x"], dp_x_scale=None, indices=t[r]["idx"], weights=t[r]["w"], **ph)
+        with pytest.raises(RuntimeError, match="element size of out_dtype"):
+            ops[0].combine(out_tokens=t[0]["o"], indices=t[0]["idx"], weights=t[0]["w"], expert_y=t[0]["y"],
+                           do_send=True, do_recv=False)
+        with pytest.raises(RuntimeError, match="as wide as out_dtype"):
+            ops[0].context.combine_send(0, t[0]["y"].data_ptr(), cfg.hidden_dim * in_dtype.itemsize, rows, 0)
+        torch.cuda.synchronize(DEV)
+        assert ops[0].context.status() == 0
+    finally:
+        for op in ops:
+            op.destroy()
+
+
 @pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
 @pytest.mark.parametrize("in_dtype,out_dtype", [
     (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32), (torch.float16, torch.float16),
@@ -123,7 +154,8 @@ def test_combine_types_and_accumulate(in_dtype, out_dtype, split):
     without accumulate (a2a_combine_recv.cu:132).  The split calls stage rows sized for the
     output type, so there expert_y has the output's element size."""
     if split and in_dtype.itemsize != out_dtype.itemsize:
-        pytest.skip("staging rows are sized for out_dtype")
+        _check_split_combine_refuses_narrow_rows(in_dtype, out_dtype)
+        return
     cfg = RefConfig("types", 4, 1, 48, 16, 256, None, 4, torch.bfloat16, out_dtype, None)
     world = [make_ref_rank(cfg, r) for r in range(4)]
     rows = rows_for(cfg, world)
@@ -458,3 +490,22 @@ def test_routing_kernel_own_events():
     finally:
         for op in ops:
             op.destroy()
+
+
+def test_operator_reports_the_reference_capacities():
+    """`P2PAllToAll.max_recv_tokens` / `max_private_tokens` of live operators on the five baseline
+    shapes against the oracle's restatement of python/pplx_garden/kernels/p2p_all_to_all.py:92-114,
+    and the DeepSeek decode value that those lines give (9216 rows)."""
+    from a2a_cases import BASELINE_CASES
+    for case in BASELINE_CASES:
+        _, ops = make_ops(case, DEV)
+        try:
+            Le, private, recv = oracle.buffer_capacity(case.num_tokens, case.num_experts, case.topk,
+                                                       case.world_size, 1, case.expert_padding)
+            for op in ops:
+                assert (op.num_local_experts, op.max_private_tokens, op.max_recv_tokens) == (Le, private, recv)
+            if case is C2:
+                assert ops[0].max_recv_tokens == 9216 and ops[0].max_private_tokens == 128
+        finally:
+            for op in ops:
+                op.destroy()

@@ -114,6 +114,29 @@ def test_static_dispatch_refuses_what_its_fixed_tables_cannot_hold():
     assert int(header_bytes.group(1)) << int(header_bytes.group(2)) == native.STATIC_SCRATCH_BYTES
 
 
+def test_operator_capacities_match_the_oracle_and_the_reference_values():
+    """Rows of a rank's receive region (python/pplx_garden/kernels/p2p_all_to_all.py:92-114): the
+    operator's arithmetic against the oracle's on the five baseline shapes, the 1-token configuration
+    of the reference's test matrix, dp groups, and the value the reference's sizes give for the
+    DeepSeek decode shape (Le 32, average int(4 * 1.2) = 4, private 128, 128 * 8 + 8192 = 9216)."""
+    from a2a_cases import BASELINE_CASES
+    from pplx_garden_amd.kernels.p2p_all_to_all import P2PAllToAll
+    shapes = [(c.num_tokens, c.num_experts, c.topk, c.world_size, 1, c.expert_padding, None) for c in BASELINE_CASES]
+    shapes += [(1, 2, 1, 2, 1, 1, 32), (8, 16, 2, 2, 1, 16, None), (1, 4, 1, 4, 2, 1, None), (8, 4, 4, 4, 2, 1, None),
+               (128, 16, 2, 2, 1, 1, 8), (4096, 256, 8, 8, 1, 1, 0), (64, 384, 8, 16, 4, 128, None)]
+    for T, E, K, N, D, pad, private in shapes:
+        got = P2PAllToAll.receive_capacity(max_num_tokens=T, num_experts=E, expert_padding=pad,
+                                           num_experts_per_token=K, world_size=N, dp_size=D,
+                                           max_private_tokens=private)
+        Le, want_private, want_recv = oracle.buffer_capacity(T, E, K, N, D, pad, private)
+        assert got == (want_private, want_recv), (T, E, K, N, D, pad, private)
+        assert Le == ceil_div(E, N)
+    assert P2PAllToAll.receive_capacity(max_num_tokens=128, num_experts=256, expert_padding=1,
+                                        num_experts_per_token=8, world_size=8) == (128, 9216)
+    assert P2PAllToAll.receive_capacity(max_num_tokens=1, num_experts=2, expert_padding=1,
+                                        num_experts_per_token=1, world_size=2, max_private_tokens=32) == (32, 66)
+
+
 def test_strides_match_the_oracle():
     lib = native.load_library()
     for H, ie, Hs, se, oe in [(7168, 1, 56, 4, 2), (2048, 1, 16, 4, 2), (128, 4, 0, 0, 4), (16, 2, 0, 0, 2),
