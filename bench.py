@@ -13,37 +13,37 @@ of all 8 logical ranks, which is one GPU's share of the group's work.  Routing
 changes every step (a few pre-generated routings are cycled), as in the
 reference's benchmark (benchmarks/bench_all_to_all.py:382-389).
 
-Prints one JSON line.  `value` is algorithmic bytes per step over the wall time
-of the timed region; per-phase times come from events recorded on the stream
-the kernels run on, around about 25 steps of the same region (an event between
-two launches idles the GPU for about 3 us, so they are kept sparse).  The 128-token decode shape is timed too and reported in
-the same line.  The CPU baseline is the oracle's C restatement, single thread,
-on the same workload.
+Prints one JSON line.  Order of the run:
+ 1. a pass of at least 200 steps that carries events, as the reference's benchmark does
+    (around each phase of every step); every fourth step instead has the pack, the gather and
+    the routing launch record events at their own start and end: those are the kernels' own
+    durations, the samples behind `roofline`;
+ 2. the timed region: W warm-up steps, then exactly K steps between two synchronisations with
+    no event in between; `value` is algorithmic bytes per step over that wall time;
+ 3. the same K steps as replays of a captured HIP graph (reported beside it);
+ 4. the other shapes of the baseline (128-token decode at both hidden sizes, the 1024-token
+    mixed batch) and the CPU baselines.
 """
 
 from __future__ import annotations
 
 import argparse
-import ctypes
+import hashlib
 import json
 import os
+import re
 import sys
 import time
 from dataclasses import replace
 from pathlib import Path
 
 REPO = Path(__file__).resolve().parent
-for _p in (REPO / "pplx-garden_amd", REPO / "oracle", REPO / "tests"):
+for _p in (REPO / "pplx-garden_amd", REPO / "pplx-garden_amd" / "benchmarks"):
     if str(_p) not in sys.path:
         sys.path.insert(0, str(_p))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-
-# HBM bytes per launch on the default workload, from hardware counters (FETCH_SIZE and WRITE_SIZE
-# passes, scaled by what the same counters read for a 512 MiB copy: x2.000 and x1.000).  The counter
-# runs and their commands are summarised in profiles/hbm_traffic_dsv3_prefill_4096_pack_and_combine.md.
-MEASURED_TRAFFIC_BYTES = {"combine_gather_kernel": 531_696_000, "dispatch_resolve_kernel": 303_561_000,
-                          "dispatch_push_kernel": 303_073_000}
+TRAFFIC_PROFILE = REPO / "profiles" / "hbm_traffic_dsv3_prefill_4096_pack_and_combine.md"
 
 
 def algorithmic_bytes(T: int, H: int, K: int):
@@ -55,13 +55,37 @@ def algorithmic_bytes(T: int, H: int, K: int):
     return dispatch, combine
 
 
+def kernel_sources_sha256() -> str:
+    """Fingerprint of the kernel sources this run uses: sha256 over the names and contents of
+    pplx-garden_amd/csrc/*, sorted by name."""
+    h = hashlib.sha256()
+    for path in sorted((REPO / "pplx-garden_amd" / "csrc").iterdir()):
+        if path.is_file():
+            h.update(path.name.encode() + b"\0" + path.read_bytes() + b"\0")
+    return h.hexdigest()
+
+
+def measured_traffic():
+    """HBM bytes per launch from the hardware-counter summary under profiles/, or {} when that
+    summary was taken on other kernel sources than the ones this run uses (then it says nothing
+    about this build)."""
+    try:
+        text = TRAFFIC_PROFILE.read_text()
+    except OSError:
+        return {}, "no counter summary under profiles/"
+    sha = re.search(r"^csrc_sha256:\s*([0-9a-f]{64})\s*$", text, flags=re.M)
+    if sha is None or sha.group(1) != kernel_sources_sha256():
+        return {}, "the counter summary under profiles/ was taken on other kernel sources"
+    out = {m.group(1): int(m.group(2)) for m in re.finditer(r"^traffic_bytes:\s*(\w+)\s*=\s*(\d+)\s*$", text, flags=re.M)}
+    return out, f"FETCH_SIZE and WRITE_SIZE passes of this build, {TRAFFIC_PROFILE.relative_to(REPO)}"
+
+
 class Workload:
     """Buffers of one case with the GPU as rank 0 of N logical ranks."""
 
     def __init__(self, case, device, num_routings: int, context_flags: int = 0):
         import torch
-        from a2a_cases import make_rank
-        from a2a_harness import rows_needed
+        from workloads import make_rank, rows_needed
         from pplx_garden_amd.native.p2p_all_to_all import (A2ACombineArgs, A2ADispatchArgs,
                                                            AllToAllContext)
 
@@ -142,17 +166,18 @@ class Workload:
         self.ctx.destroy()
 
 
-def time_workload(wl: Workload, steps: int, warmup: int, kernel_every: int = 32, call_every: int = 0,
+def time_workload(wl: Workload, steps: int, warmup: int, kernel_every: int = 0, call_every: int = 0,
                   route_events: bool = False):
     """W untimed steps, then exactly K timed steps between two synchronisations.
 
     Events cost idle GPU time (measured on the 4096-token step: 146.8 us per step without events,
     152.5 us with one after each call; a launch that records its own start and end costs about 3 us
-    more), so the timed region carries them sparsely.  Every `kernel_every`-th step has the library record
-    events at the start and end of the pack and the gather kernel themselves: the kernels' own durations
-    (with `route_events` also of the routing launch, where the step has one).  Every `call_every`-th
-    step (0 = none), never one of those, carries three events around the two calls (before the dispatch,
-    between dispatch and combine, after the combine).
+    more), so the timed region of the headline carries none (`kernel_every` = `call_every` = 0).
+    With `kernel_every` > 0 every such step has the library record events at the start and end of
+    the pack and the gather kernel themselves: the kernels' own durations (with `route_events` also
+    of the routing launch, where the step has one).  Every `call_every`-th step (0 = none), never
+    one of those, carries three events around the two calls (before the dispatch, between dispatch
+    and combine, after the combine).
 
     Returns wall seconds and, in microseconds per sampled step: dispatch call, combine call, both,
     pack kernel, gather kernel, routing kernel (empty without `route_events`, or when the dispatch
@@ -162,8 +187,6 @@ def time_workload(wl: Workload, steps: int, warmup: int, kernel_every: int = 32,
     kernel_steps = []
     if kernel_every > 0:
         kernel_steps = [i for i in range(steps) if i % kernel_every == kernel_every // 2]
-        if not kernel_steps and steps > 0:      # a very short run still gets a sample
-            kernel_steps = [steps // 2]
     call_steps = [i for i in range(steps) if call_every > 0 and i % call_every == 0 and i not in kernel_steps]
     call_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(3)] for i in call_steps}
     kern_ev = {i: [torch.cuda.Event(enable_timing=True) for _ in range(6 if route_events else 4)]
@@ -197,17 +220,50 @@ def time_workload(wl: Workload, steps: int, warmup: int, kernel_every: int = 32,
     return wall_s, disp, comb, both, pack, gather, route
 
 
+def time_graph_replay(wl: Workload, steps: int, warmup: int):
+    """The same steps as replays of ONE captured HIP graph that holds a step per routing (the calls
+    only enqueue kernels whose arguments travel by value, so they can be recorded; graph capture
+    is a stated feature of the reference, docs/fabric-lib.md:15).  Returns wall seconds per step."""
+    import torch
+    n = len(wl.routings)
+    side = torch.cuda.Stream(device=wl.device)
+    side.wait_stream(torch.cuda.current_stream(wl.device))
+    with torch.cuda.stream(side):
+        for i in range(n):
+            wl.step(i, side.cuda_stream)
+    torch.cuda.current_stream(wl.device).wait_stream(side)
+    torch.cuda.synchronize(wl.device)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        stream = torch.cuda.current_stream(wl.device).cuda_stream
+        for i in range(n):
+            wl.step(i, stream)
+    replays = max(1, -(-steps // n))
+    for _ in range(max(1, -(-warmup // n))):
+        graph.replay()
+    torch.cuda.synchronize(wl.device)
+    t0 = time.perf_counter()
+    for _ in range(replays):
+        graph.replay()
+    torch.cuda.synchronize(wl.device)
+    wall_s = time.perf_counter() - t0
+    flags = wl.ctx.status(torch.cuda.current_stream(wl.device).cuda_stream)
+    if flags:
+        raise RuntimeError(f"device error flags {flags}")
+    del graph
+    return wall_s / (replays * n), replays * n
+
+
 def cpu_baseline(case, rd, reps: int, threads: int = 1):
     """The oracle's C restatement on the same batch; best of `reps`.  Returns seconds per step and the
     seconds of its routing part (histogram, ranks, receiver layout: what the reference does on one host
-    thread, a2a_worker.rs:526-703)."""
+    thread, a2a_worker.rs:526-703).  The only part of this file that touches oracle/."""
     import numpy as np
-    from a2a_cases import bf16_codes
-    from a2a_harness import rows_needed
+    from workloads import bf16_codes, make_rank, rows_needed
+    sys.path.insert(0, str(REPO / "oracle"))
     import c_oracle
 
     N = case.world_size
-    from a2a_cases import make_rank
     world = [rd] + [make_rank(case, r, 0) for r in range(1, N)]
     rows = rows_needed(case, world)
     cw = c_oracle.CWorld(case.num_experts, N, case.node_size or N, case.expert_padding,
@@ -235,17 +291,67 @@ def cpu_baseline(case, rd, reps: int, threads: int = 1):
     return best, route_best
 
 
+def cpu_baseline_numpy(case, tokens: int):
+    """The numpy oracle (array code, whatever threads numpy's kernels use: its element-wise loops run
+    on one) on a sample of `tokens` tokens of the same workload.  Returns seconds for the sample."""
+    import numpy as np
+    from workloads import bf16_codes, make_rank, rows_needed
+    sys.path.insert(0, str(REPO / "oracle"))
+    import a2a_oracle as oracle
+
+    N = case.world_size
+    world = [make_rank(case, 0, tokens)] + [make_rank(case, r, 0) for r in range(1, N)]
+    rows = rows_needed(case, world)
+    rng = np.random.default_rng(case.seed)
+    ys = [rng.integers(0x3C00, 0x4000, size=(rows, case.hidden_dim), dtype=np.uint16) for _ in range(N)]
+    t0 = time.perf_counter()
+    inputs = [oracle.RankInput(x=bf16_codes(w.x), indices=w.indices.numpy()) for w in world]
+    outs = oracle.dispatch_world(inputs, num_experts=case.num_experts, world_size=N,
+                                 node_size=case.node_size or N, expert_padding=case.expert_padding,
+                                 out_rows=rows, quantize=True)
+    oracle.combine_world(ys, [w.indices.numpy() for w in world], [w.weights.numpy() for w in world],
+                         outs[0].slots, num_experts=case.num_experts, world_size=N)
+    return time.perf_counter() - t0
+
+
+def other_shape(case, device, routings: int, steps: int, warmup: int, ctx_flags: int, label: str, bar_us=None):
+    """Wall time per step without events, the kernels' own durations from a pass with events, and the
+    calls' p50 from a pass with events around every call."""
+    from pplx_garden_amd.utils.math import Statistics
+    wl = Workload(case, device, routings, ctx_flags)
+    _, d, c, b, p, g, _ = time_workload(wl, steps, warmup, kernel_every=4, call_every=1)
+    w, _, _, _, _, _, _ = time_workload(wl, steps, warmup)
+    graph_s, _ = time_graph_replay(wl, steps, warmup)
+    wl.close()
+    d_bytes, c_bytes = algorithmic_bytes(case.num_tokens, case.hidden_dim, case.topk)
+    step_us = w / steps * 1e6
+    out = {
+        "workload": label,
+        "step_us_wall": round(step_us, 2),
+        "step_us_graph_replay": round(graph_s * 1e6, 2),
+        "pack_kernel_us_mean": round(Statistics.create(p).mean, 2),
+        "gather_kernel_us_mean": round(Statistics.create(g).mean, 2),
+        "kernel_samples": len(g),
+        "dispatch_us_p50": round(Statistics.create(d).p50, 2),
+        "combine_us_p50": round(Statistics.create(c).p50, 2),
+        "total_us_p50": round(Statistics.create(b).p50, 2),
+        "total_us_mean": round(Statistics.create(b).mean, 2),
+        "algorithmic_bytes": d_bytes + c_bytes,
+        "pct_of_hbm_peak": round(100.0 * (d_bytes + c_bytes) / (step_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 2),
+    }
+    if bar_us is not None:
+        out["bar_us_for_70pct"] = bar_us
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--routings", type=int, default=4, help="distinct routings cycled over the steps")
-    ap.add_argument("--kernel-every", type=int, default=0,
-                    help="every how many timed steps have the pack and the gather kernel record their own "
-                         "start and end (0 = about 12 such steps, at least 16 apart)")
     ap.add_argument("--cpu-reps", type=int, default=3, help="repetitions of the CPU baseline (0 = skip)")
-    ap.add_argument("--no-decode", action="store_true", help="skip the 128-token shape")
+    ap.add_argument("--no-decode", action="store_true", help="skip the shapes other than the 4096-token one")
     ap.add_argument("--decode-only", action="store_true",
                     help="time only the 128-token shape (for a kernel trace of the decode step alone)")
     ap.add_argument("--separate-routing", action="store_true",
@@ -256,14 +362,20 @@ def main() -> int:
     ap.add_argument("--probe-copy", action="store_true",
                     help="also run plain device-to-device copies of 512 MiB (torch's copy kernel): the "
                          "known-size kernel that hardware byte counters are scaled by")
+    ap.add_argument("--print-source-hash", action="store_true",
+                    help="print the fingerprint of the kernel sources (what a counter summary under "
+                         "profiles/ records as csrc_sha256) and exit")
     args = ap.parse_args()
+    if args.print_source_hash:
+        print(kernel_sources_sha256())
+        return 0
     if args.gpus != 1:
         print("bench.py measures one GPU: every logical rank of the expert-parallel group lives in "
               "this GPU's HBM and nothing here uses a second GPU; run with --gpus 1", file=sys.stderr)
         return 2
 
     import torch
-    from a2a_cases import C2, C3
+    from workloads import C1, C2, C3, C4
     from pplx_garden_amd.utils.math import Statistics
 
     if not torch.cuda.is_available():
@@ -283,29 +395,25 @@ def main() -> int:
     ctx_flags = 2 if args.separate_routing else 0   # A2A_FLAG_SEPARATE_ROUTING
     if args.context_flags is not None:
         ctx_flags = args.context_flags
-    if args.kernel_every <= 0:
-        args.kernel_every = max(16, args.steps // 12)
+    side_steps = max(args.steps, 200)
+    decode_label = ("DeepSeek-V3 decode: 128 tokens, hidden 7168, 256 experts / 8 logical ranks, top-8 uniform, "
+                    "1% x50 outliers")
     if args.decode_only:
-        wl2 = Workload(C2, device, args.routings, ctx_flags)
-        w2, _, _, _, p2, g2, _ = time_workload(wl2, args.steps, args.warmup, args.kernel_every)
-        _, d2, c2, b2, _, _, _ = time_workload(wl2, max(args.steps, 200), 0, 0, call_every=1)
-        wl2.close()
-        print(json.dumps({"decode_128_only": {"step_us_wall": round(w2 / args.steps * 1e6, 2),
-                                              "pack_kernel_us_mean": round(Statistics.create(p2).mean, 2),
-                                              "gather_kernel_us_mean": round(Statistics.create(g2).mean, 2),
-                                              "dispatch_us_p50": round(Statistics.create(d2).p50, 2),
-                                              "combine_us_p50": round(Statistics.create(c2).p50, 2),
-                                              "total_us_p50": round(Statistics.create(b2).p50, 2)}}))
+        print(json.dumps({"decode_128_only": other_shape(C2, device, args.routings, side_steps, args.warmup,
+                                                         ctx_flags, decode_label)}))
         return 0
 
     case = C3
     wl = Workload(case, device, args.routings, ctx_flags)
-    wall_s, _, _, _, pack, gather, _ = time_workload(wl, args.steps, args.warmup, args.kernel_every)
-    # Phase statistics as the reference's benchmark reports them (events around each phase of EVERY
-    # iteration, benchmarks/bench_all_to_all.py:391-433), outside the timed region above; every fourth
-    # step times the routing launch by its own events instead.
-    _, disp, comb, both, _, _, route = time_workload(wl, max(args.steps, 200), 0, 4, call_every=1,
-                                                     route_events=True)
+    # 1. Phase statistics as the reference's benchmark reports them (events around each phase of every
+    #    iteration, benchmarks/bench_all_to_all.py:391-433); every fourth step has the three kernels
+    #    record their own start and end instead: the samples of the roofline figures.
+    _, disp, comb, both, pack, gather, route = time_workload(wl, side_steps, args.warmup, kernel_every=4,
+                                                             call_every=1, route_events=True)
+    # 2. The timed region: no events.
+    wall_s, _, _, _, _, _, _ = time_workload(wl, args.steps, args.warmup)
+    # 3. The same as graph replays.
+    graph_step_s, graph_steps = time_graph_replay(wl, args.steps, args.warmup)
     rows = wl.rows
     cpu_rd = wl.cpu_first
     wl.close()
@@ -314,46 +422,40 @@ def main() -> int:
     ms_per_step = wall_s / args.steps * 1e3
     value = (d_bytes + c_bytes) / (ms_per_step * 1e-3) / 1e9
     p_stats, g_stats = Statistics.create(pack), Statistics.create(gather)
+    traffic, traffic_note = measured_traffic()
 
     def stats_dict(xs):
         return {k: round(v, 2) for k, v in Statistics.create(xs).as_dict().items()}
 
-    def roof(bytes_, mean_us, kernel, note):
-        achieved = bytes_ / (mean_us * 1e-6) / 1e9
+    def roof(bytes_, stats, samples, kernel):
+        achieved = bytes_ / (stats.mean * 1e-6) / 1e9
         return {"kernel": kernel, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                 "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                "traffic": MEASURED_TRAFFIC_BYTES.get(kernel), "bytes_per_launch": bytes_,
-                "avg_us": round(mean_us, 2), "timing": note}
+                "traffic": traffic.get(kernel), "traffic_source": traffic_note,
+                "bytes_per_launch": bytes_, "avg_us": round(stats.mean, 2), "p50_us": round(stats.p50, 2),
+                "samples": samples,
+                "timing": "events recorded by the launch itself at the start and end of this kernel "
+                          f"(hipExtLaunchKernelGGL), on every fourth of the {side_steps} steps of the pass "
+                          "that precedes the timed region"}
 
-    note = ("events recorded by the launch itself at the start and end of this kernel (hipExtLaunchKernelGGL), "
-            f"on {len(gather)} of the {args.steps} timed steps")
-    combine_roof = roof(c_bytes, g_stats.mean, "combine_gather_kernel", note)
-    dispatch_roof = roof(d_bytes, p_stats.mean,
-                         "dispatch_push_kernel" if args.separate_routing else "dispatch_resolve_kernel", note)
+    combine_roof = roof(c_bytes, g_stats, len(gather), "combine_gather_kernel")
+    dispatch_roof = roof(d_bytes, p_stats, len(pack),
+                         "dispatch_push_kernel" if args.separate_routing else "dispatch_resolve_kernel")
     dominant, other = ((combine_roof, dispatch_roof) if g_stats.mean >= p_stats.mean
                        else (dispatch_roof, combine_roof))
 
-    decode = None
+    decode = qwen = kimi = None
     if not args.no_decode:
-        wl2 = Workload(C2, device, args.routings, ctx_flags)
-        steps2 = max(args.steps, 200)
-        w2, _, _, _, p2, g2, _ = time_workload(wl2, steps2, args.warmup, args.kernel_every)
-        _, d2, c2, b2, _, _, _ = time_workload(wl2, steps2, 0, 0, call_every=1)
-        wl2.close()
-        decode = {
-            "workload": "DeepSeek-V3 decode: 128 tokens, hidden 7168, 256 experts / 8 logical ranks, top-8 uniform, 1% x50 outliers",
-            "step_us_wall": round(w2 / steps2 * 1e6, 2),
-            "pack_kernel_us_mean": round(Statistics.create(p2).mean, 2),
-            "gather_kernel_us_mean": round(Statistics.create(g2).mean, 2),
-            "dispatch_us_p50": round(Statistics.create(d2).p50, 2),
-            "combine_us_p50": round(Statistics.create(c2).p50, 2),
-            "total_us_p50": round(Statistics.create(b2).p50, 2),
-            "total_us_mean": round(Statistics.create(b2).mean, 2),
-            "note": "working set (26 MB) fits the 256 MB Infinity Cache and is not flushed between steps; "
-                    "step_us_wall is wall time over the timed steps, the kernel figures come from events the "
-                    "launches record themselves on a few of those steps, the p50 figures from a second pass "
-                    "with events around the calls of every step (each event adds about 3 us)",
-        }
+        decode = other_shape(C2, device, args.routings, side_steps, args.warmup, ctx_flags, decode_label)
+        decode["note"] = ("working set (26 MB) fits the 256 MB Infinity Cache and is not flushed between steps; "
+                          "step_us_wall is wall time over steps without events, the kernel figures come from "
+                          "events the launches record themselves, the p50 figures from events around the calls "
+                          "of every step (each event adds about 3 us)")
+        qwen = other_shape(C1, device, args.routings, side_steps, args.warmup, ctx_flags,
+                           "Qwen3-30B-A3B decode: 128 tokens, hidden 2048, 128 experts / 8 logical ranks, top-8 uniform")
+        kimi = other_shape(C4, device, args.routings, side_steps, args.warmup, ctx_flags,
+                           "Kimi-K2 mixed batch: 1024 tokens, hidden 7168, 384 experts / 16 logical ranks, top-8 "
+                           "Zipf(1.0), receive slots padded to 128 per expert", bar_us=37.0)
 
     cpu = cpu_more = None
     if args.cpu_reps > 0:
@@ -367,13 +469,22 @@ def main() -> int:
         }
         cores = min(16, os.cpu_count() or 1)
         dt_all, _ = cpu_baseline(case, cpu_rd, args.cpu_reps, threads=cores)
+        sample_tokens = 1024
+        dt_np = cpu_baseline_numpy(case, sample_tokens)
+        s_d, s_c = algorithmic_bytes(sample_tokens, case.hidden_dim, case.topk)
         cpu_more = {
             "routing_only_us_one_thread": round(route_dt * 1e6, 1),
             "all_cores": {"value": round((d_bytes + c_bytes) / dt_all / 1e9, 3), "unit": "GB/s", "cores": cores,
                           "us_per_step": round(dt_all * 1e6, 1),
                           "note": "same code, tokens split over OpenMP threads; routing stays on one thread"},
+            "numpy_oracle": {"value": round((s_d + s_c) / dt_np / 1e9, 3), "unit": "GB/s",
+                             "cores": 1, "seconds": round(dt_np, 2),
+                             "sample": f"{sample_tokens} tokens of the same workload through the numpy oracle "
+                                       "(array code; numpy's element-wise loops use one thread whatever the "
+                                       f"host has: {os.cpu_count()} cores here)"},
         }
 
+    graph_value = (d_bytes + c_bytes) / graph_step_s / 1e9
     line = {
         "metric": "dispatch+combine µs & HBM GB/s (% peak), DSv3 shape, 128 and 4096 tokens",
         "value": round(value, 1),
@@ -398,22 +509,28 @@ def main() -> int:
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
         "prefill_4096": {
             "step_us_wall": round(ms_per_step * 1e3, 2),
-            "timed_steps_with_kernel_events": len(gather),
-            "pack_kernel_us": {"p50": round(p_stats.p50, 2), "mean": round(p_stats.mean, 2)},
-            "gather_kernel_us": {"p50": round(g_stats.p50, 2), "mean": round(g_stats.mean, 2)},
+            "graph_replay": {"step_us_wall": round(graph_step_s * 1e6, 2), "steps": graph_steps,
+                             "value": round(graph_value, 1),
+                             "pct_of_hbm_peak": round(100.0 * graph_value / HBM_PEAK_GBS, 2),
+                             "note": f"one captured HIP graph of {args.routings} steps (one per routing), replayed"},
+            "pack_kernel_us": {"p50": round(p_stats.p50, 2), "mean": round(p_stats.mean, 2), "samples": len(pack)},
+            "gather_kernel_us": {"p50": round(g_stats.p50, 2), "mean": round(g_stats.mean, 2), "samples": len(gather)},
+            "route_kernel_us": ({"p50": round(Statistics.create(route).p50, 2),
+                                 "mean": round(Statistics.create(route).mean, 2), "samples": len(route)}
+                                if route else None),
             "algorithmic_bytes": {"dispatch": d_bytes, "combine": c_bytes},
             "with_events_on_every_step": {
-                "note": "a second pass outside the timed region, events around each phase of every iteration as "
-                        "in the reference's benchmark (each event adds about 3 us); every fourth step has the "
-                        "routing launch record its own start and end instead",
+                "note": f"the pass of {side_steps} steps before the timed region, events around each phase of every "
+                        "iteration as in the reference's benchmark (each event adds about 3 us); every fourth step "
+                        "has the three kernels record their own start and end instead",
                 "dispatch_us": stats_dict(disp),
                 "combine_us": stats_dict(comb),
                 "total_us": stats_dict(both),
-                "route_kernel_us": ({"p50": round(Statistics.create(route).p50, 2),
-                                     "mean": round(Statistics.create(route).mean, 2)} if route else None),
             },
         },
         "decode_128": decode,
+        "qwen3_decode_128": qwen,
+        "kimi_1024": kimi,
         "roofline": dominant,
         "roofline_other": other,
         "cpu_baseline": cpu,

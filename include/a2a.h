@@ -77,7 +77,8 @@ typedef struct a2a_config {
     uint32_t scale_elemsize;         /* 0 or 4 */
     uint32_t max_num_tokens;         /* per rank and step */
     uint32_t max_recv_tokens;        /* rows of a rank's staging region */
-    uint32_t max_private_tokens;     /* accepted for parity; selects no code path in loopback */
+    uint32_t max_private_tokens;     /* rows per source in the private part of a receive region: moves no row
+                                        in loopback, but the offset tables of a2a_dispatch_recv encode it */
     uint32_t num_experts;            /* E <= A2A_MAX_EXPERTS */
     uint32_t expert_padding;         /* each expert's slot range is rounded up to this */
     uint32_t num_experts_per_token;  /* K <= A2A_MAX_EXPERTS_PER_TOKEN */
@@ -276,7 +277,11 @@ typedef enum a2a_table {
     A2A_TABLE_PADDED_INDEX = 4,     /* [num_recv] a2a_worker.rs:669-671 (split calls only) */
     A2A_TABLE_SOURCE_RANK = 5,      /* [num_recv] a2a_worker.rs:668 (split calls only) */
     A2A_TABLE_SOURCE_POSITION = 6,  /* [num_recv] row in the sender's expert-sorted order (split calls only) */
-    A2A_TABLE_NUM_RECV_TOKENS = 7   /* [1] (split calls only) */
+    A2A_TABLE_NUM_RECV_TOKENS = 7,  /* [2] rows received, rows from other nodes (split calls only) */
+    A2A_TABLE_SOURCE_DISPATCH_OFFSET = 8,  /* [num_recv] a2a_worker.rs:636-656: private-region row,
+                                              sender's position with bit 31 set (same node), or
+                                              overflow-region row (split calls only) */
+    A2A_TABLE_COMBINE_SEND_OFFSET = 9      /* [num_recv] a2a_worker.rs:659-667 (split calls only) */
 } a2a_table;
 
 int a2a_ctx_read_table(a2a_ctx *ctx, uint32_t rank, uint32_t which,

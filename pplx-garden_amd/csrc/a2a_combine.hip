@@ -140,14 +140,8 @@ __device__ __forceinline__ void fma_chunk(const u32x4 raw, float w, float (&acc)
     }
 }
 
-#ifndef A2A_COMBINE_WAVES
-#define A2A_COMBINE_WAVES 1
-#endif
-#ifndef A2A_COMBINE_CHUNKS
-#define A2A_COMBINE_CHUNKS 1
-#endif
-constexpr int kCombineWaves = A2A_COMBINE_WAVES;    // wavefronts per workgroup; each works on its own
-constexpr int kCombineChunks = A2A_COMBINE_CHUNKS;  // 16-byte chunks of a row per lane
+constexpr int kCombineWaves = 1;    // wavefronts per workgroup; each works on its own
+constexpr int kCombineChunks = 1;   // 16-byte chunks of a row per lane
 constexpr int kSlabChunks = kWave * kCombineChunks;
 
 // T: type of the expert_y rows, U: type of out_tokens.  One WAVEFRONT handles
@@ -227,11 +221,7 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
     float acc[kCombineChunks][V];
 #pragma unroll
     for (int u = 0; u < kCombineChunks; ++u) {
-#ifdef A2A_COMBINE_ADJ
-        c[u] = slab * kSlabChunks + lane * kCombineChunks + u;
-#else
         c[u] = slab * kSlabChunks + u * kWave + lane;
-#endif
         active[u] = c[u] < num_chunks;
         out_chunk[u] = dst.out + (size_t)token * dst.out_stride + (size_t)c[u] * V * Elem<U>::kSize;
 #pragma unroll

@@ -27,9 +27,16 @@ struct a2a_ctx {
     void *arena = nullptr;
     size_t arena_bytes = 0;
     std::string error;
+    // A HIP call failed on this context (a launch, a copy): what was enqueued before it may have
+    // left the routing tables half updated (the two copies of the step totals are handed over by
+    // the launch that consumes them), so every later step would be wrong without saying so.
+    // The context refuses further work; destroy it.
+    bool poisoned = false;
+    std::string first_failure;
 
     // State of the current step.
     uint32_t sent_mask = 0;        // split calls: ranks whose dispatch_send ran in this step
+    uint32_t empty_mask = 0;       // split calls: those of them that sent no tokens (no launch, tables untouched)
     bool step_open = false;        // split calls: a send has run and no recv yet closed the step
     bool recv_seen = false;        // split calls: a recv has run in this step
     bool group_routing = false;    // the last dispatch was a group call (route_slot is valid)
@@ -67,7 +74,19 @@ int fail(a2a_ctx *ctx, int code, const char *fmt, ...) {
 }
 
 int hip_fail(a2a_ctx *ctx, hipError_t e, const char *what) {
-    return fail(ctx, (int)e, "%s: %s", what, hipGetErrorString(e));
+    const int rc = fail(ctx, (int)e, "%s: %s", what, hipGetErrorString(e));
+    if (ctx != nullptr && !ctx->poisoned) {
+        ctx->poisoned = true;
+        ctx->first_failure = ctx->error;
+    }
+    return rc;
+}
+
+// Entry check of every call that enqueues work on a context.
+int check_usable(a2a_ctx *ctx) {
+    if (!ctx->poisoned) return A2A_OK;
+    return fail(ctx, A2A_ERR_BAD_ORDER, "this context is unusable after an earlier failure (%s): destroy it",
+                ctx->first_failure.c_str());
 }
 
 size_t align_up(size_t n, size_t a) { return (n + a - 1) / a * a; }
@@ -222,14 +241,12 @@ uint32_t rows_upper_bound(const a2a_ctx *ctx) {
 // and all entries in every receiver workgroup: quadratic in the chunks of a
 // source.  Measured at 8 entries per token: 2 us faster than the two-launch
 // pass up to 8 chunks per source, equal at 16, 4 us slower at 32.
-#ifndef A2A_FUSED_MAX_CHUNKS
-#define A2A_FUSED_MAX_CHUNKS 12
-#endif
+constexpr uint32_t kFusedMaxChunks = 12;
 bool fused_routing_pays(const FinalizeArgs &fa, uint32_t world, uint32_t total_blocks) {
     for (uint32_t r = 0; r < world; ++r) {
-        if (fa.num_blocks[r] > A2A_FUSED_MAX_CHUNKS) return false;
+        if (fa.num_blocks[r] > kFusedMaxChunks) return false;
     }
-    return total_blocks <= 4 * A2A_FUSED_MAX_CHUNKS;
+    return total_blocks <= 4 * kFusedMaxChunks;
 }
 
 // Dimensions of the device workspace for steps of at most `max_tokens` tokens per
@@ -574,6 +591,7 @@ int a2a_ctx_status(a2a_ctx *ctx, void *stream, uint32_t *flags) {
 
 int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize, void *stream) {
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (int rc = check_usable(ctx)) return rc;
     if (args == nullptr) return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "null args");
     DeviceGuard guard(ctx->cfg.device);
     const KernelTiming pack_timing = ctx->timing[A2A_KERNEL_PACK];
@@ -586,6 +604,7 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
     ctx->group_routing = true;
     ctx->step_open = false;
     ctx->sent_mask = 0;
+    ctx->empty_mask = 0;
     ctx->quantized = quantize;
     return A2A_OK;
 }
@@ -635,6 +654,7 @@ int a2a_dispatch_static(const a2a_config *config, const a2a_dispatch_args *args,
 int a2a_combine(a2a_ctx *ctx, const a2a_combine_args *args, uint32_t expert_y_dtype,
                 uint32_t accumulate, void *stream) {
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (int rc = check_usable(ctx)) return rc;
     if (args == nullptr) return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "null args");
     const a2a_config &c = ctx->cfg;
     const uint32_t N = c.world_size;
@@ -737,6 +757,8 @@ int a2a_ctx_read_table(a2a_ctx *ctx, uint32_t rank, uint32_t which, uint32_t *ou
         case A2A_TABLE_SOURCE_RANK:
         case A2A_TABLE_SOURCE_POSITION:
         case A2A_TABLE_NUM_RECV_TOKENS:
+        case A2A_TABLE_SOURCE_DISPATCH_OFFSET:
+        case A2A_TABLE_COMBINE_SEND_OFFSET:
             src = staging_table(ctx->staging, ctx->cfg, receiver, which, &limit);
             if (src == nullptr)
                 return fail(ctx, A2A_ERR_BAD_ORDER, "receive tables exist only after a2a_dispatch_recv");
@@ -745,6 +767,11 @@ int a2a_ctx_read_table(a2a_ctx *ctx, uint32_t rank, uint32_t which, uint32_t *ou
             return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "unknown table %u", which);
     }
     if (count > limit) return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "count %zu exceeds the table (%zu)", count, limit);
+    if (which <= A2A_TABLE_TOKEN_OFFSET && !ctx->group_routing && (ctx->empty_mask >> rank & 1)) {
+        // a split send without tokens launches nothing and leaves its tables alone: they read as zeros
+        memset(out, 0, count * sizeof(uint32_t));
+        return A2A_OK;
+    }
     DeviceGuard guard(ctx->cfg.device);
     hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return hip_fail(ctx, e, "hipStreamSynchronize");
@@ -765,18 +792,27 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     (void)weights;
     (void)weights_stride;
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (int rc = check_usable(ctx)) return rc;
     if (int rc = check_rank(ctx, rank)) return rc;
     if (int rc = check_send(ctx, ctx->cfg, rank, num_tokens, x_ptr, x_stride, quantize, x_scale_ptr, indices))
         return rc;
     const a2a_config &c = ctx->cfg;
     DeviceGuard guard(c.device);
     if (!ctx->staging.allocated) {
+        // the first split call of a context allocates the staging: not while a stream is being captured
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capture) == hipSuccess &&
+            capture != hipStreamCaptureStatusNone)
+            return fail(ctx, A2A_ERR_BAD_ORDER,
+                        "the first a2a_dispatch_send of a context allocates its staging buffers, which a stream "
+                        "capture forbids: create the context with A2A_FLAG_PREALLOC_STAGING");
         std::string msg;
         if (int rc = staging_allocate(ctx->staging, c, &msg)) return fail(ctx, rc, "%s", msg.c_str());
     }
     // A send after a recv starts a new step.
     if (!ctx->step_open || ctx->recv_seen) {
         ctx->sent_mask = 0;
+        ctx->empty_mask = 0;
         ctx->recv_seen = false;
         ctx->step_open = true;
         ctx->staging.recv_mask = 0;
@@ -791,6 +827,17 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     // The sender is the rank's dp group; when several members of a group send, each repeats
     // the same routing and stages the same rows.
     const uint32_t group = rank / c.dp_size;
+    if (T == 0) {
+        // Nothing to route or stage: no launch.  The receivers of this step count the source as
+        // empty (it is left out of their mask of valid sources) and its tables read as zeros.
+        ctx->sent_mask |= 1u << group;
+        ctx->empty_mask |= 1u << group;
+        ctx->num_tokens[group] = 0;
+        ctx->quantized = quantize;
+        ctx->group_routing = false;
+        return A2A_OK;
+    }
+    ctx->empty_mask &= ~(1u << group);
     StageSendArgs sa;
     memset(&sa, 0, sizeof sa);
     sa.rank = rank;
@@ -858,6 +905,7 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
                       size_t out_x_scale_stride_elem, size_t out_x_scale_stride_token,
                       void *stream) {
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (int rc = check_usable(ctx)) return rc;
     if (int rc = check_rank(ctx, rank)) return rc;
     if (!ctx->step_open || ctx->sent_mask == 0)
         return fail(ctx, A2A_ERR_BAD_ORDER, "a2a_dispatch_recv before any a2a_dispatch_send of the step");
@@ -871,7 +919,7 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
     StageRecvArgs rv;
     memset(&rv, 0, sizeof rv);
     rv.rank = rank;
-    rv.valid_mask = ctx->sent_mask;
+    rv.valid_mask = ctx->sent_mask & ~ctx->empty_mask;
     rv.dst.out_x = static_cast<uint8_t *>(out_x);
     rv.dst.out_scale = out_x_scale;
     rv.dst.out_stride = out_x_stride;
@@ -882,6 +930,7 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
     rv.row_bytes = (uint32_t)row_bytes_of(c);
     rv.hidden_dim_scale = c.hidden_dim_scale;
     rv.max_rows = rows_upper_bound(ctx);
+    rv.max_private = c.max_private_tokens;
     hipError_t e = launch_stage_recv(rv, ctx->ws, ctx->staging, s);
     if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_recv");
     ctx->recv_seen = true;
@@ -892,6 +941,7 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
 int a2a_combine_send(a2a_ctx *ctx, uint32_t rank, const void *expert_y, size_t expert_y_stride,
                      size_t expert_y_rows, void *stream) {
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (int rc = check_usable(ctx)) return rc;
     if (int rc = check_rank(ctx, rank)) return rc;
     if (!ctx->staging.allocated || !(ctx->staging.recv_mask >> rank & 1))
         return fail(ctx, A2A_ERR_BAD_ORDER, "a2a_combine_send before a2a_dispatch_recv of rank %u", rank);
@@ -929,6 +979,7 @@ int a2a_combine_recv(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, size_t num_
                      void *stream) {
     (void)num_recv_tokens;
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    if (int rc = check_usable(ctx)) return rc;
     if (int rc = check_rank(ctx, rank)) return rc;
     const a2a_config &c = ctx->cfg;
     if (!ctx->staging.allocated || ctx->staging.combine_sent_mask == 0)

@@ -133,10 +133,7 @@ __device__ __forceinline__ uint32_t resolve_copy(const PushDst &dst, const Works
 
 uint32_t push_threads(const PushArgs &args, bool quantize) {
     const uint32_t chunks = quantize ? args.hidden_dim / 16 : args.row_bytes / 16;
-#ifndef A2A_PUSH_SLABS
-#define A2A_PUSH_SLABS 1
-#endif
-    uint32_t threads = ((chunks + kWave - 1) / kWave + A2A_PUSH_SLABS - 1) / A2A_PUSH_SLABS * kWave;
+    uint32_t threads = (chunks + kWave - 1) / kWave * kWave;
     if (threads < (uint32_t)kWave) threads = kWave;
     if (threads > 1024) threads = 1024;
     return threads;
@@ -218,8 +215,17 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
 // The counting is redundant: its cost grows with tokens x entries, so the host
 // takes this path only below a bound on the entries of a step.
 //
+//
+// SINGLE: the common shape of a decode step on one GPU's share: exactly one
+// source has tokens and its index rows are dense (stride K).  Then the entries
+// of the step are one flat array, read directly: no table of where every
+// token's ids are (building it costs a trip to memory before the counting can
+// start), no division of entry numbers, and no copies of other sources to
+// place before mine, so the order in which receivers lay out their sources
+// drops out too.
+//
 // Dynamic LDS: (G + 3) * E words and 8 bytes per token of the step.
-template <bool QUANT>
+template <bool QUANT, bool SINGLE>
 __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs args, const FinalizeArgs fin,
                                                               const Workspace ws) {
     extern __shared__ uint64_t s_dyn64[];
@@ -245,7 +251,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     // bound.  This is what the counting pass below looks up per entry.
     const uint32_t table_words = ((G + 3) * E + 1) & ~1u;
     uint64_t *tok_ids = reinterpret_cast<uint64_t *>(s_dyn + table_words);
-    for (uint32_t ft = tid; ft < total_tokens; ft += blockDim.x) {
+    for (uint32_t ft = tid; !SINGLE && ft < total_tokens; ft += blockDim.x) {
         // token_start is non-decreasing and equals the total from G on, so the
         // fixed trip count is safe and lets the loads go out together
         uint32_t g = 0, start = 0;
@@ -267,13 +273,24 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     uint32_t *rows_before = prior + E;                      // [E] padded rows of all experts before e
     uint32_t *copies_before = rows_before + E;              // [E] copies of the sources laid out before mine
     const uint32_t table = receiver ? G * Le : G * E + E;
-    for (uint32_t i = tid; i < table; i += blockDim.x) s_dyn[i] = 0;
+    if (SINGLE && !receiver) {
+        // only the row of the one source and the counts before my token are used
+        for (uint32_t i = tid; i < E; i += blockDim.x) {
+            s_dyn[(args.single_source - 1) * E + i] = 0;
+            s_dyn[G * E + i] = 0;
+        }
+    } else {
+        for (uint32_t i = tid; i < table; i += blockDim.x) s_dyn[i] = 0;
+    }
     uint32_t my_g = 0, token = 0;
-    if (!receiver) {
+    if constexpr (SINGLE) {
+        my_g = args.single_source - 1;      // receivers too: the one source they count
+        token = receiver ? 0 : blockIdx.x;
+    } else if (!receiver) {
         while (my_g + 1 < G && blockIdx.x >= args.token_start[my_g + 1]) ++my_g;
         token = blockIdx.x - args.token_start[my_g];
-        if (tid < ws.world) s_dst[tid] = args.dst[tid];
     }
+    if (!receiver && tid < ws.world) s_dst[tid] = args.dst[tid];
     // Sources without tokens have no workgroup of their own: the first receiver
     // workgroup (the first workgroup, if nobody receives) clears their tables.
     if (blockIdx.x == (fin.recv_mask != 0 ? total_tokens : 0)) {
@@ -288,26 +305,26 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     __syncthreads();
 
     // One pass over the entries of all sources, kBatch loads in flight per lane.
-#ifndef A2A_SMALL_BATCH
-#define A2A_SMALL_BATCH 8
-#endif
-    constexpr uint32_t kBatch = A2A_SMALL_BATCH;
+    constexpr uint32_t kBatch = 8;
     const PushSrc &src = args.src[my_g];
     const uint32_t rank = blockIdx.x - total_tokens;        // receivers only
     const uint32_t my_first = (args.token_start[my_g] + token) * K;   // flat index of my first entry
     uint32_t my_expert = 0xFFFFFFFFu;
     // The order in which every receiver lays out the sources comes from device
     // memory: asked for here, stored to LDS after the counting.
-    const uint32_t order_words = receiver ? 0 : ws.world * (kMaxWorld / 4);
+    const uint32_t order_words = receiver || SINGLE ? 0 : ws.world * (kMaxWorld / 4);
     const uint32_t order_word = tid < order_words ? ws.order[tid] : 0;
+    const uint32_t flat_entries = SINGLE ? effective_tokens(src.bound_m, src.num_tokens) * K : 0;
     for (uint32_t f0 = 0; f0 < total_entries || f0 == 0; f0 += kBatch * blockDim.x) {
         uint32_t expert[kBatch], src_of[kBatch];
 #pragma unroll
         for (uint32_t j = 0; j < kBatch; ++j) {
             const uint32_t f = f0 + j * blockDim.x + tid;
             expert[j] = 0xFFFFFFFFu;
-            src_of[j] = 0;
-            if (f < total_entries) {
+            src_of[j] = SINGLE ? my_g : 0;
+            if constexpr (SINGLE) {
+                if (f < flat_entries) expert[j] = (uint32_t)src.indices[f];
+            } else if (f < total_entries) {
                 const uint32_t flat_token = K > 1 ? __umulhi(f, args.topk_magic) : f;
                 const uint64_t ids = tok_ids[flat_token];
                 src_of[j] = (uint32_t)(ids >> 56);
@@ -350,7 +367,9 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     for (uint32_t e0 = 0; e0 < E; e0 += blockDim.x) {
         const uint32_t e = e0 + tid;
         uint32_t total = 0, before = 0;
-        if (e < E) {
+        if (SINGLE) {
+            total = e < E ? cnt[my_g * E + e] : 0;   // nobody else sends: nothing is laid out before mine
+        } else if (e < E) {
             const uint32_t r = owner_of_expert(ws, e);
             bool seen = false;
             // eight sources at a time, their LDS reads in flight together
@@ -615,7 +634,7 @@ bool dispatch_small_fits(const PushArgs &args, const Workspace &ws, bool quantiz
     // sources and 8 entries per token against the two-launch dispatch: 13.0 against 15.4 us at
     // 256 tokens x 2048 entries, 17.0 against 16.3 us at 512 x 4096, 32.8 against 25.8 us at
     // 1024 x 8192.
-    return entries <= A2A_SMALL_MAX_ENTRIES && entries * total_tokens <= A2A_SMALL_MAX_VISITS &&
+    return entries <= kSmallMaxEntries && entries * total_tokens <= kSmallMaxVisits &&
            total_tokens <= 1024 && table <= 8192 + 3072 &&
            ws.experts_per_rank <= push_threads(args, quantize);
 }
@@ -627,13 +646,25 @@ hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, 
     if (blocks == 0) return hipSuccess;
     const size_t table_words = (((size_t)ws.num_groups + 3) * ws.num_experts + 1) & ~(size_t)1;
     const size_t lds = table_words * sizeof(uint32_t) + (size_t)total_tokens * sizeof(uint64_t);
-    if (quantize) {
-        hipExtLaunchKernelGGL(dispatch_small_kernel<true>, dim3(blocks), dim3(threads), lds, stream, timing.start,
-                              timing.stop, 0, args, fin, ws);
-    } else {
-        hipExtLaunchKernelGGL(dispatch_small_kernel<false>, dim3(blocks), dim3(threads), lds, stream, timing.start,
-                              timing.stop, 0, args, fin, ws);
+    // One source with tokens whose index rows are dense: the flat-array variant.
+    PushArgs a = args;
+    a.single_source = 0;
+    uint32_t senders = 0;
+    for (uint32_t g = 0; g < ws.num_groups; ++g) {
+        if (args.src[g].num_tokens == 0) continue;
+        ++senders;
+        a.single_source = g + 1;
     }
+    if (senders != 1 || args.src[a.single_source - 1].indices_stride != ws.topk) a.single_source = 0;
+#define A2A_LAUNCH_SMALL(Q, S)                                                                                       \
+    hipExtLaunchKernelGGL((dispatch_small_kernel<Q, S>), dim3(blocks), dim3(threads), lds, stream, timing.start,  \
+                          timing.stop, 0, a, fin, ws)
+    if (quantize) {
+        if (a.single_source != 0) A2A_LAUNCH_SMALL(true, true); else A2A_LAUNCH_SMALL(true, false);
+    } else {
+        if (a.single_source != 0) A2A_LAUNCH_SMALL(false, true); else A2A_LAUNCH_SMALL(false, false);
+    }
+#undef A2A_LAUNCH_SMALL
     return hipGetLastError();
 }
 

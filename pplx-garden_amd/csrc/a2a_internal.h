@@ -107,6 +107,8 @@ struct PushArgs {
     uint32_t hidden_dim;
     uint32_t hidden_dim_scale;
     uint32_t topk_magic;                  // ceil(2^32 / K) (0 for K = 1): n / K = mulhi(n, magic) while n * K < 2^32
+    uint32_t single_source;               // one-launch dispatch of small steps: g + 1 when source g alone has tokens
+                                          // and its index rows are dense, else 0 (set by the launcher)
 };
 
 struct CombSrc {  // one per receiver rank: the expert outputs it holds
@@ -168,12 +170,8 @@ hipError_t launch_route_fused(const RouteArgs &args, const FinalizeArgs &fin, co
 hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool quantize,
                                 uint32_t total_tokens, hipStream_t stream, KernelTiming timing = KernelTiming());
 // One-launch routing + pack for small steps: whether a step qualifies, and the launch.
-#ifndef A2A_SMALL_MAX_ENTRIES
-#define A2A_SMALL_MAX_ENTRIES 8192
-#endif
-#ifndef A2A_SMALL_MAX_VISITS
-#define A2A_SMALL_MAX_VISITS (3u << 19)   // entries x tokens
-#endif
+constexpr uint32_t kSmallMaxEntries = 8192;
+constexpr uint32_t kSmallMaxVisits = 3u << 19;   // entries x tokens
 bool dispatch_small_fits(const PushArgs &args, const Workspace &ws, bool quantize, uint32_t total_tokens);
 hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
                                  bool quantize, uint32_t total_tokens, hipStream_t stream,

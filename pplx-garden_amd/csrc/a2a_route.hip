@@ -397,13 +397,6 @@ __global__ __launch_bounds__(kRouteBlock) void route_fused_kernel(const RouteArg
     }
 }
 
-// A step in which no source has tokens and nobody receives: only the tables of
-// the routed sources have to be cleared.  One workgroup.
-__global__ __launch_bounds__(kRouteBlock) void route_clear_empty_kernel(const FinalizeArgs fin,
-                                                                        const Workspace ws) {
-    clear_empty_sources(fin, ws);
-}
-
 // Two workgroups per logical rank, independent of each other: workgroup i folds
 // source i, workgroup N + i lays out receiver i.
 __global__ __launch_bounds__(kRouteBlock) void route_finalize_kernel(const FinalizeArgs args,
@@ -443,11 +436,8 @@ hipError_t launch_route_accumulate(const RouteArgs &args, const Workspace &ws, u
 hipError_t launch_route_fused(const RouteArgs &args, const FinalizeArgs &fin, const Workspace &ws,
                               hipStream_t stream) {
     const uint32_t blocks = args.block_start[ws.num_groups] + (fin.recv_mask != 0 ? ws.world : 0);
-    if (blocks != 0) {
-        hipLaunchKernelGGL(route_fused_kernel, dim3(blocks), dim3(kRouteBlock), 0, stream, args, fin, ws);
-    } else {
-        hipLaunchKernelGGL(route_clear_empty_kernel, dim3(1), dim3(kRouteBlock), 0, stream, fin, ws);
-    }
+    if (blocks == 0) return hipSuccess;   // nothing routed, nobody laid out
+    hipLaunchKernelGGL(route_fused_kernel, dim3(blocks), dim3(kRouteBlock), 0, stream, args, fin, ws);
     return hipGetLastError();
 }
 

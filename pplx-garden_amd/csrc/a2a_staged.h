@@ -10,7 +10,9 @@
 // Differences that follow from every rank living in one HBM: a token is staged
 // ONCE (quantised), not once per route, and the receiver finds it through a
 // position -> token table; the private / overflow split of the receive buffer
-// (max_private_tokens) does not exist.
+// (max_private_tokens) moves no row here, but the recv still writes the two
+// offset tables that encode it (source_dispatch_offset, combine_send_offset),
+// bit for bit what the reference's host worker computes.
 #pragma once
 
 #include <string>
@@ -28,6 +30,8 @@ struct Staging {
     uint32_t *padded_index = nullptr;    // [N][max_recv]
     uint32_t *source_rank = nullptr;     // [N][max_recv]
     uint32_t *source_position = nullptr; // [N][max_recv]
+    uint32_t *source_dispatch_offset = nullptr;  // [N][max_recv]  a2a_worker.rs:636-656
+    uint32_t *combine_send_offset = nullptr;     // [N][max_recv]  a2a_worker.rs:659-667
     uint32_t *num_recv = nullptr;        // [N][2]: received rows, rows from other nodes
     size_t disp_stride = 0;
     size_t comb_stride = 0;
@@ -57,6 +61,7 @@ struct StageRecvArgs {
     uint32_t hidden_dim_scale;
     uint32_t max_rows;        // upper bound of received rows known to the host
     uint32_t team_waves;      // wavefronts that share a row (set by the launcher)
+    uint32_t max_private;     // rows per source in the private part of a receive region (a2a_worker.rs:646-656)
 };
 
 struct CombineSendArgs {

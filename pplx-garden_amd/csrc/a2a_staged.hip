@@ -327,7 +327,7 @@ __device__ __forceinline__ void copy_row_by_team(const u32x4 *src, u32x4 *dst, u
 // and scales are copied from the sender's staged token
 // (a2a_dispatch_recv.cu:139-155).
 //
-// Dynamic LDS: 4 * G * Le + 1 words.
+// Dynamic LDS: 4 * G * Le + 1 + 2 * G words.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs args, const Workspace ws,
                                                           const Staging st) {
@@ -345,6 +345,8 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     uint32_t *excl = tot + items;        // [g][le]  position of the run in the sender's expert-sorted order
     uint32_t *run_row = excl + items;    // [i][le]  first row of the run in the receiver's buffer (i = order index)
     uint32_t *seg = run_row + items;     // [i][le]  first ARRIVAL index of the run; seg[items] = rows received
+    uint32_t *grp_dst = seg + items + 1; // [g]      position of source g's first row for this receiver in g's send order
+    uint32_t *grp_src = grp_dst + G;     // [g]      rows this receiver gets from the sources numbered below g
 
     for (uint32_t w = tid; w < items; w += blockDim.x) {
         const uint32_t g = Le > 1 ? __umulhi(w, ws.le_magic) : w;
@@ -355,6 +357,15 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
         excl[w] = live && e > 0 ? ws.expert_offsets[g * E + e - 1] : 0;
     }
     __syncthreads();
+    // Per source: where its rows for this receiver begin in its own send order (dst_group_offset,
+    // a2a_worker.rs:571-575) and how many rows the lower-numbered sources send here
+    // (src_group_offset, a2a_worker.rs:582-590: numeric order, not the order of arrival).
+    for (uint32_t g = tid; g < G; g += blockDim.x) {
+        grp_dst[g] = Le != 0 ? excl[g * Le] : 0;
+        uint32_t below = 0;
+        for (uint32_t w = 0; w < g * Le; ++w) below += tot[w];
+        grp_src[g] = below;
+    }
 
     // Rows per expert, padded offsets, first row of every run.
     const uint32_t pad = ws.expert_padding;
@@ -411,6 +422,7 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     if (tid == 0) seg[items] = total;
     __syncthreads();
     if (publish && tid == 0) {
+        if (total > st.max_recv) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
         st.num_recv[2 * r] = total;
         // rows that come from other nodes (num_efa_tokens, a2a_worker.rs:681-687)
         const uint32_t remote_segs = (ws.world / ws.node_size - 1) * (ws.node_size / ws.dp_size) * Le;
@@ -443,11 +455,31 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
         const uint32_t j = row - seg[s];
         const uint32_t pos = excl[g * Le + le] + j;
         const uint32_t dst_row = run_row[s] + j;
-        if (member == 0 && row < st.max_recv) {
+        if (row >= st.max_recv) continue;   // flagged above: more rows than the receive region was sized for
+        if (member == 0) {
             st.padded_index[(size_t)r * st.max_recv + row] = dst_row;
             // the member of the group that sends to this rank (a2a_worker.rs:633)
             st.source_rank[(size_t)r * st.max_recv + row] = g * ws.dp_size + r % ws.dp_size;
             st.source_position[(size_t)r * st.max_recv + row] = pos;
+            // How the reference addresses the row on its way in and on its way back
+            // (a2a_worker.rs:636-667).  Nothing here reads these two: they are what a rank on a
+            // GPU of its own would consume.
+            const uint32_t peer = g * ws.dp_size + r % ws.dp_size;
+            const uint32_t index_on_rank = pos - grp_dst[g];       // rows of this source before this one
+            const bool same_node = peer / ws.node_size == r / ws.node_size;
+            uint32_t sdo = pos, cso = pos;                         // own rows: the sender's position
+            if (peer != r) {
+                if (index_on_rank < args.max_private) {
+                    sdo = args.max_private * g + index_on_rank;                        // private region
+                } else if (same_node) {
+                    sdo = pos | 0x80000000u;                                           // read from the peer's send buffer
+                } else {
+                    sdo = grp_src[g] + index_on_rank + args.max_private * (G - 1);     // overflow region
+                }
+            }
+            if ((peer != r || ws.dp_size > 1) && !same_node) cso = grp_src[g] + index_on_rank;
+            st.source_dispatch_offset[(size_t)r * st.max_recv + row] = sdo;
+            st.combine_send_offset[(size_t)r * st.max_recv + row] = cso;
         }
         if (dst.out_x == nullptr) continue;
         if (dst_row >= dst.out_rows) {
@@ -547,8 +579,11 @@ int staging_allocate(Staging &st, const a2a_config &cfg, std::string *error) {
     st.comb_stride = a2a_combine_token_stride(&cfg);
     st.payload_bytes = (uint32_t)align_up_sz((size_t)cfg.hidden_dim * cfg.in_elemsize, 16);
     st.max_tokens = cfg.max_num_tokens;
-    // A receiver can get every copy of every sender.
-    const size_t max_recv = N * max_tk;
+    // Rows of the per-receiver tables: what the caller sized a rank's receive region for
+    // (max_recv_tokens), and never more than every copy of every sender.  A receiver that gets
+    // more rows than that is flagged (A2A_DEV_RECV_OVERFLOW) and the rows beyond are dropped.
+    size_t max_recv = N * max_tk;
+    if (cfg.max_recv_tokens != 0 && cfg.max_recv_tokens < max_recv) max_recv = cfg.max_recv_tokens;
     if (max_recv > 0x7FFFFFFFull) {
         if (error) *error = "world_size * max_num_tokens * num_experts_per_token too large";
         return A2A_ERR_UNSUPPORTED;
@@ -567,6 +602,8 @@ int staging_allocate(Staging &st, const a2a_config &cfg, std::string *error) {
     const size_t o_pidx = carve(N * max_recv * sizeof(uint32_t));
     const size_t o_srank = carve(N * max_recv * sizeof(uint32_t));
     const size_t o_spos = carve(N * max_recv * sizeof(uint32_t));
+    const size_t o_sdo = carve(N * max_recv * sizeof(uint32_t));
+    const size_t o_cso = carve(N * max_recv * sizeof(uint32_t));
     const size_t o_nrecv = carve(N * 2 * sizeof(uint32_t));
     hipError_t e = hipMalloc(&st.arena, off);
     if (e != hipSuccess) {
@@ -583,6 +620,8 @@ int staging_allocate(Staging &st, const a2a_config &cfg, std::string *error) {
     st.padded_index = reinterpret_cast<uint32_t *>(base + o_pidx);
     st.source_rank = reinterpret_cast<uint32_t *>(base + o_srank);
     st.source_position = reinterpret_cast<uint32_t *>(base + o_spos);
+    st.source_dispatch_offset = reinterpret_cast<uint32_t *>(base + o_sdo);
+    st.combine_send_offset = reinterpret_cast<uint32_t *>(base + o_cso);
     st.num_recv = reinterpret_cast<uint32_t *>(base + o_nrecv);
     // Tables are read before they are written only through misuse; start from zero.
     e = hipMemset(base + o_pos, 0, o_comb - o_pos);
@@ -620,6 +659,12 @@ const uint32_t *staging_table(const Staging &st, const a2a_config &cfg, uint32_t
         case A2A_TABLE_NUM_RECV_TOKENS:
             *limit = 2;
             return st.num_recv + (size_t)rank * 2;
+        case A2A_TABLE_SOURCE_DISPATCH_OFFSET:
+            *limit = st.max_recv;
+            return st.source_dispatch_offset + (size_t)rank * st.max_recv;
+        case A2A_TABLE_COMBINE_SEND_OFFSET:
+            *limit = st.max_recv;
+            return st.combine_send_offset + (size_t)rank * st.max_recv;
         default:
             return nullptr;
     }
@@ -642,7 +687,7 @@ hipError_t launch_stage_send(const StageSendArgs &args, const Workspace &ws, con
 bool stage_send_small_fits(const StageSendArgs &args, const Workspace &ws) {
     const uint64_t T = args.src.num_tokens;
     const uint64_t entries = T * ws.topk;
-    return T != 0 && entries <= A2A_SMALL_MAX_ENTRIES && entries * T <= A2A_SMALL_MAX_VISITS;
+    return T != 0 && entries <= kSmallMaxEntries && entries * T <= kSmallMaxVisits;
 }
 
 hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &ws, const Staging &st,
@@ -683,7 +728,7 @@ hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, con
     if (l.blocks == 0) l.blocks = 1;    // the layout is published even when nothing was sent
     StageRecvArgs a = args;
     a.team_waves = l.team_waves;
-    const size_t lds = (4 * (size_t)ws.num_groups * ws.experts_per_rank + 1) * sizeof(uint32_t);
+    const size_t lds = (4 * (size_t)ws.num_groups * ws.experts_per_rank + 1 + 2 * (size_t)ws.num_groups) * sizeof(uint32_t);
     hipLaunchKernelGGL(stage_recv_kernel, dim3(l.blocks), dim3(l.threads), lds, stream, a, ws, st);
     return hipGetLastError();
 }

@@ -38,6 +38,8 @@ TABLE_PADDED_INDEX = 4
 TABLE_SOURCE_RANK = 5
 TABLE_SOURCE_POSITION = 6
 TABLE_NUM_RECV_TOKENS = 7
+TABLE_SOURCE_DISPATCH_OFFSET = 8
+TABLE_COMBINE_SEND_OFFSET = 9
 
 DEV_BAD_EXPERT_ID = 1
 DEV_RECV_OVERFLOW = 2

@@ -53,7 +53,8 @@ def run_oracle(case: Case, world: Sequence[RankData], rows: int) -> WorldResult:
     return res
 
 
-def make_ops(case: Case, device: torch.device, max_num_tokens: Optional[int] = None, context_flags: int = 0):
+def make_ops(case: Case, device: torch.device, max_num_tokens: Optional[int] = None, context_flags: int = 0,
+             max_private_tokens: Optional[int] = None):
     from pplx_garden_amd.distributed.loopback import LoopbackWorld
     from pplx_garden_amd.kernels.p2p_all_to_all import P2PAllToAll
 
@@ -64,7 +65,7 @@ def make_ops(case: Case, device: torch.device, max_num_tokens: Optional[int] = N
             expert_padding=case.expert_padding, hidden_dim=case.hidden_dim,
             hidden_dim_scale=case.hidden_dim_scale, in_dtype=torch.float8_e4m3fn,
             out_dtype=torch.bfloat16, scale_dtype=torch.float32,
-            num_experts_per_token=case.topk, nets_per_gpu=1, max_private_tokens=None, device=device,
+            num_experts_per_token=case.topk, nets_per_gpu=1, max_private_tokens=max_private_tokens, device=device,
             dp_group=None, node_group=None, global_group=world.group(r))
         for r in range(case.world_size)
     ]

@@ -8,8 +8,8 @@ import torch
 
 import a2a_oracle as oracle
 from a2a_cases import C0, C1, C2, bf16_codes, make_world, scaled
-from a2a_harness import (SENTINEL, assert_combine_close, assert_dispatch_equal, make_ops, rows_needed, run_gpu,
-                         run_oracle)
+from a2a_harness import (SENTINEL, WorldResult, assert_combine_close, assert_dispatch_equal, make_ops, rows_needed,
+                         run_gpu, run_oracle)
 from a2a_transport import RefConfig, make_ref_rank, oracle_combine, oracle_dispatch, rows_for
 from a2a_transport import make_ops as make_transport_ops
 from pplx_garden_amd.native import p2p_all_to_all as native
@@ -322,47 +322,74 @@ def test_operator_asserts_like_the_reference():
             op.destroy()
 
 
-@pytest.mark.parametrize("case,sources", [(C1, "all"), (scaled(C1, 1200), "one"), (scaled(C1, 300), "all")],
-                         ids=["one_launch_dispatch", "two_launch_dispatch_one_source", "two_launch_dispatch"])
-def test_calls_can_be_captured_in_a_hip_graph(case, sources):
+@pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
+@pytest.mark.parametrize("case,sources", [(C1, "all"), (scaled(C1, 1200), "one"), (scaled(C1, 300), "all"),
+                                          (scaled(C1, 40), "ragged")],
+                         ids=["one_launch_dispatch", "two_launch_dispatch_one_source", "two_launch_dispatch", "ragged"])
+def test_calls_can_be_captured_in_a_hip_graph(case, sources, split):
     """The calls only enqueue kernels whose arguments travel by value (no allocation, copy or
     synchronisation inside), so a dispatch + combine can be captured once and replayed
-    (docs/fabric-lib.md:15 lists graph capture as a feature of the reference).  Every replay,
-    with eager work in between, must reproduce the eager result.  The larger cases take the
-    two-launch dispatch, whose step totals alternate between two copies in device memory: the
-    replays land on either copy."""
+    (docs/fabric-lib.md:15 lists graph capture as a feature of the reference): the two group calls
+    of every rank, or the four split calls of every rank (all sends, all recvs, all combine-sends,
+    all combine-recvs) on a context whose staging was allocated at create.  Every replay, with eager
+    work in between, must reproduce what the ORACLE says, bit for bit for the dispatch and within the
+    combine's tolerance.  The larger cases take the two-launch dispatch, whose step totals alternate
+    between two copies in device memory: the replays land on either copy."""
     world = make_world(case, sources)
     rows = rows_needed(case, world)
     N, Le, H, Hs = case.world_size, case.experts_per_rank, case.hidden_dim, case.hidden_dim_scale
-    _, ops = make_ops(case, DEV)
+    want = run_oracle(case, world, rows)
+    gen = torch.Generator().manual_seed(3)
+    ys = [torch.randn((rows, H), generator=gen).to(torch.bfloat16) for _ in range(N)]
+    want_out = oracle.combine_world([bf16_codes(y) for y in ys], [rd.indices.numpy() for rd in world],
+                                    [rd.weights.numpy() for rd in world], want.slots,
+                                    num_experts=case.num_experts, world_size=N)
+    _, ops = make_ops(case, DEV, context_flags=native.FLAG_PREALLOC_STAGING if split else 0)
     try:
         t = []
-        gen = torch.Generator().manual_seed(3)
         for r, rd in enumerate(world):
             t.append(dict(x=rd.x.to(DEV), idx=rd.indices_u32.to(DEV), w=rd.weights.to(DEV),
                           n=torch.zeros(Le, dtype=torch.int32, device=DEV),
                           ox=torch.zeros((rows, H), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn),
                           os=torch.zeros((rows, Hs), dtype=torch.float32, device=DEV),
-                          y=torch.randn((rows, H), generator=gen).to(torch.bfloat16).to(DEV),
+                          y=ys[r].to(DEV),
                           o=torch.zeros((rd.x.shape[0], H), dtype=torch.bfloat16, device=DEV)))
+        phases = [dict(do_send=True, do_recv=False), dict(do_send=False, do_recv=True)] if split else [dict()]
 
         def step():
-            for r in range(N):
-                ops[r].dispatch(out_expert_num_tokens=t[r]["n"], out_expert_x=t[r]["ox"], out_expert_x_scale=t[r]["os"],
-                                dp_x=t[r]["x"], dp_x_scale=None, indices=t[r]["idx"], weights=t[r]["w"])
-            for r in range(N):
-                ops[r].combine(out_tokens=t[r]["o"], indices=t[r]["idx"], weights=t[r]["w"], expert_y=t[r]["y"])
+            for ph in phases:
+                for r in range(N):
+                    ops[r].dispatch(out_expert_num_tokens=t[r]["n"], out_expert_x=t[r]["ox"],
+                                    out_expert_x_scale=t[r]["os"], dp_x=t[r]["x"], dp_x_scale=None,
+                                    indices=t[r]["idx"], weights=t[r]["w"], **ph)
+            for ph in phases:
+                for r in range(N):
+                    ops[r].combine(out_tokens=t[r]["o"], indices=t[r]["idx"], weights=t[r]["w"],
+                                   expert_y=t[r]["y"], **ph)
 
-        def snapshot():
+        def check(label):
             torch.cuda.synchronize(DEV)
-            return [(a["n"].clone(), a["ox"].view(torch.uint8).clone(), a["os"].clone(), a["o"].clone()) for a in t]
+            got = WorldResult([a["n"].cpu().numpy() for a in t],
+                              [a["ox"].view(torch.uint8).cpu().numpy() for a in t],
+                              [a["os"].cpu().numpy() for a in t],
+                              [a["o"].view(torch.int16).cpu().numpy().view(np.uint16) for a in t])
+            for r in range(N):
+                n_local = max(min(Le, case.num_experts - r * Le), 0)
+                np.testing.assert_array_equal(got.num_tokens[r][:n_local], want.num_tokens[r][:n_local], err_msg=label)
+                w = want.written[r]
+                np.testing.assert_array_equal(got.x[r][w], want.x[r][w], err_msg=label)
+                np.testing.assert_array_equal(got.x_scale[r][w].view(np.uint32), want.x_scale[r][w].view(np.uint32),
+                                              err_msg=label)
+                if got.out_tokens[r].size:
+                    np.testing.assert_allclose(oracle.bf16_to_f32(got.out_tokens[r]), oracle.bf16_to_f32(want_out[r]),
+                                               rtol=1e-2, atol=1e-2, err_msg=label)
 
         def clear():
             for a in t:
                 a["n"].zero_(); a["ox"].view(torch.uint8).zero_(); a["os"].zero_(); a["o"].zero_()
 
         step()
-        eager = snapshot()
+        check("eager")
         assert ops[0].context.status() == 0
         graph = torch.cuda.CUDAGraph()
         side = torch.cuda.Stream(device=DEV)
@@ -373,16 +400,41 @@ def test_calls_can_be_captured_in_a_hip_graph(case, sources):
         torch.cuda.synchronize(DEV)
         with torch.cuda.graph(graph):
             step()
-        for _ in range(3):
+        for i in range(3):
             clear()
             scratch = torch.randn(1 << 20, device=DEV).sum()       # eager work between replays
             torch.cuda.synchronize(DEV)
             graph.replay()
-            got = snapshot()
-            for (en, ex, es, eo), (gn, gx, gs, go) in zip(eager, got):
-                assert torch.equal(en, gn) and torch.equal(ex, gx) and torch.equal(es, gs)
-                assert torch.equal(eo.view(torch.int16), go.view(torch.int16))
+            check(f"replay {i}")
             del scratch
+        assert ops[0].context.status() == 0
+    finally:
+        for op in ops:
+            op.destroy()
+
+
+def test_a_first_split_send_under_capture_needs_preallocated_staging():
+    """The split calls allocate their staging on first use unless the context was created with
+    A2A_FLAG_PREALLOC_STAGING; allocating is illegal while a stream is being captured, so that
+    first send is refused there instead (and works once the capture is over)."""
+    case = scaled(C0, 8)
+    world = make_world(case, "all")
+    _, ops = make_ops(case, DEV)
+    try:
+        rd = world[0]
+        x, idx, w = rd.x.to(DEV), rd.indices_u32.to(DEV), rd.weights.to(DEV)
+        n = torch.zeros(case.experts_per_rank, dtype=torch.int32, device=DEV)
+        ox = torch.zeros((64, case.hidden_dim), dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn)
+        os_ = torch.zeros((64, case.hidden_dim_scale), dtype=torch.float32, device=DEV)
+        send = lambda: ops[0].dispatch(out_expert_num_tokens=n, out_expert_x=ox, out_expert_x_scale=os_, dp_x=x,
+                                       dp_x_scale=None, indices=idx, weights=w, do_send=True, do_recv=False)
+        torch.cuda.synchronize(DEV)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            with pytest.raises(RuntimeError, match="A2A_FLAG_PREALLOC_STAGING"):
+                send()
+        send()
+        torch.cuda.synchronize(DEV)
         assert ops[0].context.status() == 0
     finally:
         for op in ops:

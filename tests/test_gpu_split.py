@@ -35,17 +35,21 @@ def test_split_parity(case, sources, device):
     assert_combine_close(case, got, want)
 
 
+@pytest.mark.parametrize("max_private", [0, 3, 8, None], ids=lambda v: f"private_{v}")
 @pytest.mark.parametrize("node_size", [4, 2, 1])
-def test_routing_tables_match_the_host_worker(node_size, device):
+def test_routing_tables_match_the_host_worker(node_size, max_private, device):
     """num_routed, expert_offsets, token_offset per sender; padded_index, source_rank, source
-    position and the received-row counts per receiver (a2a_worker.rs:526-703)."""
+    position, the two offset tables with their private / same-node (bit 31) / overflow encoding
+    and the received-row counts per receiver (a2a_worker.rs:526-703)."""
     case = replace(C0, name=f"c0_node{node_size}", node_size=node_size, expert_padding=4)
     world = make_world(case, "ragged")
     rows = rows_needed(case, world)
     N, E, K, Le = case.world_size, case.num_experts, case.topk, case.experts_per_rank
-    _, ops = make_ops(case, device)
+    _, ops = make_ops(case, device, max_private_tokens=max_private)
     try:
         ctx = ops[0].context
+        private = ops[0].max_private_tokens
+        assert private == (max_private if max_private is not None else 72)   # int(ceil(64*4/32) * 1.2) * 8
         dev = [dict(x=rd.x.to(device), idx=rd.indices_u32.to(device), w=rd.weights.to(device)) for rd in world]
         outs = [dict(n=torch.zeros(Le, dtype=torch.int32, device=device),
                      x=torch.zeros((rows, case.hidden_dim), dtype=torch.uint8, device=device).view(torch.float8_e4m3fn),
@@ -67,13 +71,17 @@ def test_routing_tables_match_the_host_worker(node_size, device):
             np.testing.assert_array_equal(ctx.read_table(g, native.TABLE_EXPERT_OFFSETS, E).numpy(), eoff)
             np.testing.assert_array_equal(ctx.read_table(g, native.TABLE_TOKEN_OFFSET, T * K).numpy(), toff)
         for r in range(N):
-            lay = oracle.process_routing_info(num_routed, r, N, node_size, 1, case.expert_padding, 0)
+            lay = oracle.process_routing_info(num_routed, r, N, node_size, 1, case.expert_padding, private)
             nrecv = ctx.read_table(r, native.TABLE_NUM_RECV_TOKENS, 2).numpy()
             assert nrecv.tolist() == [lay.num_recv_tokens, lay.num_efa_tokens]
             n = lay.num_recv_tokens
             np.testing.assert_array_equal(ctx.read_table(r, native.TABLE_PADDED_INDEX, n).numpy(), lay.padded_index)
             np.testing.assert_array_equal(ctx.read_table(r, native.TABLE_SOURCE_RANK, n).numpy(), lay.source_rank)
             np.testing.assert_array_equal(ctx.read_table(r, native.TABLE_SOURCE_POSITION, n).numpy(), lay.source_position)
+            np.testing.assert_array_equal(ctx.read_table(r, native.TABLE_SOURCE_DISPATCH_OFFSET, n).numpy(),
+                                          lay.source_dispatch_offset)
+            np.testing.assert_array_equal(ctx.read_table(r, native.TABLE_COMBINE_SEND_OFFSET, n).numpy(),
+                                          lay.combine_send_offset)
             np.testing.assert_array_equal(outs[r]["n"].cpu().numpy(), lay.tokens_per_expert)
     finally:
         for op in ops:

@@ -142,6 +142,51 @@ def test_source_dispatch_offset_variants_name_the_same_row():
         np.testing.assert_array_equal(lay.source_dispatch_offset[rows[:k]], 3 * g + np.arange(k))
 
 
+@pytest.mark.parametrize("N,node,D,private", [(4, 2, 1, 2), (8, 4, 1, 0), (8, 2, 2, 3), (6, 2, 1, 100), (8, 4, 2, 1)])
+def test_dispatch_offsets_name_distinct_rows_of_the_three_regions(N, node, D, private):
+    """`source_dispatch_offset` addresses a receive region of G private parts of `private` rows each,
+    followed by the overflow part (a2a_worker.rs:636-656).  Whatever the counts: a row of another
+    rank is in its source's private part while that lasts, then in the sender's own buffer (bit 31,
+    same node) or in the overflow part (other nodes); no two rows share an address of one buffer; the overflow part
+    is filled source by source in rank order, each source's rows in arrival order."""
+    rng = np.random.default_rng(N * 7 + node + private)
+    G, E = N // D, 2 * N
+    Le = E // N
+    num_routed = rng.integers(0, 6, (G, E)).astype(np.uint32)
+    for r in range(N):
+        lay = oracle.process_routing_info(num_routed, r, N, node, D, 1, private)
+        fe = r * Le
+        per_group = num_routed[:, fe:fe + Le].astype(np.int64).sum(axis=1)
+        below = np.r_[0, np.cumsum(per_group)[:-1]]
+        seen_of_group = np.zeros(G, dtype=np.int64)
+        addresses = set()
+        for i in range(lay.num_recv_tokens):
+            peer = int(lay.source_rank[i])
+            g = peer // D
+            assert peer % D == r % D
+            sdo = int(lay.source_dispatch_offset[i])
+            if peer == r:
+                assert sdo == lay.source_position[i] == lay.combine_send_offset[i] or D > 1
+                assert sdo == lay.source_position[i]
+                continue
+            j = int(seen_of_group[g])
+            seen_of_group[g] += 1
+            if j < private:
+                assert sdo == private * g + j and sdo < private * G
+            elif peer // node == r // node:
+                assert sdo == (int(lay.source_position[i]) | 1 << 31)
+            else:
+                assert sdo == private * G + (below[g] + j - private)
+                assert sdo >= private * G
+            where = (peer, sdo) if sdo >> 31 else sdo      # bit 31: a row of THAT peer's send buffer
+            assert where not in addresses
+            addresses.add(where)
+            # the way back: the sender's own position on the same node, else the row's place among
+            # all rows this rank got, source by source in rank order (a2a_worker.rs:659-667)
+            want_cso = int(lay.source_position[i]) if peer // node == r // node else below[g] + j
+            assert lay.combine_send_offset[i] == want_cso
+
+
 def test_strides_and_capacities_known_answers():
     # a2a_dispatch_send.cu:586-588: fp8 H=7168 with 56 scales -> 7168 + 224 + 16
     assert oracle.dispatch_token_stride(7168, 1, 56, 4) == 7408
