@@ -354,6 +354,8 @@ def main() -> int:
     ap.add_argument("--no-decode", action="store_true", help="skip the shapes other than the 4096-token one")
     ap.add_argument("--decode-only", action="store_true",
                     help="time only the 128-token shape (for a kernel trace of the decode step alone)")
+    ap.add_argument("--only-shape", choices=("decode_128", "qwen3_decode_128", "kimi_1024"), default=None,
+                    help="time only this one of the other shapes of the baseline (for a kernel trace of it alone)")
     ap.add_argument("--separate-routing", action="store_true",
                     help="create the context with A2A_FLAG_SEPARATE_ROUTING (routing kernels, then the pack): "
                          "for comparisons with the default paths")
@@ -398,9 +400,17 @@ def main() -> int:
     side_steps = max(args.steps, 200)
     decode_label = ("DeepSeek-V3 decode: 128 tokens, hidden 7168, 256 experts / 8 logical ranks, top-8 uniform, "
                     "1% x50 outliers")
+    qwen_label = "Qwen3-30B-A3B decode: 128 tokens, hidden 2048, 128 experts / 8 logical ranks, top-8 uniform"
+    kimi_label = ("Kimi-K2 mixed batch: 1024 tokens, hidden 7168, 384 experts / 16 logical ranks, top-8 Zipf(1.0), "
+                  "receive slots padded to 128 per expert")
+    others = {"decode_128": (C2, decode_label, None), "qwen3_decode_128": (C1, qwen_label, None),
+              "kimi_1024": (C4, kimi_label, 37.0)}
     if args.decode_only:
-        print(json.dumps({"decode_128_only": other_shape(C2, device, args.routings, side_steps, args.warmup,
-                                                         ctx_flags, decode_label)}))
+        args.only_shape = "decode_128"
+    if args.only_shape is not None:
+        shape, label, bar = others[args.only_shape]
+        print(json.dumps({args.only_shape + "_only": other_shape(shape, device, args.routings, side_steps, args.warmup,
+                                                                 ctx_flags, label, bar_us=bar)}))
         return 0
 
     case = C3
@@ -451,11 +461,8 @@ def main() -> int:
                           "step_us_wall is wall time over steps without events, the kernel figures come from "
                           "events the launches record themselves, the p50 figures from events around the calls "
                           "of every step (each event adds about 3 us)")
-        qwen = other_shape(C1, device, args.routings, side_steps, args.warmup, ctx_flags,
-                           "Qwen3-30B-A3B decode: 128 tokens, hidden 2048, 128 experts / 8 logical ranks, top-8 uniform")
-        kimi = other_shape(C4, device, args.routings, side_steps, args.warmup, ctx_flags,
-                           "Kimi-K2 mixed batch: 1024 tokens, hidden 7168, 384 experts / 16 logical ranks, top-8 "
-                           "Zipf(1.0), receive slots padded to 128 per expert", bar_us=37.0)
+        qwen = other_shape(C1, device, args.routings, side_steps, args.warmup, ctx_flags, qwen_label)
+        kimi = other_shape(C4, device, args.routings, side_steps, args.warmup, ctx_flags, kimi_label, bar_us=37.0)
 
     cpu = cpu_more = None
     if args.cpu_reps > 0:

@@ -327,7 +327,7 @@ __device__ __forceinline__ void copy_row_by_team(const u32x4 *src, u32x4 *dst, u
 // and scales are copied from the sender's staged token
 // (a2a_dispatch_recv.cu:139-155).
 //
-// Dynamic LDS: 4 * G * Le + 1 + 2 * G words.
+// Dynamic LDS: 4 * G * Le + 1 + 3 * G words.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs args, const Workspace ws,
                                                           const Staging st) {
@@ -347,6 +347,7 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     uint32_t *seg = run_row + items;     // [i][le]  first ARRIVAL index of the run; seg[items] = rows received
     uint32_t *grp_dst = seg + items + 1; // [g]      position of source g's first row for this receiver in g's send order
     uint32_t *grp_src = grp_dst + G;     // [g]      rows this receiver gets from the sources numbered below g
+    uint32_t *grp_cnt = grp_src + G;     // [g]      rows this receiver gets from source g
 
     for (uint32_t w = tid; w < items; w += blockDim.x) {
         const uint32_t g = Le > 1 ? __umulhi(w, ws.le_magic) : w;
@@ -360,11 +361,16 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     // Per source: where its rows for this receiver begin in its own send order (dst_group_offset,
     // a2a_worker.rs:571-575) and how many rows the lower-numbered sources send here
     // (src_group_offset, a2a_worker.rs:582-590: numeric order, not the order of arrival).
-    for (uint32_t g = tid; g < G; g += blockDim.x) {
-        grp_dst[g] = Le != 0 ? excl[g * Le] : 0;
-        uint32_t below = 0;
-        for (uint32_t w = 0; w < g * Le; ++w) below += tot[w];
-        grp_src[g] = below;
+    // (one wavefront per source adds up its row of `tot` here; the short sum over the sources below
+    // it follows after the barriers of the next scan)
+    for (uint32_t g = tid / kWave; g < G; g += blockDim.x / kWave) {
+        uint32_t part = 0;
+        for (uint32_t le = tid & (kWave - 1); le < Le; le += kWave) part += tot[g * Le + le];
+        for (int off = kWave / 2; off > 0; off >>= 1) part += __shfl_down(part, off);
+        if ((tid & (kWave - 1)) == 0) {
+            grp_dst[g] = excl[g * Le];
+            grp_cnt[g] = part;
+        }
     }
 
     // Rows per expert, padded offsets, first row of every run.
@@ -401,6 +407,12 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
             __syncthreads();
             carry = s_carry;
         }
+    }
+
+    if (tid < G) {   // grp_cnt was written before the barriers of the scan above
+        uint32_t rows_below = 0;
+        for (uint32_t g = 0; g < tid; ++g) rows_below += grp_cnt[g];
+        grp_src[tid] = rows_below;
     }
 
     // Arrival order: sources as the worker visits them, local experts inside a source.
@@ -728,7 +740,7 @@ hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, con
     if (l.blocks == 0) l.blocks = 1;    // the layout is published even when nothing was sent
     StageRecvArgs a = args;
     a.team_waves = l.team_waves;
-    const size_t lds = (4 * (size_t)ws.num_groups * ws.experts_per_rank + 1 + 2 * (size_t)ws.num_groups) * sizeof(uint32_t);
+    const size_t lds = (4 * (size_t)ws.num_groups * ws.experts_per_rank + 1 + 3 * (size_t)ws.num_groups) * sizeof(uint32_t);
     hipLaunchKernelGGL(stage_recv_kernel, dim3(l.blocks), dim3(l.threads), lds, stream, a, ws, st);
     return hipGetLastError();
 }

@@ -9,6 +9,19 @@
 //              rows are a random permutation of a dense buffer
 //   gather     one wavefront per token and 1 KiB piece: 16 bytes from each of
 //              8 rows of 14336 bytes, summed, 16 bytes out (the combine's shape)
+//   variants   the same gather with its output written through every cache
+//              policy the store instruction has, with cached loads, and in
+//              three shapes meant to make the writes overlap the reads (a
+//              persistent wavefront that asks for the next unit's rows before
+//              it stores the current one; a wavefront per workgroup that only
+//              stores what three others hand it through LDS; persistent
+//              workgroups that collect 16 to 64 KiB of output in LDS and write
+//              it in one burst)
+//
+// Every gather variant takes the number of units (token x 1 KiB piece) and
+// returns at once for a unit beyond it; the host derives each grid from the
+// unit count in one place (launch_units) and refuses a grid that would cover
+// more than the buffers hold.
 //
 // What ran before matters, because it decides what the caches hold when the
 // timed kernel starts: after a kernel that mostly reads (clean lines) the push
@@ -77,6 +90,7 @@ __global__ void copy_sweep(const u32x4 *__restrict__ in, u32x4 *__restrict__ out
 __global__ __launch_bounds__(448) void push(const uint8_t *__restrict__ x, uint8_t *__restrict__ out,
                                             const uint32_t *__restrict__ slots) {
     const uint32_t t = blockIdx.x, c = threadIdx.x;
+    if (t >= kTokens || c >= kHidden / 16) return;
     const u32x4 *p = reinterpret_cast<const u32x4 *>(x + (size_t)t * kInRow + (size_t)c * 32);
     const u32x4 a = __builtin_nontemporal_load(p), b = __builtin_nontemporal_load(p + 1);
     const u32x4 q = a ^ b;
@@ -92,6 +106,7 @@ template <bool STORE>
 __global__ __launch_bounds__(64) void gather(const uint8_t *__restrict__ y, uint8_t *__restrict__ out,
                                              const uint32_t *__restrict__ slots, uint32_t never) {
     const uint32_t t = blockIdx.x / 14, piece = blockIdx.x % 14;
+    if (t >= kTokens) return;
     const uint32_t c = piece * 64 + threadIdx.x;
     u32x4 v[kTopk];
 #pragma unroll
@@ -107,6 +122,144 @@ __global__ __launch_bounds__(64) void gather(const uint8_t *__restrict__ y, uint
         __builtin_nontemporal_store(acc, o);
     } else if (acc[0] == never) {
         *o = acc;
+    }
+}
+
+
+// ---- variants of the gather; a unit is one (token, 1 KiB piece) ----
+constexpr uint32_t kPieces = (uint32_t)(kInRow / 1024);   // 14
+constexpr uint32_t kUnits = kTokens * kPieces;
+
+__device__ __forceinline__ void load_unit(u32x4 (&v)[kTopk], const uint8_t *y, const uint32_t *slots, uint32_t unit) {
+    const uint32_t t = unit / kPieces, piece = unit - t * kPieces;
+    const uint32_t c = piece * 64 + (threadIdx.x & 63);
+#pragma unroll
+    for (uint32_t k = 0; k < kTopk; ++k) {
+        v[k] = __builtin_nontemporal_load(
+            reinterpret_cast<const u32x4 *>(y + (size_t)slots[t * kTopk + k] * kInRow + (size_t)c * 16));
+    }
+}
+
+__device__ __forceinline__ u32x4 sum_unit(const u32x4 (&v)[kTopk]) {
+    u32x4 acc = v[0];
+#pragma unroll
+    for (uint32_t k = 1; k < kTopk; ++k) acc += v[k];
+    return acc;
+}
+
+__device__ __forceinline__ u32x4 *out_of_unit(uint8_t *out, uint32_t unit) {
+    const uint32_t t = unit / kPieces, piece = unit - t * kPieces;
+    return reinterpret_cast<u32x4 *>(out + (size_t)t * kInRow + (size_t)(piece * 64 + (threadIdx.x & 63)) * 16);
+}
+
+// Cache policy of the 16-byte output store.
+enum StorePolicy { kStoreNt, kStorePlain, kStoreSc0Sc1, kStoreSc1, kStoreSc0, kStoreSc0Sc1Nt };
+
+template <int POLICY>
+__device__ __forceinline__ void store_unit(u32x4 v, u32x4 *p) {
+    if (POLICY == kStoreNt) {
+        __builtin_nontemporal_store(v, p);
+    } else if (POLICY == kStorePlain) {
+        *p = v;
+    } else if (POLICY == kStoreSc0Sc1) {
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1" ::"v"(p), "v"(v) : "memory");
+    } else if (POLICY == kStoreSc1) {
+        asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+    } else if (POLICY == kStoreSc0) {
+        asm volatile("global_store_dwordx4 %0, %1, off sc0" ::"v"(p), "v"(v) : "memory");
+    } else {
+        asm volatile("global_store_dwordx4 %0, %1, off sc0 sc1 nt" ::"v"(p), "v"(v) : "memory");
+    }
+}
+
+// One unit per wavefront, as `gather`, with the store policy a parameter.
+template <int POLICY>
+__global__ __launch_bounds__(64) void gather_policy(const uint8_t *__restrict__ y, uint8_t *__restrict__ out,
+                                                    const uint32_t *__restrict__ slots, uint32_t units) {
+    const uint32_t unit = blockIdx.x;
+    if (unit >= units) return;
+    u32x4 v[kTopk];
+    load_unit(v, y, slots, unit);
+    store_unit<POLICY>(sum_unit(v), out_of_unit(out, unit));
+}
+
+// Ordinary (cached) loads instead of non-temporal ones.
+__global__ __launch_bounds__(64) void gather_cached_loads(const uint8_t *__restrict__ y, uint8_t *__restrict__ out,
+                                                          const uint32_t *__restrict__ slots, uint32_t units) {
+    const uint32_t unit = blockIdx.x;
+    if (unit >= units) return;
+    const uint32_t t = unit / kPieces, piece = unit - t * kPieces, c = piece * 64 + threadIdx.x;
+    u32x4 v[kTopk];
+#pragma unroll
+    for (uint32_t k = 0; k < kTopk; ++k) {
+        v[k] = *reinterpret_cast<const u32x4 *>(y + (size_t)slots[t * kTopk + k] * kInRow + (size_t)c * 16);
+    }
+    __builtin_nontemporal_store(sum_unit(v), out_of_unit(out, unit));
+}
+
+// Persistent wavefronts, software-pipelined: the rows of the next unit are asked
+// for before the current unit is stored.
+__global__ __launch_bounds__(64) void gather_pipelined(const uint8_t *__restrict__ y, uint8_t *__restrict__ out,
+                                                       const uint32_t *__restrict__ slots, uint32_t units) {
+    const uint32_t stride = gridDim.x;
+    uint32_t unit = blockIdx.x;
+    if (unit >= units) return;
+    u32x4 cur[kTopk], nxt[kTopk];
+    load_unit(cur, y, slots, unit);
+    while (true) {
+        const uint32_t next = unit + stride;
+        const bool more = next < units;
+        if (more) load_unit(nxt, y, slots, next);
+        __builtin_nontemporal_store(sum_unit(cur), out_of_unit(out, unit));
+        if (!more) break;
+        for (uint32_t k = 0; k < kTopk; ++k) cur[k] = nxt[k];
+        unit = next;
+    }
+}
+
+// Three wavefronts gather; the fourth only stores what they hand it through LDS.
+__global__ __launch_bounds__(256) void gather_store_wave(const uint8_t *__restrict__ y, uint8_t *__restrict__ out,
+                                                         const uint32_t *__restrict__ slots, uint32_t units) {
+    __shared__ u32x4 stage[3][64];
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x & 63;
+    const uint32_t first = blockIdx.x * 3;
+    if (wave < 3 && first + wave < units) {
+        u32x4 v[kTopk];
+        load_unit(v, y, slots, first + wave);
+        stage[wave][lane] = sum_unit(v);
+    }
+    __syncthreads();
+    if (wave == 3) {
+#pragma unroll
+        for (uint32_t w = 0; w < 3; ++w) {
+            if (first + w < units) __builtin_nontemporal_store(stage[w][lane], out_of_unit(out, first + w));
+        }
+    }
+}
+
+// Persistent workgroups of 16 wavefronts collect ROUNDS x 16 KiB of output in LDS,
+// then write it in one burst.
+template <int ROUNDS>
+__global__ __launch_bounds__(1024) void gather_bursts(const uint8_t *__restrict__ y, uint8_t *__restrict__ out,
+                                                      const uint32_t *__restrict__ slots, uint32_t units) {
+    extern __shared__ u32x4 collected[];   // [ROUNDS][16][64]
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x & 63;
+    const uint32_t per_group = 16 * ROUNDS;
+    for (uint32_t first = blockIdx.x * per_group; first < units; first += gridDim.x * per_group) {
+        for (uint32_t r = 0; r < ROUNDS; ++r) {
+            const uint32_t unit = first + r * 16 + wave;
+            if (unit < units) {
+                u32x4 v[kTopk];
+                load_unit(v, y, slots, unit);
+                collected[(r * 16 + wave) * 64 + lane] = sum_unit(v);
+            }
+        }
+        __syncthreads();
+        for (uint32_t r = 0; r < ROUNDS; ++r) {
+            const uint32_t unit = first + r * 16 + wave;
+            if (unit < units) __builtin_nontemporal_store(collected[(r * 16 + wave) * 64 + lane], out_of_unit(out, unit));
+        }
+        __syncthreads();
     }
 }
 
@@ -230,5 +383,35 @@ int main() {
     report("  the gather's output alone, 56 MiB striped fill",
            timer.median_us(fill_other, [&] { hipLaunchKernelGGL(write_sweep, dim3(512), dim3(256), 0, s, (u32x4 *)combined, kTokens * kInRow / 16, 9u); }),
            (double)kTokens * kInRow);
+    // Variants of the gather.  Every launch goes through launch_units: the grid comes from the unit
+    // count, and a grid whose last workgroup would start beyond the units is refused on the host
+    // (the kernels also return for such a unit).
+    std::printf("variants of the gather (after a push):\n");
+    auto launch_units = [&](auto kernel, uint32_t blocks, uint32_t threads, size_t lds, uint32_t units_per_block) {
+        if (blocks == 0 || (uint64_t)(blocks - 1) * units_per_block >= kUnits || lds > 64 * 1024) {
+            std::fprintf(stderr, "refusing a grid of %u workgroups x %u units for %u units\n", blocks,
+                         units_per_block, kUnits);
+            std::exit(2);
+        }
+        hipLaunchKernelGGL(kernel, dim3(blocks), dim3(threads), lds, s, (const uint8_t *)y, combined,
+                           (const uint32_t *)d_slots, kUnits);
+    };
+    auto variant = [&](const char *name, auto kernel, uint32_t blocks, uint32_t threads, size_t lds,
+                       uint32_t units_per_block) {
+        report(name, timer.median_us(run_push, [&] { launch_units(kernel, blocks, threads, lds, units_per_block); }),
+               gather_bytes);
+    };
+    variant("  store nt (as the library)", gather_policy<kStoreNt>, kUnits, 64, 0, 1);
+    variant("  store plain", gather_policy<kStorePlain>, kUnits, 64, 0, 1);
+    variant("  store sc0 sc1", gather_policy<kStoreSc0Sc1>, kUnits, 64, 0, 1);
+    variant("  store sc1", gather_policy<kStoreSc1>, kUnits, 64, 0, 1);
+    variant("  store sc0", gather_policy<kStoreSc0>, kUnits, 64, 0, 1);
+    variant("  store sc0 sc1 nt", gather_policy<kStoreSc0Sc1Nt>, kUnits, 64, 0, 1);
+    variant("  cached loads, store nt", gather_cached_loads, kUnits, 64, 0, 1);
+    variant("  pipelined, 2048 persistent wavefronts", gather_pipelined, 2048, 64, 0, 1);
+    variant("  pipelined, 16384 persistent wavefronts", gather_pipelined, 16384, 64, 0, 1);
+    variant("  a wavefront that only stores (3 + 1)", gather_store_wave, (kUnits + 2) / 3, 256, 0, 3);
+    variant("  16 KiB bursts from LDS, 256 workgroups", gather_bursts<1>, 256, 1024, 16 * 1024, 16);
+    variant("  64 KiB bursts from LDS, 512 workgroups", gather_bursts<4>, 512, 1024, 64 * 1024, 64);
     return 0;
 }
