@@ -156,12 +156,7 @@ __device__ uint32_t rank_chunk(const RouteSrc &src, const Workspace &ws, uint32_
     const uint32_t K = ws.topk;
     const uint32_t num_entries = effective_tokens(src.bound_m, src.num_tokens) * K;
 
-    if (tid < E) {
-#pragma unroll
-        for (int w = 0; w < kRouteWaves; ++w) wave_hist[w][tid] = 0;
-    }
-    __syncthreads();
-
+    // The entry's expert id is asked for first: it travels while the table is cleared.
     const uint32_t entry = chunk * kRouteBlock + tid;
     bool valid = entry < num_entries;
     uint32_t expert = 0;
@@ -169,10 +164,15 @@ __device__ uint32_t rank_chunk(const RouteSrc &src, const Workspace &ws, uint32_
         const uint32_t token = entry / K;
         const uint32_t k = entry - token * K;
         expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + k];
-        if (expert >= E) {
-            valid = false;
-            atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
-        }
+    }
+    if (tid < E) {
+#pragma unroll
+        for (int w = 0; w < kRouteWaves; ++w) wave_hist[w][tid] = 0;
+    }
+    __syncthreads();
+    if (valid && expert >= E) {
+        valid = false;
+        atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
     }
 
     // Lanes of this wavefront that hold the same expert id.

@@ -259,6 +259,73 @@ int main() {
         }
     }
 
+    // a2a_dispatch_static: no context, no allocation; must write what a2a_dispatch writes.
+    {
+        a2a_dispatch_args d[N], d2[N];
+        std::memset(d, 0, sizeof d);
+        std::vector<void *> n2(N), ox2(N), os2(N);
+        uint32_t *d_flags = nullptr;
+        HIP_OK(hipMalloc(&d_flags, sizeof(uint32_t)));
+        HIP_OK(hipMemset(d_flags, 0, sizeof(uint32_t)));
+        for (uint32_t r = 0; r < N; ++r) {
+            Rank &k = ranks[r];
+            HIP_OK(hipMalloc(&n2[r], Le * 4));
+            HIP_OK(hipMalloc(&ox2[r], rows * H));
+            HIP_OK(hipMalloc(&os2[r], rows * Hs * 4));
+            HIP_OK(hipMemset(k.d_ox, 0, rows * H));
+            HIP_OK(hipMemset(k.d_os, 0, rows * Hs * 4));
+            HIP_OK(hipMemset(ox2[r], 0, rows * H));
+            HIP_OK(hipMemset(os2[r], 0, rows * Hs * 4));
+            d[r].num_tokens = T;
+            d[r].x_ptr = k.d_x;
+            d[r].x_stride = H * 2;
+            d[r].indices = (const int32_t *)k.d_idx;
+            d[r].indices_stride = K;
+            d[r].out_num_tokens = (int32_t *)k.d_n;
+            d[r].out_x = k.d_ox;
+            d[r].out_x_stride = H;
+            d[r].out_x_rows = rows;
+            d[r].out_x_scale = (float *)k.d_os;
+            d[r].out_x_scale_stride_elem = 1;
+            d[r].out_x_scale_stride_token = Hs;
+            d2[r] = d[r];
+            d2[r].out_num_tokens = (int32_t *)n2[r];
+            d2[r].out_x = ox2[r];
+            d2[r].out_x_scale = (float *)os2[r];
+        }
+        A2A_OK_OR_FAIL(a2a_dispatch(ctx, d, /*quantize=*/1, stream));
+        const int rc = a2a_dispatch_static(&cfg, d2, /*quantize=*/1, d_flags, stream);
+        if (rc != 0) {
+            std::fprintf(stderr, "a2a_dispatch_static failed (%d): %s\n", rc, a2a_last_error(nullptr));
+            return 1;
+        }
+        HIP_OK(hipStreamSynchronize(stream));
+        uint32_t flags = 1;
+        HIP_OK(hipMemcpy(&flags, d_flags, sizeof flags, hipMemcpyDeviceToHost));
+        bool same = flags == 0;
+        std::vector<uint8_t> a(rows * H), b(rows * H);
+        std::vector<float> sa(rows * Hs), sb(rows * Hs);
+        for (uint32_t r = 0; r < N && same; ++r) {
+            int32_t na[Le], nb[Le];
+            HIP_OK(hipMemcpy(na, ranks[r].d_n, sizeof na, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(nb, n2[r], sizeof nb, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(a.data(), ranks[r].d_ox, a.size(), hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(b.data(), ox2[r], b.size(), hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(sa.data(), ranks[r].d_os, sa.size() * 4, hipMemcpyDeviceToHost));
+            HIP_OK(hipMemcpy(sb.data(), os2[r], sb.size() * 4, hipMemcpyDeviceToHost));
+            same = std::memcmp(na, nb, sizeof na) == 0 && a == b &&
+                   std::memcmp(sa.data(), sb.data(), sa.size() * 4) == 0;
+        }
+        std::printf("static dispatch: %s\n", same ? "identical to a2a_dispatch" : "DIFFERS from a2a_dispatch");
+        if (!same) ++failures;
+        for (uint32_t r = 0; r < N; ++r) {
+            (void)hipFree(n2[r]);
+            (void)hipFree(ox2[r]);
+            (void)hipFree(os2[r]);
+        }
+        (void)hipFree(d_flags);
+    }
+
     for (Rank &k : ranks) {
         for (void *p : {k.d_x, k.d_idx, k.d_w, k.d_n, k.d_ox, k.d_os, k.d_y, k.d_out}) (void)hipFree(p);
     }

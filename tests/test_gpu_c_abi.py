@@ -1,5 +1,6 @@
 """The C ABI driven by a C++ program with nothing but the HIP runtime around it (no Python, no torch):
-one step through the group calls and one through the split calls, checked on the host by the program
+one step through the group calls, one through the split calls and one through the dispatch that
+allocates nothing, checked on the host by the program
 itself (expert counts against a host histogram, the reference's round-trip identity)."""
 
 import subprocess
@@ -22,6 +23,7 @@ def test_cpp_caller_of_the_c_abi():
     assert done.returncode == 0, done.stderr
     assert "selftest passed" in done.stdout
     assert "group calls" in done.stdout and "split calls" in done.stdout
+    assert "static dispatch: identical to a2a_dispatch" in done.stdout
 
 
 def test_memory_ceilings_program_runs():
