@@ -476,7 +476,7 @@ def main() -> int:
         }
         cores = min(16, os.cpu_count() or 1)
         dt_all, _ = cpu_baseline(case, cpu_rd, args.cpu_reps, threads=cores)
-        sample_tokens = 1024
+        sample_tokens = case.num_tokens
         dt_np = cpu_baseline_numpy(case, sample_tokens)
         s_d, s_c = algorithmic_bytes(sample_tokens, case.hidden_dim, case.topk)
         cpu_more = {
@@ -486,7 +486,7 @@ def main() -> int:
                           "note": "same code, tokens split over OpenMP threads; routing stays on one thread"},
             "numpy_oracle": {"value": round((s_d + s_c) / dt_np / 1e9, 3), "unit": "GB/s",
                              "cores": 1, "seconds": round(dt_np, 2),
-                             "sample": f"{sample_tokens} tokens of the same workload through the numpy oracle "
+                             "sample": f"the same {sample_tokens}-token batch, once, through the numpy oracle "
                                        "(array code; numpy's element-wise loops use one thread whatever the "
                                        f"host has: {os.cpu_count()} cores here)"},
         }

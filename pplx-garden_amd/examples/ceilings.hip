@@ -16,7 +16,8 @@
 //              it stores the current one; a wavefront per workgroup that only
 //              stores what three others hand it through LDS; persistent
 //              workgroups that collect 16 to 64 KiB of output in LDS and write
-//              it in one burst)
+//              it in one burst); and the push with the same store policies and
+//              with half a token per workgroup
 //
 // Every gather variant takes the number of units (token x 1 KiB piece) and
 // returns at once for a unit beyond it; the host derives each grid from the
@@ -263,6 +264,24 @@ __global__ __launch_bounds__(1024) void gather_bursts(const uint8_t *__restrict_
     }
 }
 
+// The push with the cache policy of its stores a parameter, and HALF of a token per
+// workgroup when SPLIT is set (twice the workgroups, 224 of 256 threads active).
+template <int POLICY, bool SPLIT>
+__global__ __launch_bounds__(SPLIT ? 256 : 448) void push_policy(const uint8_t *__restrict__ x,
+                                                                uint8_t *__restrict__ out,
+                                                                const uint32_t *__restrict__ slots, uint32_t tokens) {
+    const uint32_t t = SPLIT ? blockIdx.x / 2 : blockIdx.x;
+    const uint32_t c = SPLIT ? (blockIdx.x & 1) * 224 + threadIdx.x : threadIdx.x;
+    if (t >= tokens || c >= kHidden / 16 || (SPLIT && threadIdx.x >= 224)) return;
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(x + (size_t)t * kInRow + (size_t)c * 32);
+    const u32x4 a = __builtin_nontemporal_load(p), b = __builtin_nontemporal_load(p + 1);
+    const u32x4 q = a ^ b;
+#pragma unroll
+    for (uint32_t k = 0; k < kTopk; ++k) {
+        store_unit<POLICY>(q, reinterpret_cast<u32x4 *>(out + (size_t)slots[t * kTopk + k] * kOutRow + (size_t)c * 16));
+    }
+}
+
 struct Timer {
     hipStream_t stream;
     hipEvent_t start, stop;
@@ -413,5 +432,26 @@ int main() {
     variant("  a wavefront that only stores (3 + 1)", gather_store_wave, (kUnits + 2) / 3, 256, 0, 3);
     variant("  16 KiB bursts from LDS, 256 workgroups", gather_bursts<1>, 256, 1024, 16 * 1024, 16);
     variant("  64 KiB bursts from LDS, 512 workgroups", gather_bursts<4>, 512, 1024, 64 * 1024, 64);
+
+    // Variants of the push: the cache policy of its stores, and half a token per workgroup.
+    std::printf("variants of the push (after a gather):\n");
+    auto push_variant = [&](const char *name, auto kernel, uint32_t blocks, uint32_t threads) {
+        if (blocks == 0 || blocks > 2 * kTokens) {
+            std::fprintf(stderr, "refusing a grid of %u workgroups for %u tokens\n", blocks, kTokens);
+            std::exit(2);
+        }
+        report(name, timer.median_us(run_gather, [&] {
+                   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(threads), 0, s, (const uint8_t *)x, dispatched,
+                                      (const uint32_t *)d_slots, kTokens);
+               }),
+               push_bytes);
+    };
+    push_variant("  store plain", (push_policy<kStorePlain, false>), kTokens, 448);
+    push_variant("  store nt", (push_policy<kStoreNt, false>), kTokens, 448);
+    push_variant("  store sc0 sc1 nt", (push_policy<kStoreSc0Sc1Nt, false>), kTokens, 448);
+    push_variant("  store sc0", (push_policy<kStoreSc0, false>), kTokens, 448);
+    push_variant("  store sc1 (as the library)", (push_policy<kStoreSc1, false>), kTokens, 448);
+    push_variant("  store sc0 sc1", (push_policy<kStoreSc0Sc1, false>), kTokens, 448);
+    push_variant("  store sc1, half a token per workgroup", (push_policy<kStoreSc1, true>), 2 * kTokens, 256);
     return 0;
 }
