@@ -77,7 +77,7 @@ def measured_traffic():
     if sha is None or sha.group(1) != kernel_sources_sha256():
         return {}, "the counter summary under profiles/ was taken on other kernel sources"
     out = {m.group(1): int(m.group(2)) for m in re.finditer(r"^traffic_bytes:\s*(\w+)\s*=\s*(\d+)\s*$", text, flags=re.M)}
-    return out, f"FETCH_SIZE and WRITE_SIZE passes of this build, {TRAFFIC_PROFILE.relative_to(REPO)}"
+    return out, f"FETCH_SIZE and WRITE_SIZE passes of this build, profiles/{TRAFFIC_PROFILE.name}"
 
 
 class Workload:
