@@ -561,3 +561,59 @@ def test_operator_reports_the_reference_capacities():
         finally:
             for op in ops:
                 op.destroy()
+
+
+@pytest.mark.parametrize("sender,bound,strided", [(0, None, False), (2, None, False), (3, 37, False), (1, 0, False),
+                                                   (2, None, True), (1, 5, True)],
+                         ids=["rank0", "rank2", "rank3_bound37", "rank1_bound0", "rank2_strided", "rank1_bound5_strided"])
+def test_one_launch_dispatch_with_a_single_source(sender, bound, strided):
+    """A small step in which ONE rank has tokens takes a variant of the one-launch dispatch that reads the
+    entries as a flat array, provided the index rows are dense; with a row stride other than K the general
+    variant runs.  Either way: any rank may be the sender, `bound_m` may shorten the step on the device, and
+    the result is the oracle's, bit for bit."""
+    case = C1                                      # 128 tokens, 128 experts over 8 ranks, top-8
+    N, Le, H, Hs, K = case.world_size, case.experts_per_rank, case.hidden_dim, case.hidden_dim_scale, case.topk
+    world = [make_world(case, "all")[r] if r == sender else make_world(scaled(case, 0), "all")[r] for r in range(N)]
+    rows = rows_needed(case, world)
+    inputs = [oracle.RankInput(x=bf16_codes(rd.x), indices=rd.indices.numpy(), bound_m=bound if r == sender else None)
+              for r, rd in enumerate(world)]
+    want = oracle.dispatch_world(inputs, num_experts=case.num_experts, world_size=N, node_size=N, expert_padding=1,
+                                 out_rows=rows, quantize=True)
+    _, ops = make_ops(case, DEV)
+    try:
+        t = []
+        for r, rd in enumerate(world):
+            idx = rd.indices_u32.to(DEV)
+            if strided and rd.indices.shape[0]:
+                wide = torch.zeros((rd.indices.shape[0], K + 3), dtype=torch.uint32, device=DEV)
+                wide[:, :K] = idx
+                idx = wide[:, :K]                  # row stride K + 3
+                assert idx.stride(0) == K + 3
+            t.append(dict(x=rd.x.to(DEV), idx=idx, w=rd.weights.to(DEV),
+                          b=torch.tensor([bound], dtype=torch.int32, device=DEV) if r == sender and bound is not None else None,
+                          n=torch.full((Le,), -1, dtype=torch.int32, device=DEV),
+                          ox=torch.full((rows, H), SENTINEL, dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn),
+                          os=torch.full((rows, Hs), -7.0, dtype=torch.float32, device=DEV)))
+        for r in range(N):
+            ops[r].dispatch(out_expert_num_tokens=t[r]["n"], out_expert_x=t[r]["ox"], out_expert_x_scale=t[r]["os"],
+                            dp_x=t[r]["x"], dp_x_scale=None, indices=t[r]["idx"], weights=t[r]["w"], bound_m=t[r]["b"])
+        torch.cuda.synchronize(DEV)
+        ctx = ops[0].context
+        assert ctx.status() == 0
+        for r in range(N):
+            np.testing.assert_array_equal(t[r]["n"].cpu().numpy(), want[r].num_tokens)
+            wr = want[r].written
+            got_x = t[r]["ox"].view(torch.uint8).cpu().numpy()
+            np.testing.assert_array_equal(got_x[wr], want[r].x[wr])
+            np.testing.assert_array_equal(t[r]["os"].cpu().numpy()[wr].view(np.uint32), want[r].x_scale[wr].view(np.uint32))
+            assert (got_x[~wr] == SENTINEL).all()
+        n_eff = world[sender].indices.shape[0] if bound is None else bound
+        count, toff, eoff = oracle.route(world[sender].indices.numpy()[:n_eff], case.num_experts)
+        np.testing.assert_array_equal(ctx.read_table(sender, native.TABLE_NUM_ROUTED, case.num_experts).numpy(), count)
+        np.testing.assert_array_equal(ctx.read_table(sender, native.TABLE_EXPERT_OFFSETS, case.num_experts).numpy(), eoff)
+        np.testing.assert_array_equal(ctx.read_table(sender, native.TABLE_TOKEN_OFFSET, n_eff * K).numpy(), toff)
+        np.testing.assert_array_equal(ctx.read_table(sender, native.TABLE_SLOT, n_eff * K).numpy(),
+                                      want[0].slots[sender][:n_eff].reshape(-1))
+    finally:
+        for op in ops:
+            op.destroy()
