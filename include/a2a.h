@@ -247,6 +247,9 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
  *   - `device_flags`: optional DEVICE pointer to one uint32 that the kernels OR
  *     the A2A_DEV_* bits into (the caller clears it); with NULL bad input is
  *     dropped silently as described at those bits.
+ *   - The first call on a GPU also looks up where that GPU holds the array
+ *     (hipGetSymbolAddress, once per device): make one call outside any
+ *     stream capture before capturing calls into a graph.
  *   - The routing of the step stays inside the library: a2a_combine needs a
  *     context and the a2a_dispatch that goes with it.
  * Error text: a2a_last_error(NULL) on the calling thread.

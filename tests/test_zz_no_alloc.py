@@ -126,3 +126,44 @@ def test_static_dispatch_reports_bad_input_through_the_callers_flag_word():
     # without a flag word the same call drops the copy silently and still completes
     native.dispatch_static(cfg, _Buffers(case, world, rows).args, True, None, stream)
     torch.cuda.synchronize(DEV)
+
+
+def test_static_dispatch_can_be_captured_in_a_hip_graph():
+    """What the entry point is for: a caller under stream capture.  After one eager call (which looks up the
+    address of the fixed array on this GPU), a call is captured and replayed three times with eager work and
+    another, different static call in between (it overwrites the shared tables): every replay must write
+    what the oracle says."""
+    case = Case("static_graph", 600, 256, 32, 4, 8, 9300, expert_padding=2)
+    stream = torch.cuda.current_stream(DEV).cuda_stream
+    cfg = _config(case, case.num_tokens)
+    world = [make_rank(case, r, t) for r, t in enumerate([600, 0, 333, 590])]      # two-launch path
+    other = [make_rank(case, r, t) for r, t in enumerate([9, 50, 0, 1])]           # one-launch path
+    rows = max(rows_needed(case, world), rows_needed(case, other))
+    want = _oracle(case, world, rows)
+    b = _Buffers(case, world, rows)
+    o = _Buffers(case, other, rows)
+    native.dispatch_static(cfg, b.args, True, None, stream)                        # eager: also the set-up call
+    assert_dispatch_equal(case, b.result(), want)
+    args = (native.A2ADispatchArgs * case.world_size)(*b.args)
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream(device=DEV)
+    side.wait_stream(torch.cuda.current_stream(DEV))
+    with torch.cuda.stream(side):
+        native.dispatch_static(cfg, args, True, None, side.cuda_stream)
+    torch.cuda.current_stream(DEV).wait_stream(side)
+    torch.cuda.synchronize(DEV)
+    with torch.cuda.graph(graph):
+        native.dispatch_static(cfg, args, True, None, torch.cuda.current_stream(DEV).cuda_stream)
+    for i in range(3):
+        for t in b.n + b.x + b.s:
+            t.fill_(0)
+        for t in b.x:
+            t.fill_(SENTINEL)
+        for t in b.s:
+            t.fill_(-7.0)
+        native.dispatch_static(cfg, o.args, True, None, stream)                    # leaves other tables behind
+        scratch = torch.randn(1 << 20, device=DEV).sum()
+        torch.cuda.synchronize(DEV)
+        graph.replay()
+        assert_dispatch_equal(case, b.result(), want)
+        del scratch
