@@ -18,6 +18,7 @@
 //              workgroups that collect 16 to 64 KiB of output in LDS and write
 //              it in one burst); and the push with the same store policies and
 //              with half a token per workgroup
+//   1024       push and gather over the first 1024 tokens only
 //
 // Every gather variant takes the number of units (token x 1 KiB piece) and
 // returns at once for a unit beyond it; the host derives each grid from the
@@ -453,5 +454,22 @@ int main() {
     push_variant("  store sc1 (as the library)", (push_policy<kStoreSc1, false>), kTokens, 448);
     push_variant("  store sc0 sc1", (push_policy<kStoreSc0Sc1, false>), kTokens, 448);
     push_variant("  store sc1, half a token per workgroup", (push_policy<kStoreSc1, true>), 2 * kTokens, 256);
+
+    // The same two shapes at 1024 tokens (the Kimi-K2 mixed batch): the push is a single wave of
+    // workgroups, so nothing overlaps its launch, its reads and its burst of writes.
+    std::printf("at 1024 tokens, push and gather in turn:\n");
+    constexpr uint32_t kFewTokens = 1024;
+    auto few_push = [&] {
+        hipLaunchKernelGGL((push_policy<kStoreSc1, false>), dim3(kFewTokens), dim3(448), 0, s, (const uint8_t *)x,
+                           dispatched, (const uint32_t *)d_slots, kFewTokens);
+    };
+    auto few_gather = [&] {
+        hipLaunchKernelGGL(gather_policy<kStoreNt>, dim3(kFewTokens * kPieces), dim3(64), 0, s, (const uint8_t *)y,
+                           combined, (const uint32_t *)d_slots, kFewTokens * kPieces);
+    };
+    report("  push, 1024 tokens, store sc1", timer.median_us(few_gather, few_push),
+           (double)kFewTokens * (kInRow + kTopk * kOutRow));
+    report("  gather, 1024 tokens", timer.median_us(few_push, few_gather),
+           (double)kFewTokens * (kTopk + 1) * kInRow);
     return 0;
 }
