@@ -32,3 +32,33 @@ def test_benchmark_cli(tmp_path, extra):
             stats = doc[phase][part]
             assert set(stats) == STAT_KEYS, sorted(stats)
             assert 0 < stats["min"] <= stats["p50"] <= stats["max"]
+
+
+def test_bench_py_prints_one_line_with_the_agreed_fields():
+    """`python bench.py --steps K --warmup W`: one JSON line; the step metric, the roofline of the dominant
+    kernel from at least 50 kernel-own samples whatever K is, the CPU baseline, and the other baseline shapes."""
+    repo = Path(__file__).resolve().parent.parent
+    cmd = [sys.executable, str(repo / "bench.py"), "--steps", "8", "--warmup", "2", "--cpu-reps", "1"]
+    print(" ".join(cmd), flush=True)
+    done = subprocess.run(cmd, capture_output=True, text=True, timeout=115)
+    assert done.returncode == 0, done.stderr[-2000:]
+    lines = [l for l in done.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    line = json.loads(lines[0])
+    for key, want in (("unit", "GB/s"), ("n_gpus", 1), ("steps", 8), ("warmup", 2), ("higher_is_better", True),
+                      ("vs_baseline", None), ("data", "synthetic")):
+        assert line[key] == want, key
+    assert "workload" in line["config"] and "model" not in line["config"]
+    assert abs(line["value"] - 829_816_832 / (line["ms_per_step"] * 1e-3) / 1e9) < 1.0
+    roof = line["roofline"]
+    assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and roof["unit"] == "GB/s"
+    assert abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
+    assert roof["samples"] >= 50
+    assert roof["traffic"] is None or roof["traffic"] >= roof["bytes_per_launch"]
+    cpu = line["cpu_baseline"]
+    assert cpu["kind"] == "port" and cpu["cores"] == 1 and cpu["value"] > 0 and cpu["sample"]
+    assert line["cpu_baseline_more"]["numpy_oracle"]["value"] > 0
+    for shape in ("decode_128", "qwen3_decode_128", "kimi_1024"):
+        assert line[shape]["step_us_wall"] > 0 and line[shape]["kernel_samples"] >= 50
+    assert line["prefill_4096"]["graph_replay"]["step_us_wall"] > 0
+    assert line["kimi_1024"]["bar_us_for_70pct"] == 37.0
