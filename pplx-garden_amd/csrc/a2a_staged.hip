@@ -334,6 +334,7 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     extern __shared__ uint32_t s_recv[];
     __shared__ uint32_t scratch[kRouteWaves];
     __shared__ uint32_t s_carry;
+    __shared__ uint8_t s_order[kMaxWorld];
     const uint32_t G = ws.num_groups, E = ws.num_experts, Le = ws.experts_per_rank;
     const uint32_t r = args.rank;
     const uint32_t first = r * Le;
@@ -349,6 +350,10 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     uint32_t *grp_src = grp_dst + G;     // [g]      rows this receiver gets from the sources numbered below g
     uint32_t *grp_cnt = grp_src + G;     // [g]      rows this receiver gets from source g
 
+    // The order in which this receiver lays out its sources (one byte per source, from the table the
+    // context computed once) travels with the counts and is read from LDS from then on: looked up in
+    // memory where it is used, it put a dependent trip into both scans and one in front of every row.
+    if (tid < G) s_order[tid] = (uint8_t)source_order_lookup(ws.order, r, tid);
     for (uint32_t w = tid; w < items; w += blockDim.x) {
         const uint32_t g = Le > 1 ? __umulhi(w, ws.le_magic) : w;
         const uint32_t le = w - g * Le;
@@ -390,7 +395,7 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
             const uint32_t e = first + le;
             uint32_t running = poff;
             for (uint32_t i = 0; i < G; ++i) {
-                const uint32_t g = source_order_lookup(ws.order, r, i);
+                const uint32_t g = s_order[i];
                 run_row[i * Le + le] = running;
                 if (publish) ws.slot_base[g * E + e] = running;
                 running += tot[g * Le + le];
@@ -422,7 +427,7 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
         uint32_t cnt = 0;
         if (s < items) {
             const uint32_t i = Le > 1 ? __umulhi(s, ws.le_magic) : s;
-            cnt = tot[source_order_lookup(ws.order, r, i) * Le + (s - i * Le)];
+            cnt = tot[s_order[i] * Le + (s - i * Le)];
         }
         const uint32_t incl = carry + block_inclusive_scan(cnt, scratch);
         if (s < items) seg[s] = incl - cnt;
@@ -463,7 +468,7 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
         }
         const uint32_t i = Le > 1 ? __umulhi(s, ws.le_magic) : s;
         const uint32_t le = s - i * Le;
-        const uint32_t g = source_order_lookup(ws.order, r, i);
+        const uint32_t g = s_order[i];
         const uint32_t j = row - seg[s];
         const uint32_t pos = excl[g * Le + le] + j;
         const uint32_t dst_row = run_row[s] + j;
