@@ -229,12 +229,15 @@ __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs
     uint32_t fill = 0;
     if constexpr (MODE != 0) {
         fill = turn[0] & 1u;
-        if (blockIdx.x == 0) {
+        // The hand-over between steps is the job of one workgroup of its own, the last of the grid:
+        // it has to wait for `turn` before it can do anything, which a chunk workgroup has not (its
+        // entries travel meanwhile, and it needs `fill` only for its final atomics).
+        if (blockIdx.x + 1 == gridDim.x) {
             uint32_t *next = totals + (size_t)(fill ^ 1u) * words;
             for (uint32_t i = threadIdx.x; i < words; i += kRouteBlock) next[i] = 0;
             if (threadIdx.x == 0) turn[1] = fill;
+            return;
         }
-        if (blockIdx.x >= args.block_start[G]) return;   // a step without entries: only the duties above
     }
     // Which source and which chunk of it this workgroup handles (uniform).
     uint32_t g = 0;
@@ -422,8 +425,8 @@ hipError_t launch_route(const RouteArgs &args, const Workspace &ws, uint32_t tot
 
 hipError_t launch_route_accumulate(const RouteArgs &args, const Workspace &ws, uint32_t total_blocks,
                                    hipStream_t stream, bool for_send, KernelTiming timing) {
-    // at least one workgroup: the launch also hands over the totals between steps
-    const dim3 grid(total_blocks != 0 ? total_blocks : 1);
+    // one workgroup per chunk and one more that hands over the totals between steps
+    const dim3 grid(total_blocks + 1);
     if (for_send) {
         hipLaunchKernelGGL(route_hist_kernel<2>, grid, dim3(kRouteBlock), 0, stream, args, ws);
     } else {
