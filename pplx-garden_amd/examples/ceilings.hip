@@ -19,6 +19,12 @@
 //              it in one burst); and the push with the same store policies and
 //              with half a token per workgroup
 //   1024       push and gather over the first 1024 tokens only
+//              and the push with its store policies, from 256 persistent
+//              workgroups (fewer concurrent writers), and turned round into a
+//              pull by destination row (sequential writes, input read 8 times)
+//   streams    a write-only sweep from 128 workgroups in 64 KiB pieces: few, long
+//              write streams are the fastest writes seen here (more workgroups
+//              or shorter pieces fall back to the plain sweep's rate)
 //
 // Every gather variant takes the number of units (token x 1 KiB piece) and
 // returns at once for a unit beyond it; the host derives each grid from the
@@ -283,6 +289,48 @@ __global__ __launch_bounds__(SPLIT ? 256 : 448) void push_policy(const uint8_t *
     }
 }
 
+// Write-only sweep in which each workgroup writes `chunk16` consecutive 16-byte pieces and then
+// jumps by grid x chunk: the number of concurrent write streams and their length are the knobs.
+// Few, long streams (128 workgroups x 64 KiB) are the fastest writes this GPU showed.
+__global__ __launch_bounds__(256) void write_streams(u32x4 *out, size_t n16, uint32_t chunk16, uint32_t seed) {
+    const size_t stride = (size_t)gridDim.x * chunk16;
+    for (size_t base = (size_t)blockIdx.x * chunk16; base < n16; base += stride) {
+        for (uint32_t i = threadIdx.x; i < chunk16; i += 256) {
+            const size_t idx = base + i;
+            if (idx < n16) {
+                const uint32_t v = (uint32_t)idx * 2654435761u + seed;
+                store_unit<kStoreSc1>(u32x4{v, v ^ 0x9E3779B9u, v * 3u, v + 7u}, out + idx);
+            }
+        }
+    }
+}
+
+// The push from persistent workgroups: workgroup b takes tokens b, b + grid, ... (a throttled
+// number of writers instead of one workgroup per token).
+__global__ __launch_bounds__(448) void push_persistent(const uint8_t *__restrict__ x, uint8_t *__restrict__ out,
+                                                       const uint32_t *__restrict__ slots, uint32_t tokens) {
+    const uint32_t c = threadIdx.x;
+    if (c >= kHidden / 16) return;
+    for (uint32_t t = blockIdx.x; t < tokens; t += gridDim.x) {
+        const u32x4 *p = reinterpret_cast<const u32x4 *>(x + (size_t)t * kInRow + (size_t)c * 32);
+        const u32x4 q = __builtin_nontemporal_load(p) ^ __builtin_nontemporal_load(p + 1);
+#pragma unroll
+        for (uint32_t k = 0; k < kTopk; ++k) {
+            store_unit<kStoreSc1>(q, reinterpret_cast<u32x4 *>(out + (size_t)slots[t * kTopk + k] * kOutRow + (size_t)c * 16));
+        }
+    }
+}
+
+// The pack turned round: one workgroup per DESTINATION row, rows in order, so the writes are one
+// sequential stream; the price is that every token's input is read once per route (8 times).
+__global__ __launch_bounds__(448) void pull_by_row(const uint8_t *__restrict__ x, uint8_t *__restrict__ out,
+                                                   const uint32_t *__restrict__ token_of_row, uint32_t rows) {
+    const uint32_t r = blockIdx.x, c = threadIdx.x;
+    if (r >= rows || c >= kHidden / 16) return;
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(x + (size_t)token_of_row[r] * kInRow + (size_t)c * 32);
+    store_unit<kStoreSc1>(p[0] ^ p[1], reinterpret_cast<u32x4 *>(out + (size_t)r * kOutRow + (size_t)c * 16));
+}
+
 struct Timer {
     hipStream_t stream;
     hipEvent_t start, stop;
@@ -338,6 +386,11 @@ int main() {
     uint32_t *d_slots;
     CHECK(hipMalloc(&d_slots, kRows * sizeof(uint32_t)));
     CHECK(hipMemcpy(d_slots, slots.data(), kRows * sizeof(uint32_t), hipMemcpyHostToDevice));
+    std::vector<uint32_t> token_of_row(kRows);
+    for (uint32_t i = 0; i < kRows; ++i) token_of_row[slots[i]] = i / kTopk;
+    uint32_t *d_token_of_row;
+    CHECK(hipMalloc(&d_token_of_row, kRows * sizeof(uint32_t)));
+    CHECK(hipMemcpy(d_token_of_row, token_of_row.data(), kRows * sizeof(uint32_t), hipMemcpyHostToDevice));
 
     uint8_t *x, *x_const, *dispatched, *y, *combined, *big_a, *big_b;
     const size_t sweep_bytes = (size_t)512 << 20;
@@ -384,6 +437,9 @@ int main() {
            (double)sweep_bytes);
     report("  write-only sweep, 512 MiB, 4096 workgroups",
            timer.median_us(read_other, [&] { hipLaunchKernelGGL(write_sweep, dim3(4096), dim3(256), 0, s, (u32x4 *)big_b, n16, 5u); }),
+           (double)sweep_bytes);
+    report("  write-only, 128 workgroups x 64 KiB streams, sc1",
+           timer.median_us(read_other, [&] { hipLaunchKernelGGL(write_streams, dim3(128), dim3(256), 0, s, (u32x4 *)big_b, n16, 4096u, 5u); }),
            (double)sweep_bytes);
     report("  copy, 512 MiB read + 512 MiB written",
            timer.median_us(read_other, [&] { hipLaunchKernelGGL(copy_sweep, dim3(2048), dim3(256), 0, s, (const u32x4 *)big_a, (u32x4 *)big_b, n16); }),
@@ -454,6 +510,13 @@ int main() {
     push_variant("  store sc1 (as the library)", (push_policy<kStoreSc1, false>), kTokens, 448);
     push_variant("  store sc0 sc1", (push_policy<kStoreSc0Sc1, false>), kTokens, 448);
     push_variant("  store sc1, half a token per workgroup", (push_policy<kStoreSc1, true>), 2 * kTokens, 256);
+    push_variant("  store sc1, 256 persistent workgroups", push_persistent, 256, 448);
+    report("  pulled by destination row (input read 8 times)",
+           timer.median_us(run_gather, [&] {
+               hipLaunchKernelGGL(pull_by_row, dim3(kRows), dim3(448), 0, s, (const uint8_t *)x, dispatched,
+                                  (const uint32_t *)d_token_of_row, kRows);
+           }),
+           push_bytes);
 
     // The same two shapes at 1024 tokens (the Kimi-K2 mixed batch): the push is a single wave of
     // workgroups, so nothing overlaps its launch, its reads and its burst of writes.
