@@ -104,7 +104,7 @@ int a2a_ctx_create(const a2a_config *config, a2a_ctx **out_ctx);
 int a2a_ctx_destroy(a2a_ctx *ctx);
 
 /* Text of the last error of this context (never NULL).  With ctx == NULL:
- * the last error of a2a_ctx_create on this thread. */
+ * the last error of a2a_ctx_create or a2a_dispatch_static on this thread. */
 const char *a2a_last_error(const a2a_ctx *ctx);
 
 /* Synchronises `stream`, then reads and clears the device-side error word
