@@ -19,7 +19,10 @@
 //              it in one burst); and the push with the same store policies and
 //              with half a token per workgroup
 //   1024       push and gather over the first 1024 tokens only
-//              and the push with its store policies, from 256 persistent
+//              the gather with fewer wavefronts per compute unit, and with the
+//              workgroup -> unit mapping arranged by XCD (a token per XCD; a
+//              contiguous eighth of the tokens per XCD);
+//              and the push with its store policies, by XCD ranges, from 256 persistent
 //              workgroups (fewer concurrent writers), and turned round into a
 //              pull by destination row (sequential writes, input read 8 times)
 //   streams    a write-only sweep from 128 workgroups in 64 KiB pieces: few, long
@@ -191,6 +194,23 @@ __global__ __launch_bounds__(64) void gather_policy(const uint8_t *__restrict__ 
     store_unit<POLICY>(sum_unit(v), out_of_unit(out, unit));
 }
 
+// Which XCD works on what: workgroups are dealt to the 8 XCDs round-robin (workgroup b runs on XCD
+// b % 8), so `unit = b` spreads every token's pieces over all XCDs and the output advances as ONE
+// front.  MAP 1 keeps the 14 pieces of a token on one XCD (tokens dealt round-robin); MAP 2 gives each
+// XCD a contiguous eighth of the tokens (8 separate output fronts).
+template <int MAP>
+__global__ __launch_bounds__(64) void gather_mapped(const uint8_t *__restrict__ y, uint8_t *__restrict__ out,
+                                                    const uint32_t *__restrict__ slots, uint32_t units) {
+    const uint32_t b = blockIdx.x;
+    if (b >= units) return;
+    const uint32_t xcd = b & 7, i = b >> 3;
+    const uint32_t unit = MAP == 1 ? ((i / kPieces) * 8 + xcd) * kPieces + i % kPieces : xcd * (kUnits / 8) + i;
+    if (unit >= units) return;
+    u32x4 v[kTopk];
+    load_unit(v, y, slots, unit);
+    store_unit<kStoreNt>(sum_unit(v), out_of_unit(out, unit));
+}
+
 // Ordinary (cached) loads instead of non-temporal ones.
 __global__ __launch_bounds__(64) void gather_cached_loads(const uint8_t *__restrict__ y, uint8_t *__restrict__ out,
                                                           const uint32_t *__restrict__ slots, uint32_t units) {
@@ -318,6 +338,20 @@ __global__ __launch_bounds__(448) void push_persistent(const uint8_t *__restrict
         for (uint32_t k = 0; k < kTopk; ++k) {
             store_unit<kStoreSc1>(q, reinterpret_cast<u32x4 *>(out + (size_t)slots[t * kTopk + k] * kOutRow + (size_t)c * 16));
         }
+    }
+}
+
+// The push with each XCD working through a contiguous eighth of the tokens.
+__global__ __launch_bounds__(448) void push_xcd_ranges(const uint8_t *__restrict__ x, uint8_t *__restrict__ out,
+                                                       const uint32_t *__restrict__ slots, uint32_t tokens) {
+    const uint32_t b = blockIdx.x, c = threadIdx.x;
+    const uint32_t t = (b & 7) * (tokens / 8) + (b >> 3);
+    if (b >= tokens || t >= tokens || c >= kHidden / 16) return;
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(x + (size_t)t * kInRow + (size_t)c * 32);
+    const u32x4 q = __builtin_nontemporal_load(p) ^ __builtin_nontemporal_load(p + 1);
+#pragma unroll
+    for (uint32_t k = 0; k < kTopk; ++k) {
+        store_unit<kStoreSc1>(q, reinterpret_cast<u32x4 *>(out + (size_t)slots[t * kTopk + k] * kOutRow + (size_t)c * 16));
     }
 }
 
@@ -487,6 +521,11 @@ int main() {
     variant("  pipelined, 2048 persistent wavefronts", gather_pipelined, 2048, 64, 0, 1);
     variant("  pipelined, 16384 persistent wavefronts", gather_pipelined, 16384, 64, 0, 1);
     variant("  a wavefront that only stores (3 + 1)", gather_store_wave, (kUnits + 2) / 3, 256, 0, 3);
+    variant("  16 of 32 wavefronts per CU (10 KiB LDS each)", gather_policy<kStoreNt>, kUnits, 64, 10 * 1024, 1);
+    variant("  8 of 32 wavefronts per CU (20 KiB LDS each)", gather_policy<kStoreNt>, kUnits, 64, 20 * 1024, 1);
+    variant("  4 of 32 wavefronts per CU (40 KiB LDS each)", gather_policy<kStoreNt>, kUnits, 64, 40 * 1024, 1);
+    variant("  a token's 14 pieces on one XCD", gather_mapped<1>, kUnits, 64, 0, 1);
+    variant("  each XCD a contiguous eighth of the tokens", gather_mapped<2>, kUnits, 64, 0, 1);
     variant("  16 KiB bursts from LDS, 256 workgroups", gather_bursts<1>, 256, 1024, 16 * 1024, 16);
     variant("  64 KiB bursts from LDS, 512 workgroups", gather_bursts<4>, 512, 1024, 64 * 1024, 64);
 
@@ -511,6 +550,7 @@ int main() {
     push_variant("  store sc0 sc1", (push_policy<kStoreSc0Sc1, false>), kTokens, 448);
     push_variant("  store sc1, half a token per workgroup", (push_policy<kStoreSc1, true>), 2 * kTokens, 256);
     push_variant("  store sc1, 256 persistent workgroups", push_persistent, 256, 448);
+    push_variant("  store sc1, each XCD a contiguous eighth", push_xcd_ranges, kTokens, 448);
     report("  pulled by destination row (input read 8 times)",
            timer.median_us(run_gather, [&] {
                hipLaunchKernelGGL(pull_by_row, dim3(kRows), dim3(448), 0, s, (const uint8_t *)x, dispatched,

@@ -37,7 +37,7 @@ def test_memory_ceilings_program_runs():
     print(done.stdout, done.stderr, flush=True)
     assert done.returncode == 0, done.stderr
     lines = [l for l in done.stdout.splitlines() if "GB/s" in l]
-    assert len(lines) == 35
+    assert len(lines) == 41
     assert any("push (pack's shape), random payload" in l for l in lines)
     assert any("gather (combine's shape)" in l for l in lines)
     for name in ("store nt (as the library)", "store sc0 sc1 nt", "cached loads", "pipelined, 2048", "only stores",
