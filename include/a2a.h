@@ -10,6 +10,12 @@
  * `stream` and never synchronise it, except `a2a_ctx_create`,
  * `a2a_ctx_destroy` and `a2a_ctx_status`.
  *
+ * A context is not re-entrant (the reference's methods take `&mut self`,
+ * a2a_context.rs:275,339,395,437): calls on ONE context, from whatever thread,
+ * must not overlap; different contexts are independent.  Calls may be made with
+ * any device current: each selects the context's device and restores the
+ * caller's.
+ *
  * Every function returns 0 on success, a positive `hipError_t` when a HIP call
  * failed, or a negative `a2a_status`; `a2a_last_error` gives the text.  No
  * exception crosses this boundary.

@@ -168,7 +168,8 @@ int check_rank(a2a_ctx *ctx, uint32_t rank) {
 
 // Arguments of the send half that do not depend on who receives.
 int check_send(a2a_ctx *ctx, const a2a_config &c, uint32_t rank, uint64_t num_tokens, const void *x,
-               uint64_t x_stride, uint32_t quantize, const float *xs, const int32_t *indices) {
+               uint64_t x_stride, uint32_t quantize, const float *xs, uint64_t xs_stride_elem,
+               uint64_t xs_stride_token, const int32_t *indices, uint64_t indices_stride) {
     if (num_tokens > c.max_num_tokens)
         return fail(ctx, A2A_ERR_TOO_MANY_TOKENS, "Number of tokens exceeds maximum allowed (rank %u: %llu > %u)",
                     rank, (unsigned long long)num_tokens, c.max_num_tokens);
@@ -198,11 +199,17 @@ int check_send(a2a_ctx *ctx, const a2a_config &c, uint32_t rank, uint64_t num_to
     if (!quantize && c.hidden_dim_scale != 0 && xs == nullptr)
         return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "rank %u: hidden_dim_scale is %u but x_scale is null",
                     rank, c.hidden_dim_scale);
+    if (indices_stride < c.num_experts_per_token && num_tokens > 1)
+        return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "rank %u: indices_stride %llu smaller than a row of %u ids", rank,
+                    (unsigned long long)indices_stride, c.num_experts_per_token);
+    // the kernels carry these strides as 32-bit element counts
+    if (indices_stride > 0xFFFFFFFFull || xs_stride_elem > 0xFFFFFFFFull || xs_stride_token > 0xFFFFFFFFull)
+        return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: an index or scale stride does not fit 32 bits", rank);
     return A2A_OK;
 }
 
 int check_recv(a2a_ctx *ctx, const a2a_config &c, uint32_t rank, const void *out_x, uint64_t out_stride,
-               const float *out_scale) {
+               const float *out_scale, uint64_t os_stride_elem, uint64_t os_stride_token) {
     if (out_x == nullptr) return A2A_OK;  // a rank may decline to receive
     if (!aligned16(out_x) || out_stride % 16 != 0)
         return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: out_x rows must be 16-byte aligned", rank);
@@ -212,6 +219,22 @@ int check_recv(a2a_ctx *ctx, const a2a_config &c, uint32_t rank, const void *out
     if (c.hidden_dim_scale != 0 && out_scale == nullptr)
         return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "rank %u: hidden_dim_scale is %u but out_x_scale is null",
                     rank, c.hidden_dim_scale);
+    if (os_stride_elem > 0xFFFFFFFFull || os_stride_token > 0xFFFFFFFFull)
+        return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: a stride of out_x_scale does not fit 32 bits", rank);
+    return A2A_OK;
+}
+
+// The recv half of a combine: the routes it gathers are those the dispatch of the step recorded
+// for the rank's group, so it cannot cover more tokens than that dispatch sent.
+int check_combine_tokens(a2a_ctx *ctx, uint32_t rank, uint64_t num_tokens, uint64_t indices_stride,
+                         uint64_t weights_stride) {
+    const uint32_t dispatched = ctx->num_tokens[rank / ctx->cfg.dp_size];
+    if (num_tokens > dispatched)
+        return fail(ctx, A2A_ERR_INVALID_ARGUMENT,
+                    "rank %u combines %llu tokens but the dispatch of this step routed %u of its group", rank,
+                    (unsigned long long)num_tokens, dispatched);
+    if (indices_stride > 0xFFFFFFFFull || weights_stride > 0xFFFFFFFFull)
+        return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: an index or weight stride does not fit 32 bits", rank);
     return A2A_OK;
 }
 
@@ -322,9 +345,12 @@ int dispatch_group(a2a_ctx *ctx, const a2a_config &c, const Workspace &ws, const
     const uint32_t N = c.world_size, K = c.num_experts_per_token;
     for (uint32_t r = 0; r < N; ++r) {
         const a2a_dispatch_args &a = args[r];
-        if (int rc = check_send(ctx, c, r, a.num_tokens, a.x_ptr, a.x_stride, quantize, a.x_scale_ptr, a.indices))
+        if (int rc = check_send(ctx, c, r, a.num_tokens, a.x_ptr, a.x_stride, quantize, a.x_scale_ptr,
+                                a.x_scale_stride_elem, a.x_scale_stride_token, a.indices, a.indices_stride))
             return rc;
-        if (int rc = check_recv(ctx, c, r, a.out_x, a.out_x_stride, a.out_x_scale)) return rc;
+        if (int rc = check_recv(ctx, c, r, a.out_x, a.out_x_stride, a.out_x_scale, a.out_x_scale_stride_elem,
+                                a.out_x_scale_stride_token))
+            return rc;
     }
 
     RouteArgs ra;
@@ -392,6 +418,9 @@ int dispatch_group(a2a_ctx *ctx, const a2a_config &c, const Workspace &ws, const
     if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && dispatch_small_fits(pa, ws, quantize != 0, tokens)) {
         e = launch_dispatch_small(pa, fa, ws, quantize != 0, tokens, s, pack_timing);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_small");
+    } else if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && dispatch_single_fits(pa, ws, quantize != 0, tokens)) {
+        e = launch_dispatch_single(pa, fa, ws, quantize != 0, tokens, s, pack_timing);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch dispatch_single");
     } else if (c.flags & A2A_FLAG_SEPARATE_ROUTING) {
         if (fused_routing_pays(fa, G, blocks)) {
             e = launch_route_fused(ra, fa, ws, s);
@@ -676,6 +705,7 @@ int a2a_combine(a2a_ctx *ctx, const a2a_combine_args *args, uint32_t expert_y_dt
         const a2a_combine_args &a = args[r];
         if (a.num_tokens > c.max_num_tokens)
             return fail(ctx, A2A_ERR_TOO_MANY_TOKENS, "Number of tokens exceeds maximum allowed (rank %u)", r);
+        if (int rc = check_combine_tokens(ctx, r, a.num_tokens, a.indices_stride, a.weights_stride)) return rc;
         if (a.expert_y != nullptr && (!aligned16(a.expert_y) || a.expert_y_stride % 16 != 0))
             return fail(ctx, A2A_ERR_UNSUPPORTED, "rank %u: expert_y rows must be 16-byte aligned", r);
         const uint64_t out_stride_bytes = a.out_tokens_stride * c.out_elemsize;
@@ -794,7 +824,8 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
     if (int rc = check_usable(ctx)) return rc;
     if (int rc = check_rank(ctx, rank)) return rc;
-    if (int rc = check_send(ctx, ctx->cfg, rank, num_tokens, x_ptr, x_stride, quantize, x_scale_ptr, indices))
+    if (int rc = check_send(ctx, ctx->cfg, rank, num_tokens, x_ptr, x_stride, quantize, x_scale_ptr,
+                            x_scale_stride_elem, x_scale_stride_token, indices, indices_stride))
         return rc;
     const a2a_config &c = ctx->cfg;
     DeviceGuard guard(c.device);
@@ -909,7 +940,9 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
     if (int rc = check_rank(ctx, rank)) return rc;
     if (!ctx->step_open || ctx->sent_mask == 0)
         return fail(ctx, A2A_ERR_BAD_ORDER, "a2a_dispatch_recv before any a2a_dispatch_send of the step");
-    if (int rc = check_recv(ctx, ctx->cfg, rank, out_x, out_x_stride, out_x_scale)) return rc;
+    if (int rc = check_recv(ctx, ctx->cfg, rank, out_x, out_x_stride, out_x_scale, out_x_scale_stride_elem,
+                            out_x_scale_stride_token))
+        return rc;
     const a2a_config &c = ctx->cfg;
     DeviceGuard guard(c.device);
     hipStream_t s = static_cast<hipStream_t>(stream);
@@ -986,6 +1019,7 @@ int a2a_combine_recv(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, size_t num_
         return fail(ctx, A2A_ERR_BAD_ORDER, "a2a_combine_recv before any a2a_combine_send of the step");
     if (num_tokens > c.max_num_tokens)
         return fail(ctx, A2A_ERR_TOO_MANY_TOKENS, "Number of tokens exceeds maximum allowed (rank %u)", rank);
+    if (int rc = check_combine_tokens(ctx, rank, num_tokens, indices_stride, weights_stride)) return rc;
     if (accumulate && c.dp_size != 1)   // python/pplx_garden/kernels/p2p_all_to_all.py:457-458
         return fail(ctx, A2A_ERR_UNSUPPORTED, "accumulate needs dp_size 1");
     if (elem_size_of(expert_y_dtype) != c.out_elemsize)

@@ -42,20 +42,26 @@ __device__ __forceinline__ void store_copy(u32x4 v, u32x4 *p) {
 // the row pointer, scale pointer and scale stride of route k (0 = no copy).
 // The row is loaded here, AFTER the routes are known: asking for it earlier to
 // hide its latency was measured slower at every size (4 us on the 4096-token
-// pack, 0.4 us on the 128-token one).  Whole workgroup.
+// pack, 0.4 us on the 128-token one).
+// The work is done by a TEAM of `team_threads` threads (a multiple of 64), in
+// which the caller is thread `team_tid`; a workgroup is one team or several of
+// the same size, each with a token and LDS arrays of its own.  Every thread of
+// the workgroup must call (there is a barrier inside); a team without a token
+// passes `live` false.
 template <bool QUANT>
 __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &src, uint32_t token, uint32_t K,
                                           uint64_t row_ptr, uint64_t scale_ptr, uint32_t scale_stride,
-                                          float *s_scale, uint64_t *s_scale_ptr, uint32_t *s_scale_stride) {
-    const uint32_t tid = threadIdx.x;
+                                          float *s_scale, uint64_t *s_scale_ptr, uint32_t *s_scale_stride,
+                                          uint32_t team_tid, uint32_t team_threads, bool live) {
+    const uint32_t tid = team_tid;
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
     const uint8_t *x_row = src.x + (size_t)token * src.x_stride;
 
     if constexpr (QUANT) {
-        const uint32_t num_chunks = args.hidden_dim / 16;  // 16 bf16 in, 16 fp8 out per lane
+        const uint32_t num_chunks = live ? args.hidden_dim / 16 : 0;  // 16 bf16 in, 16 fp8 out per lane
         const uint32_t Hs = args.hidden_dim_scale;
-        for (uint32_t base = wave * kWave; base < num_chunks; base += blockDim.x) {
+        for (uint32_t base = wave * kWave; base < num_chunks; base += team_threads) {
             const uint32_t c = base + lane;
             const bool active = c < num_chunks;
             u32x4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
@@ -77,20 +83,20 @@ __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &s
         // The token's scales meet in LDS so that each copy's scale row goes out
         // as one contiguous run instead of one 32-byte piece per wavefront.
         if (wave == 0 && lane < K) {
-            s_scale_ptr[lane] = scale_ptr;
+            s_scale_ptr[lane] = live ? scale_ptr : 0;
             s_scale_stride[lane] = scale_stride;
         }
         __syncthreads();
         const uint32_t Hl = Hs < (uint32_t)kMaxLdsScales ? Hs : (uint32_t)kMaxLdsScales;
-        for (uint32_t i = tid; i < K * Hl; i += blockDim.x) {
+        for (uint32_t i = tid; i < K * Hl; i += team_threads) {
             const uint32_t k = i / Hl;
             const uint32_t j = i - k * Hl;
             const uint64_t sp = s_scale_ptr[k];
             if (sp != 0) reinterpret_cast<float *>(sp)[(size_t)j * s_scale_stride[k]] = s_scale[j];
         }
     } else {
-        const uint32_t num_chunks = args.row_bytes / 16;
-        for (uint32_t c = tid; c < num_chunks; c += blockDim.x) {
+        const uint32_t num_chunks = live ? args.row_bytes / 16 : 0;
+        for (uint32_t c = tid; c < num_chunks; c += team_threads) {
             const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
             for (uint32_t k = 0; k < K; ++k) {
                 const uint64_t row = read_lane64(row_ptr, k);
@@ -99,9 +105,9 @@ __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &s
                 }
             }
         }
-        if (src.x_scale != nullptr) {
+        if (src.x_scale != nullptr && live) {
             const float *xs = src.x_scale + (size_t)token * src.xs_stride_token;
-            for (uint32_t j = tid; j < args.hidden_dim_scale; j += blockDim.x) {
+            for (uint32_t j = tid; j < args.hidden_dim_scale; j += team_threads) {
                 const float s = xs[(size_t)j * src.xs_stride_elem];
                 for (uint32_t k = 0; k < K; ++k) {
                     const uint64_t sp = read_lane64(scale_ptr, k);
@@ -203,7 +209,8 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
         scale_ptr = s_route_scale_ptr[lane];
         scale_stride = s_route_scale_stride[lane];
     }
-    push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride);
+    push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride,
+                     threadIdx.x, blockDim.x, true);
 }
 
 // Routing pass and dispatch pack in ONE launch, for small steps (decode).  The
@@ -232,7 +239,8 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
 // place before mine, so the order in which receivers lay out their sources
 // drops out too.
 //
-// Dynamic LDS: (G + 3) * E words and 8 bytes per token of the step.
+// Dynamic LDS: (G + 3) * E words and 8 bytes per token of the step; SINGLE:
+// 4 * E words (or G * Le, if that is more: the receiver workgroups' table).
 template <bool QUANT, bool SINGLE>
 __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs args, const FinalizeArgs fin,
                                                               const Workspace ws) {
@@ -276,17 +284,14 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
         const uint64_t ids = (uint64_t)(from.indices + (size_t)t * from.indices_stride) | (uint64_t)g << 56;
         tok_ids[ft] = t < effective_tokens(from.bound_m, from.num_tokens) ? ids : 0;
     }
-    uint32_t *cnt = s_dyn;                                  // [G][E] or, receivers, [G][Le]
-    uint32_t *prior = s_dyn + (size_t)G * E;                // [E] own source, tokens before mine
+    // SINGLE: a token workgroup keeps only the row of the one source, at the front
+    uint32_t *cnt = s_dyn;                                  // [G][E] (SINGLE: [E]) or, receivers, [G][Le]
+    uint32_t *prior = s_dyn + (SINGLE ? (size_t)E : (size_t)G * E);   // [E] own source, tokens before mine
     uint32_t *rows_before = prior + E;                      // [E] padded rows of all experts before e
     uint32_t *copies_before = rows_before + E;              // [E] copies of the sources laid out before mine
     const uint32_t table = receiver ? G * Le : G * E + E;
     if (SINGLE && !receiver) {
-        // only the row of the one source and the counts before my token are used
-        for (uint32_t i = tid; i < E; i += blockDim.x) {
-            s_dyn[(args.single_source - 1) * E + i] = 0;
-            s_dyn[G * E + i] = 0;
-        }
+        for (uint32_t i = tid; i < 2 * E; i += blockDim.x) s_dyn[i] = 0;   // cnt and prior
     } else {
         for (uint32_t i = tid; i < table; i += blockDim.x) s_dyn[i] = 0;
     }
@@ -352,7 +357,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
                 const uint32_t le = x - rank * Le;   // wraps for experts of lower ranks
                 if (le < Le) atomicAdd(&cnt[src_of[j] * Le + le], 1u);
             } else {
-                atomicAdd(&cnt[src_of[j] * E + x], 1u);
+                atomicAdd(&cnt[(SINGLE ? 0 : src_of[j]) * E + x], 1u);
                 const uint32_t f = f0 + j * blockDim.x + tid;
                 if (src_of[j] == my_g && f < my_first) atomicAdd(&prior[x], 1u);
             }
@@ -376,7 +381,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
         const uint32_t e = e0 + tid;
         uint32_t total = 0, before = 0;
         if (SINGLE) {
-            total = e < E ? cnt[my_g * E + e] : 0;   // nobody else sends: nothing is laid out before mine
+            total = e < E ? cnt[e] : 0;   // nobody else sends: nothing is laid out before mine
         } else if (e < E) {
             const uint32_t r = owner_of_expert(ws, e);
             bool seen = false;
@@ -417,7 +422,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
         uint32_t run = 0;
         for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
             const uint32_t e = e0 + lane;
-            const uint32_t v = e < E ? cnt[my_g * E + e] : 0;
+            const uint32_t v = e < E ? cnt[(SINGLE ? 0 : my_g) * E + e] : 0;
             const uint32_t incl = run + wave_inclusive_scan(v, lane);
             if (e < E) {
                 ws.num_routed[my_g * E + e] = v;
@@ -453,7 +458,190 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
             ws.token_offset[(size_t)my_g * ws.max_tk + entry] = toff;
         }
     }
-    push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride);
+    push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride,
+                     threadIdx.x, blockDim.x, true);
+}
+
+// Routing pass and dispatch pack in ONE launch for steps of ONE source with
+// dense index rows that are too large for dispatch_small_kernel (a mixed batch
+// of about a thousand tokens on one GPU's share).  What makes the one-launch
+// dispatch of small steps expensive as steps grow is that every token's
+// workgroup counts every entry of the step; here a workgroup counts once for
+// `per_group` tokens (at most kTokensPerGroup; the host picks it so that the
+// token workgroups are about as many as the compute units): it is made of
+// teams of wavefronts, each as wide as a token row needs, that move one token
+// each per round.  As in
+// dispatch_small_kernel no workgroup depends on another, the receiver
+// workgroups follow the token workgroups in the grid, and the rows are the
+// same: first row of the expert in its receiver + copies of earlier tokens to
+// the expert + copies of this token at an earlier k.
+//
+// Dynamic LDS: 3 * E words (or G * Le, if that is more: the receivers' table).
+constexpr uint32_t kTokensPerGroup = 4;
+constexpr uint32_t kMaxGroupRoutes = kTokensPerGroup * A2A_MAX_EXPERTS_PER_TOKEN;
+
+template <bool QUANT>
+__global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs args, const FinalizeArgs fin,
+                                                               const Workspace ws, const uint32_t team_threads,
+                                                               const uint32_t per_group) {
+    extern __shared__ uint32_t s_tab[];
+    __shared__ float s_scale[kTokensPerGroup][QUANT ? kMaxLdsScales : 1];   // [team]: at most kTokensPerGroup teams
+    __shared__ uint64_t s_scale_ptr[kTokensPerGroup][A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint32_t s_scale_stride[kTokensPerGroup][A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint64_t s_row_ptr[kMaxGroupRoutes];            // per route of the workgroup's tokens
+    __shared__ uint64_t s_route_scale_ptr[kMaxGroupRoutes];
+    __shared__ uint32_t s_route_scale_stride[kMaxGroupRoutes];
+    __shared__ uint32_t s_route_expert[kMaxGroupRoutes];
+    __shared__ uint32_t scratch[kRouteWaves];
+    __shared__ uint32_t s_carry;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t G = ws.num_groups, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
+    const uint32_t my_g = args.single_source - 1;
+    const PushSrc &src = args.src[my_g];
+    const uint32_t token_groups = (src.num_tokens + per_group - 1) / per_group;
+    const bool receiver = blockIdx.x >= token_groups;
+    const uint32_t tokens = effective_tokens(src.bound_m, src.num_tokens);
+    const uint32_t flat_entries = tokens * K;
+    const uint32_t first_token = blockIdx.x * per_group;                // token workgroups
+    const uint32_t my_first = first_token * K;                          // flat index of my first entry
+    // every token of mine is past the bound: nothing to send; the first workgroup stays (it publishes the totals)
+    if (!receiver && blockIdx.x != 0 && first_token >= tokens) return;
+
+    uint32_t *cnt = s_tab;                 // [E] entries per expert; receivers: [G][Le]
+    uint32_t *prior = s_tab + E;           // [E] entries per expert before my first token
+    uint32_t *rows_before = prior + E;     // [E] padded rows of all experts before e
+    const uint32_t table = receiver ? G * Le : 2 * E;
+    for (uint32_t i = tid; i < table; i += blockDim.x) s_tab[i] = 0;
+    // Sources without tokens have no workgroup of their own: the first receiver
+    // workgroup (the first workgroup, if nobody receives) clears their tables.
+    if (blockIdx.x == (fin.recv_mask != 0 ? token_groups : 0)) {
+        for (uint32_t g = 0; g < G; ++g) {
+            if (args.src[g].num_tokens != 0) continue;
+            for (uint32_t e = tid; e < E; e += blockDim.x) {
+                ws.num_routed[g * E + e] = 0;
+                ws.expert_offsets[g * E + e] = 0;
+            }
+        }
+    }
+    // The routes of my tokens: one thread each.
+    const uint32_t my_routes = per_group * K;
+    uint32_t my_expert = 0xFFFFFFFFu;
+    if (!receiver && tid < my_routes && my_first + tid < flat_entries) {
+        my_expert = (uint32_t)src.indices[my_first + tid];
+    }
+    __syncthreads();
+
+    // One pass over the entries of the step, kBatch loads in flight per lane.
+    constexpr uint32_t kBatch = 8;
+    const uint32_t rank = blockIdx.x - token_groups;        // receivers only
+    for (uint32_t f0 = 0; f0 < flat_entries; f0 += kBatch * blockDim.x) {
+        uint32_t expert[kBatch];
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t f = f0 + j * blockDim.x + tid;
+            expert[j] = f < flat_entries ? (uint32_t)src.indices[f] : 0xFFFFFFFFu;
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t x = expert[j];
+            if (x >= E) continue;
+            if (receiver) {
+                const uint32_t le = x - rank * Le;   // wraps for experts of lower ranks
+                if (le < Le) atomicAdd(&cnt[my_g * Le + le], 1u);
+            } else {
+                atomicAdd(&cnt[x], 1u);
+                if (f0 + j * blockDim.x + tid < my_first) atomicAdd(&prior[x], 1u);
+            }
+        }
+    }
+    if (!receiver && tid < my_routes) s_route_expert[tid] = my_expert;
+    __syncthreads();
+
+    if (receiver) {
+        if (fin.recv_mask >> rank & 1) layout_from_totals(fin, ws, rank, cnt, scratch);
+        return;
+    }
+
+    // Per expert: padded rows of the experts before it (the difference to the scan
+    // at the first expert of a receiver is the expert's first row there).
+    const uint32_t pad = ws.expert_padding;
+    uint32_t carry = 0;
+    for (uint32_t e0 = 0; e0 < E; e0 += blockDim.x) {
+        const uint32_t e = e0 + tid;
+        const uint32_t total = e < E ? cnt[e] : 0;
+        const uint32_t padded = e < E ? (total + pad - 1) / pad * pad : 0;
+        const uint32_t incl = carry + block_inclusive_scan(padded, scratch);
+        if (e < E) rows_before[e] = incl - padded;
+        if (e0 + blockDim.x < E) {   // uniform: another round follows
+            if (tid == blockDim.x - 1) s_carry = incl;
+            __syncthreads();
+            carry = s_carry;
+        }
+    }
+    __syncthreads();
+
+    // The first workgroup publishes the source's totals (last wavefront).
+    if (blockIdx.x == 0 && tid / kWave == blockDim.x / kWave - 1) {
+        uint32_t run = 0;
+        for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
+            const uint32_t e = e0 + lane;
+            const uint32_t v = e < E ? cnt[e] : 0;
+            const uint32_t incl = run + wave_inclusive_scan(v, lane);
+            if (e < E) {
+                ws.num_routed[my_g * E + e] = v;
+                ws.expert_offsets[my_g * E + e] = incl;
+            }
+            run = __shfl(incl, kWave - 1);
+        }
+    }
+
+    // One thread per route of my tokens resolves it from LDS alone.
+    if (tid < my_routes && my_first + tid < flat_entries) {
+        uint64_t row_ptr = 0, scale_ptr = 0;
+        uint32_t scale_stride = 0;
+        uint32_t slot = kInvalidSlot, toff = 0;
+        if (my_expert < E) {
+            // copies of the source before this one: those of earlier workgroups' tokens, then mine
+            uint32_t earlier = 0;
+            for (uint32_t q = 0; q < tid; ++q) earlier += s_route_expert[q] == my_expert ? 1u : 0u;
+            toff = prior[my_expert] + earlier;
+            const uint32_t r = owner_of_expert(ws, my_expert);
+            const uint32_t row = rows_before[my_expert] - rows_before[r * Le];
+            slot = resolve_copy(args.dst[r], ws, row + toff, true, &row_ptr, &scale_ptr, &scale_stride);
+        } else {
+            atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
+        }
+        ws.route_slot[(size_t)my_g * ws.max_tk + my_first + tid] = slot;
+        ws.token_offset[(size_t)my_g * ws.max_tk + my_first + tid] = toff;
+        s_row_ptr[tid] = row_ptr;
+        s_route_scale_ptr[tid] = scale_ptr;
+        s_route_scale_stride[tid] = scale_stride;
+    }
+    __syncthreads();
+
+    // The teams move one token each per round.  The rows are asked for only now: asking for the
+    // first two rounds' rows before the entries, or between asking for the entries and counting
+    // them, made the 1024-token step 3 and 4 us slower.
+    const uint32_t teams = blockDim.x / team_threads;
+    const uint32_t team = tid / team_threads;
+    const uint32_t team_tid = tid - team * team_threads;
+    for (uint32_t first = 0; first < per_group; first += teams) {
+        const uint32_t mine = first + team;                  // which of the workgroup's tokens
+        const uint32_t token = first_token + mine;
+        const bool live = mine < per_group && token < tokens;
+        uint64_t row_ptr = 0, scale_ptr = 0;
+        uint32_t scale_stride = 0;
+        if (live && lane < K) {
+            row_ptr = s_row_ptr[mine * K + lane];
+            scale_ptr = s_route_scale_ptr[mine * K + lane];
+            scale_stride = s_route_scale_stride[mine * K + lane];
+        }
+        push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale[team], s_scale_ptr[team],
+                         s_scale_stride[team], team_tid, team_threads, live);
+        __syncthreads();   // the team's LDS arrays are reused by the next round
+    }
 }
 
 // Pack of a large group step, after a routing launch that left, per chunk, the
@@ -618,7 +806,8 @@ __global__ __launch_bounds__(1024) void dispatch_resolve_kernel(const PushArgs a
         scale_ptr = s_route_scale_ptr[lane];
         scale_stride = s_route_scale_stride[lane];
     }
-    push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride);
+    push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride,
+                     threadIdx.x, blockDim.x, true);
 }
 
 hipError_t launch_dispatch_push(const PushArgs &args, const Workspace &ws, bool quantize,
@@ -653,7 +842,7 @@ hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, 
     const uint32_t blocks = total_tokens + (fin.recv_mask != 0 ? ws.world : 0);
     if (blocks == 0) return hipSuccess;
     const size_t table_words = (((size_t)ws.num_groups + 3) * ws.num_experts + 1) & ~(size_t)1;
-    const size_t lds = table_words * sizeof(uint32_t) + (size_t)total_tokens * sizeof(uint64_t);
+    size_t lds = table_words * sizeof(uint32_t) + (size_t)total_tokens * sizeof(uint64_t);
     // One source with tokens whose index rows are dense: the flat-array variant.
     PushArgs a = args;
     a.single_source = 0;
@@ -664,6 +853,11 @@ hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, 
         a.single_source = g + 1;
     }
     if (senders != 1 || args.src[a.single_source - 1].indices_stride != ws.topk) a.single_source = 0;
+    if (a.single_source != 0) {
+        const size_t tokens_words = 4 * (size_t)ws.num_experts;
+        const size_t receiver_words = (size_t)ws.num_groups * ws.experts_per_rank;
+        lds = (tokens_words > receiver_words ? tokens_words : receiver_words) * sizeof(uint32_t);
+    }
 #define A2A_LAUNCH_SMALL(Q, S)                                                                                       \
     hipExtLaunchKernelGGL((dispatch_small_kernel<Q, S>), dim3(blocks), dim3(threads), lds, stream, timing.start,  \
                           timing.stop, 0, a, fin, ws)
@@ -673,6 +867,68 @@ hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, 
         if (a.single_source != 0) A2A_LAUNCH_SMALL(false, true); else A2A_LAUNCH_SMALL(false, false);
     }
 #undef A2A_LAUNCH_SMALL
+    return hipGetLastError();
+}
+
+// Tokens per workgroup of dispatch_single_kernel: as many as it takes to have about one token
+// workgroup per compute unit (every workgroup counts all entries, so fewer workgroups count
+// less; but a compute unit without a workgroup moves no rows).  Measured on the 1024-token
+// step with 2 / 4 / 8 tokens a workgroup: 47.4 / 44.9 / 51.1 us.
+uint32_t single_tokens_per_group(uint32_t total_tokens) {
+    constexpr uint32_t kComputeUnits = 256;
+    const uint32_t per_group = (total_tokens + kComputeUnits - 1) / kComputeUnits;
+    return per_group < 1 ? 1 : per_group > kTokensPerGroup ? kTokensPerGroup : per_group;
+}
+
+// Threads of a dispatch_single_kernel workgroup: as many teams of `team` threads as fit, at most
+// one per token of the workgroup.
+uint32_t single_threads(uint32_t team, uint32_t per_group) {
+    uint32_t teams = 1024 / team;
+    if (teams > per_group) teams = per_group;
+    return teams * team;
+}
+
+// Whether a step takes dispatch_single_kernel: one source has tokens, its index rows are dense,
+// and the step is of the size where counting its entries once per kTokensPerGroup tokens is
+// cheaper than a routing launch in front of the pack.
+bool dispatch_single_fits(const PushArgs &args, const Workspace &ws, bool quantize, uint32_t total_tokens) {
+    uint32_t senders = 0, g_single = 0;
+    for (uint32_t g = 0; g < ws.num_groups; ++g) {
+        if (args.src[g].num_tokens == 0) continue;
+        ++senders;
+        g_single = g;
+    }
+    if (senders != 1 || args.src[g_single].indices_stride != ws.topk) return false;
+    const uint64_t entries = (uint64_t)total_tokens * ws.topk;
+    const uint32_t per_group = single_tokens_per_group(total_tokens);
+    const uint32_t threads = single_threads(push_threads(args, quantize), per_group);
+    // one thread per route of the workgroup's tokens and per local expert; the receivers' table in LDS
+    return entries <= kSingleMaxEntries && per_group * ws.topk <= threads && ws.experts_per_rank <= threads &&
+           (size_t)ws.num_groups * ws.experts_per_rank <= 8192;
+}
+
+hipError_t launch_dispatch_single(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
+                                  bool quantize, uint32_t total_tokens, hipStream_t stream, KernelTiming timing) {
+    if (total_tokens == 0) return hipSuccess;
+    const uint32_t team = push_threads(args, quantize);
+    const uint32_t per_group = single_tokens_per_group(total_tokens);
+    const uint32_t threads = single_threads(team, per_group);
+    const uint32_t blocks = (total_tokens + per_group - 1) / per_group + (fin.recv_mask != 0 ? ws.world : 0);
+    const size_t token_words = 3 * (size_t)ws.num_experts;
+    const size_t receiver_words = (size_t)ws.num_groups * ws.experts_per_rank;
+    const size_t lds = (token_words > receiver_words ? token_words : receiver_words) * sizeof(uint32_t);
+    PushArgs a = args;
+    a.single_source = 0;
+    for (uint32_t g = 0; g < ws.num_groups; ++g) {
+        if (args.src[g].num_tokens != 0) a.single_source = g + 1;
+    }
+    if (quantize) {
+        hipExtLaunchKernelGGL(dispatch_single_kernel<true>, dim3(blocks), dim3(threads), lds, stream, timing.start,
+                              timing.stop, 0, a, fin, ws, team, per_group);
+    } else {
+        hipExtLaunchKernelGGL(dispatch_single_kernel<false>, dim3(blocks), dim3(threads), lds, stream, timing.start,
+                              timing.stop, 0, a, fin, ws, team, per_group);
+    }
     return hipGetLastError();
 }
 

@@ -176,6 +176,13 @@ bool dispatch_small_fits(const PushArgs &args, const Workspace &ws, bool quantiz
 hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
                                  bool quantize, uint32_t total_tokens, hipStream_t stream,
                                  KernelTiming timing = KernelTiming());
+// One-launch routing + pack for steps of one source with dense index rows that are too large for
+// the small-step kernel.
+constexpr uint32_t kSingleMaxEntries = 8192;
+bool dispatch_single_fits(const PushArgs &args, const Workspace &ws, bool quantize, uint32_t total_tokens);
+hipError_t launch_dispatch_single(const PushArgs &args, const FinalizeArgs &fin, const Workspace &ws,
+                                  bool quantize, uint32_t total_tokens, hipStream_t stream,
+                                  KernelTiming timing = KernelTiming());
 hipError_t launch_combine_gather(const CombArgs &args, const Workspace &ws, uint32_t in_dtype,
                                  uint32_t out_dtype, uint32_t total_tokens, hipStream_t stream,
                                  KernelTiming timing = KernelTiming());

@@ -19,6 +19,8 @@ CONFIGS = [
     # large enough for the two-launch dispatch (4 groups x 700 tokens x 8 = 22 400 entries)
     RefConfig("dp2_two_launch", 8, 2, 700, 32, 256, None, 8, BF16, BF16, None, expert_padding=4, node_size=4),
     RefConfig("dp4_two_launch_fp8", 8, 4, 1300, 48, 512, 4, 8, FP8, BF16, F32, node_size=8),
+    # one group of 600 tokens x 6: the one-launch dispatch of a larger single source, rows copied as bytes
+    RefConfig("dp8_single_group_larger", 8, 8, 600, 24, 256, None, 6, BF16, BF16, None, expert_padding=3),
 ]
 
 

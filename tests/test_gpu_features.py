@@ -232,6 +232,27 @@ def test_errors_are_reported_not_faulted():
         with pytest.raises(RuntimeError, match="16-byte"):
             ctx.dispatch_send(0, 4, x.data_ptr() + 2, 2 * H, None, None, None, bad.data_ptr(), case.topk, 0,
                               case.topk, None, 0, quantize=True)
+        # index rows closer together than K ids, and a stride the kernels' 32-bit fields cannot carry
+        with pytest.raises(RuntimeError, match="indices_stride"):
+            ctx.dispatch_send(0, 4, x.data_ptr(), 2 * H, None, None, None, bad.data_ptr(), case.topk - 1, 0,
+                              case.topk, None, 0, quantize=True)
+        with pytest.raises(RuntimeError, match="32 bits"):
+            ctx.dispatch_send(0, 4, x.data_ptr(), 2 * H, None, None, None, bad.data_ptr(), 1 << 32, 0,
+                              case.topk, None, 0, quantize=True)
+        # a combine of more tokens than the step's dispatch routed for that rank would gather stale routes
+        out = torch.zeros((case.num_tokens, H), dtype=torch.bfloat16, device=DEV)
+        y = torch.zeros((rows, H), dtype=torch.bfloat16, device=DEV)
+        with pytest.raises(RuntimeError, match="combines"):
+            per_rank = []
+            for r in range(N):
+                a = native.A2ACombineArgs()
+                a.expert_y, a.expert_y_stride, a.expert_y_rows = y.data_ptr(), 2 * H, rows
+                if r == 1:                                 # rank 1 sent nothing in the dispatch above
+                    a.num_tokens, a.out_tokens, a.out_tokens_stride = 2, out.data_ptr(), H
+                    a.indices, a.indices_stride = bad.view(torch.uint32).to(DEV).data_ptr(), case.topk
+                    a.weights, a.weights_stride = w.data_ptr(), case.topk
+                per_rank.append(a)
+            ctx.combine(per_rank, torch.bfloat16, False, 0)
     finally:
         for op in ops:
             op.destroy()
@@ -324,8 +345,9 @@ def test_operator_asserts_like_the_reference():
 
 @pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
 @pytest.mark.parametrize("case,sources", [(C1, "all"), (scaled(C1, 1200), "one"), (scaled(C1, 300), "all"),
-                                          (scaled(C1, 40), "ragged")],
-                         ids=["one_launch_dispatch", "two_launch_dispatch_one_source", "two_launch_dispatch", "ragged"])
+                                          (scaled(C1, 40), "ragged"), (scaled(C1, 900), "one")],
+                         ids=["one_launch_dispatch", "two_launch_dispatch_one_source", "two_launch_dispatch", "ragged",
+                              "one_launch_dispatch_larger_source"])
 def test_calls_can_be_captured_in_a_hip_graph(case, sources, split):
     """The calls only enqueue kernels whose arguments travel by value (no allocation, copy or
     synchronisation inside), so a dispatch + combine can be captured once and replayed
@@ -563,21 +585,15 @@ def test_operator_reports_the_reference_capacities():
                 op.destroy()
 
 
-@pytest.mark.parametrize("sender,bound,strided", [(0, None, False), (2, None, False), (3, 37, False), (1, 0, False),
-                                                   (2, None, True), (1, 5, True)],
-                         ids=["rank0", "rank2", "rank3_bound37", "rank1_bound0", "rank2_strided", "rank1_bound5_strided"])
-def test_one_launch_dispatch_with_a_single_source(sender, bound, strided):
-    """A small step in which ONE rank has tokens takes a variant of the one-launch dispatch that reads the
-    entries as a flat array, provided the index rows are dense; with a row stride other than K the general
-    variant runs.  Either way: any rank may be the sender, `bound_m` may shorten the step on the device, and
-    the result is the oracle's, bit for bit."""
-    case = C1                                      # 128 tokens, 128 experts over 8 ranks, top-8
+def _check_single_source(case, sender, bound, strided):
+    """Dispatch of a step in which only `sender` has tokens, against the oracle: counts, fp8 bytes, scales,
+    untouched rows, and the sender's routing tables."""
     N, Le, H, Hs, K = case.world_size, case.experts_per_rank, case.hidden_dim, case.hidden_dim_scale, case.topk
     world = [make_world(case, "all")[r] if r == sender else make_world(scaled(case, 0), "all")[r] for r in range(N)]
     rows = rows_needed(case, world)
     inputs = [oracle.RankInput(x=bf16_codes(rd.x), indices=rd.indices.numpy(), bound_m=bound if r == sender else None)
               for r, rd in enumerate(world)]
-    want = oracle.dispatch_world(inputs, num_experts=case.num_experts, world_size=N, node_size=N, expert_padding=1,
+    want = oracle.dispatch_world(inputs, num_experts=case.num_experts, world_size=N, node_size=N, expert_padding=case.expert_padding,
                                  out_rows=rows, quantize=True)
     _, ops = make_ops(case, DEV)
     try:
@@ -617,3 +633,26 @@ def test_one_launch_dispatch_with_a_single_source(sender, bound, strided):
     finally:
         for op in ops:
             op.destroy()
+
+
+@pytest.mark.parametrize("sender,bound,strided", [(0, None, False), (2, None, False), (3, 37, False), (1, 0, False),
+                                                   (2, None, True), (1, 5, True)],
+                         ids=["rank0", "rank2", "rank3_bound37", "rank1_bound0", "rank2_strided", "rank1_bound5_strided"])
+def test_one_launch_dispatch_with_a_single_source(sender, bound, strided):
+    """A small step in which ONE rank has tokens takes a variant of the one-launch dispatch that reads the
+    entries as a flat array, provided the index rows are dense; with a row stride other than K the general
+    variant runs.  Either way: any rank may be the sender, `bound_m` may shorten the step on the device, and
+    the result is the oracle's, bit for bit."""
+    _check_single_source(C1, sender, bound, strided)   # 128 tokens, 128 experts over 8 ranks, top-8
+
+
+@pytest.mark.parametrize("tokens,sender,bound,topk,pad", [(700, 2, None, 8, 1), (1024, 0, None, 8, 16), (702, 5, 333, 8, 1),
+                                                          (600, 1, 0, 8, 1), (640, 3, None, 5, 8), (1000, 7, 1, 3, 1)],
+                         ids=["700", "1024_pad16", "702_bound333", "600_bound0", "640_top5_pad8", "1000_top3_bound1"])
+def test_one_launch_dispatch_of_a_larger_single_source(tokens, sender, bound, topk, pad):
+    """Steps of one source that are too large for the one-launch dispatch of small steps (every token's
+    workgroup counting every entry) and have at most 8192 entries take a launch whose workgroups count
+    once for four tokens each.  Partial last workgroups, a bound inside a workgroup's four tokens, a bound
+    of zero and one, odd top-k, padded receive slots: the oracle's result, bit for bit."""
+    case = replace(scaled(C1, tokens), topk=topk, expert_padding=pad, name=f"single_{tokens}")
+    _check_single_source(case, sender, bound, False)
