@@ -72,9 +72,10 @@ def _oracle(case: Case, world, rows: int) -> WorldResult:
 def test_static_dispatch_matches_the_context_dispatch():
     case = Case("static_steps", 640, 512, 64, 4, 8, 9100, expert_padding=4)
     # tokens per rank of consecutive calls: large (two launches), smaller (one launch), large again but
-    # smaller than the first (the step totals of the first call must not leak), tiny, empty, large
+    # smaller than the first (the step totals of the first call must not leak), tiny, empty, one larger
+    # source alone (one launch whose workgroups take several tokens each), large
     steps = [[640, 600, 0, 512], [100, 0, 7, 64], [300, 310, 290, 5], [1, 0, 0, 0], [0, 0, 0, 0],
-             [640, 640, 640, 640]]
+             [0, 640, 0, 0], [640, 640, 640, 640]]
     stream = torch.cuda.current_stream(DEV).cuda_stream
     cfg = _config(case, case.num_tokens)
     ctx = native.AllToAllContext.create(
