@@ -314,6 +314,28 @@ def cpu_baseline_numpy(case, tokens: int):
     return time.perf_counter() - t0
 
 
+def cpu_baseline_torch(case, tokens: int):
+    """The torch restatement of the path (tensor ops on the CPU, torch's intra-op threads) on a sample of
+    `tokens` tokens of the same workload.  Returns (seconds for the sample, threads used)."""
+    import torch
+    from workloads import make_rank, rows_needed
+    sys.path.insert(0, str(REPO / "oracle"))
+    import a2a_oracle_torch as torch_oracle
+
+    N = case.world_size
+    world = [make_rank(case, 0, tokens)] + [make_rank(case, r, 0) for r in range(1, N)]
+    rows = rows_needed(case, world)
+    gen = torch.Generator().manual_seed(case.seed)
+    ys = [torch.rand((rows, case.hidden_dim), generator=gen).to(torch.bfloat16) for _ in range(N)]
+    t0 = time.perf_counter()
+    _, _, _, slots = torch_oracle.dispatch_world(
+        [w.x for w in world], [w.indices for w in world], num_experts=case.num_experts, world_size=N,
+        node_size=case.node_size or N, expert_padding=case.expert_padding, out_rows=rows)
+    torch_oracle.combine_world(ys, [w.indices for w in world], [w.weights for w in world], slots,
+                               num_experts=case.num_experts, world_size=N)
+    return time.perf_counter() - t0, torch.get_num_threads()
+
+
 def other_shape(case, device, routings: int, steps: int, warmup: int, ctx_flags: int, label: str, bar_us=None):
     """Wall time per step without events, the kernels' own durations from a pass with events, and the
     calls' p50 from a pass with events around every call."""
@@ -478,12 +500,17 @@ def main() -> int:
         dt_all, _ = cpu_baseline(case, cpu_rd, args.cpu_reps, threads=cores)
         sample_tokens = case.num_tokens
         dt_np = cpu_baseline_numpy(case, sample_tokens)
+        dt_torch, torch_threads = cpu_baseline_torch(case, sample_tokens)
         s_d, s_c = algorithmic_bytes(sample_tokens, case.hidden_dim, case.topk)
         cpu_more = {
             "routing_only_us_one_thread": round(route_dt * 1e6, 1),
             "all_cores": {"value": round((d_bytes + c_bytes) / dt_all / 1e9, 3), "unit": "GB/s", "cores": cores,
                           "us_per_step": round(dt_all * 1e6, 1),
                           "note": "same code, tokens split over OpenMP threads; routing stays on one thread"},
+            "torch_oracle_all_cores": {"value": round((s_d + s_c) / dt_torch / 1e9, 3), "unit": "GB/s",
+                                       "cores": torch_threads, "seconds": round(dt_torch, 2),
+                                       "sample": "the same 4096-token batch, once, through the torch restatement "
+                                                 "of the path (tensor ops on the CPU, torch's intra-op threads)"},
             "numpy_oracle": {"value": round((s_d + s_c) / dt_np / 1e9, 3), "unit": "GB/s",
                              "cores": 1, "seconds": round(dt_np, 2),
                              "sample": f"the same {sample_tokens}-token batch, once, through the numpy oracle "
