@@ -70,3 +70,34 @@ def test_full_size_combine_is_bit_exact_with_true_fma():
     cw.act()
     outs = cw.combine([rd.weights.numpy() for rd in world])
     np.testing.assert_array_equal(got.out_tokens[0], outs[0])
+
+
+def test_full_size_all_sources():
+    """The prefill shape with ALL 8 logical ranks sending 4096 tokens (32 768 tokens, 262 144 copies): the
+    group calls against the C restatement, dispatch and combine bit for bit."""
+    case = C3
+    device = torch.device("cuda:0")
+    world = make_world(case, "all")
+    rows = rows_needed(case, world)
+    N = case.world_size
+    rng = np.random.default_rng(1)
+    ys = [rng.integers(0x3C00, 0x4000, size=(rows, case.hidden_dim), dtype=np.uint16) for _ in range(N)]
+    got = run_gpu(case, world, rows, device, expert_y_override=ys)
+    c_oracle.set_threads(16)
+    try:
+        cw = c_oracle.CWorld(case.num_experts, N, N, case.expert_padding, case.hidden_dim, case.topk, rows)
+        cw.route_all([rd.indices.numpy() for rd in world])
+        cw.dispatch([bf16_codes(rd.x) for rd in world])
+        for r in range(N):
+            cw.y[r][:] = ys[r]
+        outs = cw.combine([rd.weights.numpy() for rd in world])
+    finally:
+        c_oracle.set_threads(1)
+    for r in range(N):
+        per_expert = cw.tpe[r * cw.Le:(r + 1) * cw.Le]
+        n = int(per_expert.sum())                      # padding 1: the rows are dense
+        np.testing.assert_array_equal(got.num_tokens[r], per_expert.astype(np.int32))
+        np.testing.assert_array_equal(got.x[r][:n], cw.out_x[r][:n])
+        np.testing.assert_array_equal(got.x_scale[r][:n].view(np.uint32), cw.out_s[r][:n].view(np.uint32))
+        assert (got.x[r][n:] == 0xA5).all()
+        np.testing.assert_array_equal(got.out_tokens[r], outs[r])
