@@ -107,8 +107,9 @@ struct PushArgs {
     uint32_t hidden_dim;
     uint32_t hidden_dim_scale;
     uint32_t topk_magic;                  // ceil(2^32 / K) (0 for K = 1): n / K = mulhi(n, magic) while n * K < 2^32
-    uint32_t single_source;               // one-launch dispatch of small steps: g + 1 when source g alone has tokens
-                                          // and its index rows are dense, else 0 (set by the launcher)
+    uint32_t single_source;               // set by the launchers.  One-launch dispatches: g + 1 when source g alone has
+                                          // tokens and its index rows are dense, else 0.  Resolving pack: nonzero
+                                          // when one source alone has tokens.
 };
 
 struct CombSrc {  // one per receiver rank: the expert outputs it holds
