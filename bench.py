@@ -81,9 +81,11 @@ def measured_traffic():
 
 
 class Workload:
-    """Buffers of one case with the GPU as rank 0 of N logical ranks."""
+    """Buffers of one case with the GPU as rank 0 of N logical ranks (`senders` "one": one GPU's share
+    of the group's work), or with every logical rank sending its own batch (`senders` "all": the work
+    of the whole group on this GPU)."""
 
-    def __init__(self, case, device, num_routings: int, context_flags: int = 0):
+    def __init__(self, case, device, num_routings: int, context_flags: int = 0, senders: str = "one"):
         import torch
         from workloads import make_rank, rows_needed
         from pplx_garden_amd.native.p2p_all_to_all import (A2ACombineArgs, A2ADispatchArgs,
@@ -99,44 +101,52 @@ class Workload:
             max_private_tokens=0, num_experts=case.num_experts, expert_padding=case.expert_padding,
             num_experts_per_token=K, dp_size=1, node_size=case.node_size or N, world_size=N,
             device=device.index or 0, flags=context_flags)
-        self.routings = []
+        self.senders = list(range(N)) if senders == "all" else [0]
+        self.routings = []                 # [routing][sender]
         rows = 1
         for i in range(num_routings):
-            rd = make_rank(replace(case, seed=case.seed + 100 * i), 0)
-            self.routings.append(rd)
-            empty = [make_rank(case, r, 0) for r in range(1, N)]
-            rows = max(rows, rows_needed(case, [rd] + empty))
+            sent = [make_rank(replace(case, seed=case.seed + 100 * i), r, T if r in self.senders else 0)
+                    for r in range(N)]
+            self.routings.append([sent[r] for r in self.senders])
+            rows = max(rows, rows_needed(case, sent))
         self.rows = rows
-        self.cpu_first = self.routings[0]
-        self.x = self.routings[0].x.to(device)
-        self.idx = [rd.indices.to(device) for rd in self.routings]
-        self.w = [rd.weights.to(device) for rd in self.routings]
+        self.cpu_first = self.routings[0][0]
+        self.x = [rd.x.to(device) for rd in self.routings[0]]                       # [sender]
+        self.idx = [[rd.indices.to(device) for rd in routing] for routing in self.routings]
+        self.w = [[rd.weights.to(device) for rd in routing] for routing in self.routings]
         self.out_n = [torch.zeros(Le, dtype=torch.int32, device=device) for _ in range(N)]
         self.out_x = [torch.zeros((rows, H), dtype=torch.uint8, device=device) for _ in range(N)]
         self.out_s = [torch.zeros((rows, Hs), dtype=torch.float32, device=device) for _ in range(N)]
-        gen = torch.Generator(device="cpu")
-        gen.manual_seed(case.seed + 5)
-        self.y = [torch.randn((rows, H), generator=gen).to(torch.bfloat16).to(device) for _ in range(N)]
-        self.out_tokens = torch.zeros((T, H), dtype=torch.bfloat16, device=device)
+        if senders == "all":               # N times the rows: drawn on the device
+            gen = torch.Generator(device=device)
+            gen.manual_seed(case.seed + 5)
+            self.y = [torch.randn((rows, H), generator=gen, device=device, dtype=torch.float32).to(torch.bfloat16)
+                      for _ in range(N)]
+        else:
+            gen = torch.Generator(device="cpu")
+            gen.manual_seed(case.seed + 5)
+            self.y = [torch.randn((rows, H), generator=gen).to(torch.bfloat16).to(device) for _ in range(N)]
+        self.out_tokens = [torch.zeros((T, H), dtype=torch.bfloat16, device=device) for _ in self.senders]
         self.dispatch_args = []
         self.combine_args = []
         for i in range(num_routings):
             d, c = [], []
             for r in range(N):
-                src = r == 0
+                src = r in self.senders
+                j = self.senders.index(r) if src else 0
                 d.append(A2ADispatchArgs(
-                    num_tokens=T if src else 0, x_ptr=self.x.data_ptr() if src else None, x_stride=2 * H,
+                    num_tokens=T if src else 0, x_ptr=self.x[j].data_ptr() if src else None, x_stride=2 * H,
                     x_scale_ptr=None, x_scale_stride_elem=0, x_scale_stride_token=0,
-                    indices=self.idx[i].data_ptr() if src else None, indices_stride=K,
-                    weights=self.w[i].data_ptr() if src else None, weights_stride=K, bound_m=None,
+                    indices=self.idx[i][j].data_ptr() if src else None, indices_stride=K,
+                    weights=self.w[i][j].data_ptr() if src else None, weights_stride=K, bound_m=None,
                     out_num_tokens=self.out_n[r].data_ptr(), out_x=self.out_x[r].data_ptr(),
                     out_x_stride=H, out_x_rows=rows, out_x_scale=self.out_s[r].data_ptr(),
                     out_x_scale_stride_elem=1, out_x_scale_stride_token=Hs))
                 c.append(A2ACombineArgs(
                     expert_y=self.y[r].data_ptr(), expert_y_stride=2 * H, expert_y_rows=rows,
-                    num_tokens=T if src else 0, out_tokens=self.out_tokens.data_ptr() if src else None,
-                    out_tokens_stride=H, indices=self.idx[i].data_ptr() if src else None,
-                    indices_stride=K, weights=self.w[i].data_ptr() if src else None, weights_stride=K,
+                    num_tokens=T if src else 0, out_tokens=self.out_tokens[j].data_ptr() if src else None,
+                    out_tokens_stride=H, indices=self.idx[i][j].data_ptr() if src else None,
+                    indices_stride=K, weights=self.w[i][j].data_ptr() if src else None, weights_stride=K,
                     bound_m=None))
             self.dispatch_args.append(self.ctx.pack_dispatch_args(d))
             self.combine_args.append(self.ctx.pack_combine_args(c))
@@ -336,16 +346,18 @@ def cpu_baseline_torch(case, tokens: int):
     return time.perf_counter() - t0, torch.get_num_threads()
 
 
-def other_shape(case, device, routings: int, steps: int, warmup: int, ctx_flags: int, label: str, bar_us=None):
+def other_shape(case, device, routings: int, steps: int, warmup: int, ctx_flags: int, label: str, bar_us=None,
+                senders: str = "one"):
     """Wall time per step without events, the kernels' own durations from a pass with events, and the
     calls' p50 from a pass with events around every call."""
     from pplx_garden_amd.utils.math import Statistics
-    wl = Workload(case, device, routings, ctx_flags)
+    wl = Workload(case, device, routings, ctx_flags, senders=senders)
+    num_senders = len(wl.senders)
     _, d, c, b, p, g, _ = time_workload(wl, steps, warmup, kernel_every=4, call_every=1)
     w, _, _, _, _, _, _ = time_workload(wl, steps, warmup)
     graph_s, _ = time_graph_replay(wl, steps, warmup)
     wl.close()
-    d_bytes, c_bytes = algorithmic_bytes(case.num_tokens, case.hidden_dim, case.topk)
+    d_bytes, c_bytes = algorithmic_bytes(case.num_tokens * num_senders, case.hidden_dim, case.topk)
     step_us = w / steps * 1e6
     out = {
         "workload": label,
@@ -476,7 +488,7 @@ def main() -> int:
     dominant, other = ((combine_roof, dispatch_roof) if g_stats.mean >= p_stats.mean
                        else (dispatch_roof, combine_roof))
 
-    decode = qwen = kimi = None
+    decode = qwen = kimi = whole_group = None
     if not args.no_decode:
         decode = other_shape(C2, device, args.routings, side_steps, args.warmup, ctx_flags, decode_label)
         decode["note"] = ("working set (26 MB) fits the 256 MB Infinity Cache and is not flushed between steps; "
@@ -485,6 +497,12 @@ def main() -> int:
                           "of every step (each event adds about 3 us)")
         qwen = other_shape(C1, device, args.routings, side_steps, args.warmup, ctx_flags, qwen_label)
         kimi = other_shape(C4, device, args.routings, side_steps, args.warmup, ctx_flags, kimi_label, bar_us=37.0)
+        # The work of the WHOLE group on this GPU: every logical rank sends its 4096 tokens (8 times the
+        # bytes of the headline's step, which is one GPU's share).  Not the baseline's configuration;
+        # reported beside it as the same kernels' sustained rate over a longer step.
+        whole_group = other_shape(C3, device, 2, 100, 20, ctx_flags,
+                                  "DeepSeek-V3 prefill, all 8 logical ranks send 4096 tokens each (32 768 tokens per "
+                                  "step on one GPU: 8 times one GPU's share)", senders="all")
 
     cpu = cpu_more = None
     if args.cpu_reps > 0:
@@ -565,6 +583,7 @@ def main() -> int:
         "decode_128": decode,
         "qwen3_decode_128": qwen,
         "kimi_1024": kimi,
+        "prefill_4096_all_ranks_send": whole_group,
         "roofline": dominant,
         "roofline_other": other,
         "cpu_baseline": cpu,

@@ -59,6 +59,8 @@ def test_bench_py_prints_one_line_with_the_agreed_fields():
     assert cpu["kind"] == "port" and cpu["cores"] == 1 and cpu["value"] > 0 and cpu["sample"]
     assert line["cpu_baseline_more"]["numpy_oracle"]["value"] > 0
     assert line["cpu_baseline_more"]["torch_oracle_all_cores"]["value"] > 0
+    whole = line["prefill_4096_all_ranks_send"]
+    assert whole["algorithmic_bytes"] == 8 * (301072384 + 528744448) and whole["step_us_wall"] > 0
     assert line["cpu_baseline_more"]["torch_oracle_all_cores"]["cores"] >= 1
     for shape in ("decode_128", "qwen3_decode_128", "kimi_1024"):
         assert line[shape]["step_us_wall"] > 0 and line[shape]["kernel_samples"] >= 50
