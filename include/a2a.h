@@ -98,9 +98,10 @@ typedef struct a2a_config {
 /* Allocate the staging buffers of the split calls in a2a_ctx_create instead of
  * on their first use. */
 #define A2A_FLAG_PREALLOC_STAGING 1u
-/* Never take the one-launch paths of small steps (routing counted inside the
- * dispatch or send kernel); always run the routing kernels, then the pack.
- * Results are identical either way; the flag exists to compare the two. */
+/* Never take the one-launch paths (routing counted inside the dispatch or send
+ * kernel: small steps, and group steps of one source up to 8192 copies); always
+ * run the routing kernels, then the pack.  Results are identical either way;
+ * the flag exists to compare the two. */
 #define A2A_FLAG_SEPARATE_ROUTING 2u
 
 /* replaces AllToAllContext::new, a2a_context.rs:124-259 */
