@@ -77,7 +77,7 @@ def build(verbose: bool = True) -> Path:
             failed = True
     if failed:
         raise RuntimeError("hipcc failed")
-    link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-o", str(library_path())]
+    link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objects, "-o", str(library_path()), "-ldl"]
     if verbose:
         print(" ".join(link), flush=True)
     subprocess.run(link, check=True)

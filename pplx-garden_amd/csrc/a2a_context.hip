@@ -8,6 +8,8 @@
 // with every logical rank on one GPU, stream order is the only synchronisation.
 #include <hip/hip_runtime.h>
 
+#include <dlfcn.h>
+
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -90,6 +92,44 @@ int check_usable(a2a_ctx *ctx) {
 }
 
 size_t align_up(size_t n, size_t a) { return (n + a - 1) / a * a; }
+
+// Named ranges for profilers around each call (`rocprofv3 --marker-trace`), with the names of the
+// reference's NVTX ranges (a2a_dispatch_send.cu:632, a2a_dispatch_recv.cu:316,
+// a2a_combine_send.cu:286, a2a_combine_recv.cu:236).  The ROCTX library is looked up at run time,
+// once: without it the library has no dependency on it and a range is two null checks.
+struct Roctx {
+    int (*push)(const char *) = nullptr;
+    int (*pop)() = nullptr;
+    Roctx() {
+        for (const char *name : {"librocprofiler-sdk-roctx.so.1", "librocprofiler-sdk-roctx.so", "libroctx64.so.4",
+                                 "libroctx64.so"}) {
+            void *lib = dlopen(name, RTLD_NOW | RTLD_LOCAL);
+            if (lib == nullptr) continue;
+            push = reinterpret_cast<int (*)(const char *)>(dlsym(lib, "roctxRangePushA"));
+            pop = reinterpret_cast<int (*)()>(dlsym(lib, "roctxRangePop"));
+            if (push != nullptr && pop != nullptr) return;
+            push = nullptr;
+            pop = nullptr;
+            dlclose(lib);
+        }
+    }
+};
+
+const Roctx &roctx() {
+    static const Roctx table;
+    return table;
+}
+
+struct ProfilerRange {
+    explicit ProfilerRange(const char *name) {
+        if (roctx().push != nullptr) roctx().push(name);
+    }
+    ~ProfilerRange() {
+        if (roctx().pop != nullptr) roctx().pop();
+    }
+    ProfilerRange(const ProfilerRange &) = delete;
+    ProfilerRange &operator=(const ProfilerRange &) = delete;
+};
 
 uint32_t ceil_div_u32(uint64_t n, uint64_t m) { return (uint32_t)((n + m - 1) / m); }
 
@@ -620,6 +660,7 @@ int a2a_ctx_status(a2a_ctx *ctx, void *stream, uint32_t *flags) {
 
 int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize, void *stream) {
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    ProfilerRange range("dispatch");
     if (int rc = check_usable(ctx)) return rc;
     if (args == nullptr) return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "null args");
     DeviceGuard guard(ctx->cfg.device);
@@ -641,6 +682,7 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
 int a2a_dispatch_static(const a2a_config *config, const a2a_dispatch_args *args, uint32_t quantize,
                         uint32_t *device_flags, void *stream) {
     if (config == nullptr || args == nullptr) return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "null argument");
+    ProfilerRange range("dispatch_static");
     if (int rc = check_config(*config)) return rc;
     const a2a_config &c = *config;
     if (c.flags != 0)
@@ -683,6 +725,7 @@ int a2a_dispatch_static(const a2a_config *config, const a2a_dispatch_args *args,
 int a2a_combine(a2a_ctx *ctx, const a2a_combine_args *args, uint32_t expert_y_dtype,
                 uint32_t accumulate, void *stream) {
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    ProfilerRange range("combine");
     if (int rc = check_usable(ctx)) return rc;
     if (args == nullptr) return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "null args");
     const a2a_config &c = ctx->cfg;
@@ -822,6 +865,7 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     (void)weights;
     (void)weights_stride;
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    ProfilerRange range("dispatch_send");
     if (int rc = check_usable(ctx)) return rc;
     if (int rc = check_rank(ctx, rank)) return rc;
     if (int rc = check_send(ctx, ctx->cfg, rank, num_tokens, x_ptr, x_stride, quantize, x_scale_ptr,
@@ -936,6 +980,7 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
                       size_t out_x_scale_stride_elem, size_t out_x_scale_stride_token,
                       void *stream) {
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    ProfilerRange range("dispatch_recv");
     if (int rc = check_usable(ctx)) return rc;
     if (int rc = check_rank(ctx, rank)) return rc;
     if (!ctx->step_open || ctx->sent_mask == 0)
@@ -974,6 +1019,7 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
 int a2a_combine_send(a2a_ctx *ctx, uint32_t rank, const void *expert_y, size_t expert_y_stride,
                      size_t expert_y_rows, void *stream) {
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    ProfilerRange range("combine_send");
     if (int rc = check_usable(ctx)) return rc;
     if (int rc = check_rank(ctx, rank)) return rc;
     if (!ctx->staging.allocated || !(ctx->staging.recv_mask >> rank & 1))
@@ -1012,6 +1058,7 @@ int a2a_combine_recv(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, size_t num_
                      void *stream) {
     (void)num_recv_tokens;
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
+    ProfilerRange range("combine_recv");
     if (int rc = check_usable(ctx)) return rc;
     if (int rc = check_rank(ctx, rank)) return rc;
     const a2a_config &c = ctx->cfg;
