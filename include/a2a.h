@@ -305,8 +305,9 @@ int a2a_ctx_read_table(a2a_ctx *ctx, uint32_t rank, uint32_t which,
  * kernel's duration, without the queue packets and idle time that events
  * recorded around a call add.  A2A_KERNEL_ROUTE is the routing launch that
  * precedes the pack of a large step; a step that counts its routing inside the
- * pack (a small one) or runs several routing kernels (A2A_FLAG_SEPARATE_ROUTING)
- * has no such launch and leaves those events alone.  One-shot: the request is
+ * pack (a small one, or one source alone with up to 8192 copies) or runs several
+ * routing kernels (A2A_FLAG_SEPARATE_ROUTING) has no such launch and leaves
+ * those events alone.  One-shot: the request is
  * consumed by that call.  Pass two nulls to withdraw it.  The stop event must
  * have completed before its time is read (synchronise the stream or the event). */
 enum { A2A_KERNEL_PACK = 0, A2A_KERNEL_GATHER = 1, A2A_KERNEL_ROUTE = 2 };
