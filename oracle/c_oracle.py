@@ -3,7 +3,7 @@
 from __future__ import annotations
 
 import ctypes
-from ctypes import POINTER, c_float, c_int, c_int32, c_size_t, c_uint8, c_uint16, c_uint32, c_void_p
+from ctypes import c_float, c_int, c_size_t, c_uint8, c_uint32, c_void_p
 from pathlib import Path
 
 import numpy as np

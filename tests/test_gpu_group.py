@@ -1,6 +1,5 @@
 """Parity of the group calls (every rank calls dispatch()/combine() with send and recv)."""
 
-import numpy as np
 import pytest
 import torch
 

@@ -2,9 +2,6 @@
 (including more routes than one scale-store round covers), hidden sizes that are not a multiple of a
 wavefront's slab, the largest group, repeated experts inside a token."""
 
-from dataclasses import replace
-
-import numpy as np
 import pytest
 import torch
 
