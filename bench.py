@@ -55,13 +55,22 @@ def algorithmic_bytes(T: int, H: int, K: int):
     return dispatch, combine
 
 
+def code_only(text: str) -> str:
+    """C++ source without its comments and blank lines, lines stripped: what the compiler sees, more or
+    less, so that rewording a comment does not make a counter summary look stale.  (No string literal
+    in these sources holds a comment marker.)"""
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    text = re.sub(r"//[^\n]*", "", text)
+    return "\n".join(line.strip() for line in text.splitlines() if line.strip())
+
+
 def kernel_sources_sha256() -> str:
-    """Fingerprint of the kernel sources this run uses: sha256 over the names and contents of
-    pplx-garden_amd/csrc/*, sorted by name."""
+    """Fingerprint of the kernel sources this run uses: sha256 over the names and the code (comments
+    and blank lines left out) of pplx-garden_amd/csrc/*, sorted by name."""
     h = hashlib.sha256()
     for path in sorted((REPO / "pplx-garden_amd" / "csrc").iterdir()):
         if path.is_file():
-            h.update(path.name.encode() + b"\0" + path.read_bytes() + b"\0")
+            h.update(path.name.encode() + b"\0" + code_only(path.read_text()).encode() + b"\0")
     return h.hexdigest()
 
 

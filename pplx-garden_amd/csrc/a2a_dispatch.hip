@@ -470,11 +470,10 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
 // `per_group` tokens (at most kTokensPerGroup; the host picks it so that the
 // token workgroups are about as many as the compute units): it is made of
 // teams of wavefronts, each as wide as a token row needs, that move one token
-// each per round.  As in
-// dispatch_small_kernel no workgroup depends on another, the receiver
-// workgroups follow the token workgroups in the grid, and the rows are the
-// same: first row of the expert in its receiver + copies of earlier tokens to
-// the expert + copies of this token at an earlier k.
+// each per round.  As in dispatch_small_kernel no workgroup depends on another,
+// the receiver workgroups follow the token workgroups in the grid, and the rows
+// are the same: first row of the expert in its receiver + copies of earlier
+// tokens to the expert + copies of this token at an earlier k.
 //
 // Dynamic LDS: 3 * E words (or G * Le, if that is more: the receivers' table).
 constexpr uint32_t kTokensPerGroup = 4;

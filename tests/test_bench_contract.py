@@ -39,6 +39,9 @@ def test_traffic_is_reported_only_for_the_sources_it_was_measured_on(tmp_path, m
     import bench
     fingerprint = bench.kernel_sources_sha256()
     assert len(fingerprint) == 64 and fingerprint == bench.kernel_sources_sha256()
+    # comments and blank lines do not count, code does
+    assert bench.code_only("int a = 1;  // one\n\n/* two\n lines */ int b;\n") == "int a = 1;\nint b;"
+    assert bench.code_only("int a = 2;") != bench.code_only("int a = 1;")
     traffic, note = bench.measured_traffic()
     if traffic:      # the committed summary belongs to the committed sources
         assert 0.99 * 528_744_448 < traffic["combine_gather_kernel"] < 1.05 * 528_744_448
