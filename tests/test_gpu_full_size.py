@@ -72,9 +72,10 @@ def test_full_size_combine_is_bit_exact_with_true_fma():
     np.testing.assert_array_equal(got.out_tokens[0], outs[0])
 
 
-def test_full_size_all_sources():
+@pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
+def test_full_size_all_sources(split):
     """The prefill shape with ALL 8 logical ranks sending 4096 tokens (32 768 tokens, 262 144 copies): the
-    group calls against the C restatement, dispatch and combine bit for bit."""
+    group calls, and the four split calls, against the C restatement, dispatch and combine bit for bit."""
     case = C3
     device = torch.device("cuda:0")
     world = make_world(case, "all")
@@ -82,7 +83,7 @@ def test_full_size_all_sources():
     N = case.world_size
     rng = np.random.default_rng(1)
     ys = [rng.integers(0x3C00, 0x4000, size=(rows, case.hidden_dim), dtype=np.uint16) for _ in range(N)]
-    got = run_gpu(case, world, rows, device, expert_y_override=ys)
+    got = run_gpu(case, world, rows, device, expert_y_override=ys, split=split)
     c_oracle.set_threads(16)
     try:
         cw = c_oracle.CWorld(case.num_experts, N, N, case.expert_padding, case.hidden_dim, case.topk, rows)
