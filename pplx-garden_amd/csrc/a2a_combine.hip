@@ -143,13 +143,18 @@ __device__ __forceinline__ void fma_chunk(const u32x4 raw, float w, float (&acc)
 constexpr int kCombineWaves = 1;    // wavefronts per workgroup; each works on its own
 constexpr int kCombineChunks = 1;   // 16-byte chunks of a row per lane
 constexpr int kSlabChunks = kWave * kCombineChunks;
+constexpr uint32_t kOneRankMaxTokens = 2048;   // largest step that takes the ONE_RANK variant of the gather
 
 // T: type of the expert_y rows, U: type of out_tokens.  One WAVEFRONT handles
 // one slab of 64 sixteen-byte chunks of one token; wavefronts share nothing, so
 // a compute unit keeps many of them in flight and the latency of resolving a
 // token's routes is hidden by the loads of its neighbours.  KFIX > 0 unrolls
-// the route loop (all K loads issued before the first use).
-template <typename T, typename U, int KFIX>
+// the route loop (all K loads issued before the first use).  ONE_RANK: one rank
+// alone has tokens and the step is small; its descriptor is read from a fixed
+// place in the argument block, which takes two dependent scalar loads out of
+// the head of every wavefront (0.1-0.4 us of a step of 128 to 1024 tokens; a
+// 4096-token step hides them and is 0.3 us faster without the variant).
+template <typename T, typename U, int KFIX, bool ONE_RANK>
 __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(const CombArgs args,
                                                                               const Workspace ws) {
     constexpr int V = vec_elems<T>();
@@ -163,11 +168,16 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
     const uint32_t unit = blockIdx.x * kCombineWaves + wave;
     const uint32_t token_global = unit / slabs;
     const uint32_t slab = unit - token_global * slabs;
-    if (token_global >= args.token_start[ws.world]) return;
-    uint32_t g = 0;
-    while (g + 1 < ws.world && token_global >= args.token_start[g + 1]) ++g;
-    const uint32_t token = token_global - args.token_start[g];
-    const CombDst &dst = args.dst[g];
+    uint32_t g = 0, token = token_global;
+    if constexpr (ONE_RANK) {
+        if (token_global >= args.token_start[kMaxWorld]) return;   // the total, at a fixed place
+        g = args.single_rank - 1;
+    } else {
+        if (token_global >= args.token_start[ws.world]) return;
+        while (g + 1 < ws.world && token_global >= args.token_start[g + 1]) ++g;
+        token = token_global - args.token_start[g];
+    }
+    const CombDst &dst = ONE_RANK ? args.single : args.dst[g];
     const uint32_t group = g / ws.dp_size;   // the routing tables belong to the rank's dp group
     if (token >= effective_tokens(dst.bound_m, dst.num_tokens)) return;
 
@@ -274,20 +284,32 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
 }
 
 template <typename T, typename U>
-static hipError_t launch_typed(const CombArgs &args, const Workspace &ws, uint32_t total_tokens,
+static hipError_t launch_typed(const CombArgs &given, const Workspace &ws, uint32_t total_tokens,
                                hipStream_t stream, KernelTiming timing) {
     constexpr int V = vec_elems<T>();
+    CombArgs args = given;
+    uint32_t ranks_with_tokens = 0;
+    args.single_rank = 0;
+    for (uint32_t r = 0; r < ws.world; ++r) {
+        if (given.dst[r].num_tokens == 0) continue;
+        ++ranks_with_tokens;
+        args.single_rank = r + 1;
+    }
+    if (ranks_with_tokens != 1 || total_tokens > kOneRankMaxTokens) args.single_rank = 0;
+    if (args.single_rank != 0) args.single = given.dst[args.single_rank - 1];
     const uint32_t chunks = args.hidden_dim / V;
     const uint32_t slabs = (chunks + kSlabChunks - 1) / kSlabChunks;
     const uint64_t units = (uint64_t)total_tokens * slabs;
     const uint32_t blocks = (uint32_t)((units + kCombineWaves - 1) / kCombineWaves);
+#define A2A_LAUNCH_GATHER(KFIX, ONE)                                                                           \
+    hipExtLaunchKernelGGL((combine_gather_kernel<T, U, KFIX, ONE>), dim3(blocks), dim3(kCombineWaves * kWave), 0, \
+                          stream, timing.start, timing.stop, 0, args, ws)
     if (ws.topk == 8) {
-        hipExtLaunchKernelGGL((combine_gather_kernel<T, U, 8>), dim3(blocks), dim3(kCombineWaves * kWave), 0,
-                              stream, timing.start, timing.stop, 0, args, ws);
+        if (args.single_rank != 0) A2A_LAUNCH_GATHER(8, true); else A2A_LAUNCH_GATHER(8, false);
     } else {
-        hipExtLaunchKernelGGL((combine_gather_kernel<T, U, 0>), dim3(blocks), dim3(kCombineWaves * kWave), 0,
-                              stream, timing.start, timing.stop, 0, args, ws);
+        if (args.single_rank != 0) A2A_LAUNCH_GATHER(0, true); else A2A_LAUNCH_GATHER(0, false);
     }
+#undef A2A_LAUNCH_GATHER
     return hipGetLastError();
 }
 

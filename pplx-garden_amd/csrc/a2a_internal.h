@@ -108,8 +108,12 @@ struct PushArgs {
     uint32_t hidden_dim_scale;
     uint32_t topk_magic;                  // ceil(2^32 / K) (0 for K = 1): n / K = mulhi(n, magic) while n * K < 2^32
     uint32_t single_source;               // set by the launchers.  One-launch dispatches: g + 1 when source g alone has
-                                          // tokens and its index rows are dense, else 0.  Resolving pack: nonzero
-                                          // when one source alone has tokens.
+                                          // tokens and its index rows are dense, else 0.  Resolving pack: g + 1
+                                          // when source g alone has tokens.
+    PushSrc single;                       // a copy of src[single_source - 1]: at a fixed place in the argument block, so
+                                          // that a kernel reaches the token rows and index rows of the one source
+                                          // without first loading which source it is (a dependent trip at the head
+                                          // of every workgroup: 0.3 us of the 128-token step)
 };
 
 struct CombSrc {  // one per receiver rank: the expert outputs it holds
@@ -142,6 +146,11 @@ struct CombArgs {
     // receivers' expert_y at route_slot.  Null for the group call.
     const uint8_t *staged_base;
     uint64_t staged_stride;
+    // r + 1 when rank r alone has tokens to combine (0 otherwise), and a copy of dst[r] at a fixed place
+    // (set by the launcher; see PushArgs::single).
+    uint32_t single_rank;
+    uint32_t pad_;
+    CombDst single;
 };
 
 // Events a caller wants recorded when a kernel itself begins and ends (both
