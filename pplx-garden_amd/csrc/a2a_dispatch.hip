@@ -48,11 +48,13 @@ __device__ __forceinline__ void store_copy(u32x4 v, u32x4 *p) {
 // the same size, each with a token and LDS arrays of its own.  Every thread of
 // the workgroup must call (there is a barrier inside); a team without a token
 // passes `live` false.
-template <bool QUANT>
+// PRE: the thread's first piece of the row was asked for earlier (first_piece) and is passed in.
+template <bool QUANT, bool PRE = false>
 __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &src, uint32_t token, uint32_t K,
                                           uint64_t row_ptr, uint64_t scale_ptr, uint32_t scale_stride,
                                           float *s_scale, uint64_t *s_scale_ptr, uint32_t *s_scale_stride,
-                                          uint32_t team_tid, uint32_t team_threads, bool live) {
+                                          uint32_t team_tid, uint32_t team_threads, bool live,
+                                          u32x4 pre_a = u32x4{0, 0, 0, 0}, u32x4 pre_b = u32x4{0, 0, 0, 0}) {
     const uint32_t tid = team_tid;
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
@@ -65,7 +67,10 @@ __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &s
             const uint32_t c = base + lane;
             const bool active = c < num_chunks;
             u32x4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
-            if (active) {
+            if (PRE && base == wave * kWave) {
+                a = pre_a;
+                b = pre_b;
+            } else if (active) {
                 const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)c * 32);
                 a = __builtin_nontemporal_load(p);
                 b = __builtin_nontemporal_load(p + 1);
@@ -97,7 +102,7 @@ __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &s
     } else {
         const uint32_t num_chunks = live ? args.row_bytes / 16 : 0;
         for (uint32_t c = tid; c < num_chunks; c += team_threads) {
-            const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
+            const u32x4 v = PRE && c == tid ? pre_a : __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
             for (uint32_t k = 0; k < K; ++k) {
                 const uint64_t row = read_lane64(row_ptr, k);
                 if (row != 0) {
@@ -115,6 +120,27 @@ __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &s
                     if (sp != 0) reinterpret_cast<float *>(sp)[(size_t)j * ss] = s;
                 }
             }
+        }
+    }
+}
+
+// The piece of `token`'s row that thread `team_tid` of a team handles first in push_rows, asked for
+// ahead of time (zeros where push_rows would not load).
+template <bool QUANT>
+__device__ __forceinline__ void first_piece(const PushArgs &args, const PushSrc &src, uint32_t token,
+                                            uint32_t team_tid, bool live, u32x4 *a, u32x4 *b) {
+    const uint8_t *x_row = src.x + (size_t)token * src.x_stride;
+    *a = u32x4{0, 0, 0, 0};
+    *b = u32x4{0, 0, 0, 0};
+    if constexpr (QUANT) {
+        if (live && team_tid < args.hidden_dim / 16) {
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)team_tid * 32);
+            *a = __builtin_nontemporal_load(p);
+            *b = __builtin_nontemporal_load(p + 1);
+        }
+    } else {
+        if (live && team_tid < args.row_bytes / 16) {
+            *a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + team_tid);
         }
     }
 }
@@ -262,6 +288,36 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     const uint32_t total_entries = total_tokens * K;
     const bool receiver = blockIdx.x >= total_tokens;
 
+    // SINGLE: the entries are asked for first of all: they travel while the tables are cleared and
+    // the receivers' descriptors copied, instead of after them (one trip to memory less in a chain
+    // of five).
+    constexpr uint32_t kBatch = 8;
+    uint32_t early[kBatch];
+    uint32_t early_mine = 0xFFFFFFFFu;
+    if constexpr (SINGLE) {
+        const PushSrc &one = args.single;
+        const uint32_t entries = effective_tokens(one.bound_m, one.num_tokens) * K;
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t f = j * blockDim.x + tid;
+            early[j] = f < entries ? (uint32_t)one.indices[f] : 0xFFFFFFFFu;
+        }
+        if (!receiver && lane < K) early_mine = (uint32_t)one.indices[(size_t)blockIdx.x * one.indices_stride + lane];
+    }
+    // A receiver workgroup also asks for the order in which it lays out the sources, a token
+    // workgroup for its row (after the entries: what the chain waits for first goes first).  A step
+    // this small leaves the memory system idle, so the row is there when the routes are known; in
+    // the larger steps of the other dispatch kernels the same early request delays the entries.
+    OrderWords my_order = {};
+    if (receiver) my_order = load_order_words(ws, blockIdx.x - total_tokens);
+    u32x4 pre_a = {0, 0, 0, 0}, pre_b = {0, 0, 0, 0};
+    bool pre_live = false;
+    if constexpr (SINGLE) {
+        const PushSrc &one = args.single;
+        pre_live = !receiver && blockIdx.x < effective_tokens(one.bound_m, one.num_tokens);
+        first_piece<QUANT>(args, one, blockIdx.x, tid, pre_live, &pre_a, &pre_b);
+    }
+
     // Per token of the step (all sources, in grid order): where its K expert ids
     // are, with the source in the top byte; 0 for tokens past their source's
     // bound.  This is what the counting pass below looks up per entry.
@@ -318,7 +374,6 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     __syncthreads();
 
     // One pass over the entries of all sources, kBatch loads in flight per lane.
-    constexpr uint32_t kBatch = 8;
     const PushSrc &src = SINGLE ? args.single : args.src[my_g];
     const uint32_t rank = blockIdx.x - total_tokens;        // receivers only
     // flat index of my first entry (the one source of SINGLE is the first with tokens: it starts at 0)
@@ -337,7 +392,11 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
             expert[j] = 0xFFFFFFFFu;
             src_of[j] = SINGLE ? my_g : 0;
             if constexpr (SINGLE) {
-                if (f < flat_entries) expert[j] = (uint32_t)src.indices[f];
+                if (f0 == 0) {
+                    expert[j] = early[j];
+                } else if (f < flat_entries) {
+                    expert[j] = (uint32_t)src.indices[f];
+                }
             } else if (f < total_entries) {
                 const uint32_t flat_token = K > 1 ? __umulhi(f, args.topk_magic) : f;
                 const uint64_t ids = tok_ids[flat_token];
@@ -348,7 +407,11 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
             }
         }
         if (f0 == 0 && !receiver) {
-            if (lane < K) my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
+            if constexpr (SINGLE) {
+                my_expert = early_mine;
+            } else if (lane < K) {
+                my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
+            }
         }
 #pragma unroll
         for (uint32_t j = 0; j < kBatch; ++j) {
@@ -369,7 +432,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     __syncthreads();
 
     if (receiver) {
-        if (fin.recv_mask >> rank & 1) layout_from_totals(fin, ws, rank, cnt, scratch);
+        if (fin.recv_mask >> rank & 1) layout_from_totals(fin, ws, rank, cnt, scratch, my_order);
         return;
     }
 
@@ -459,8 +522,13 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
             ws.token_offset[(size_t)my_g * ws.max_tk + entry] = toff;
         }
     }
-    push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride,
-                     threadIdx.x, blockDim.x, true);
+    if constexpr (SINGLE) {
+        push_rows<QUANT, true>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr,
+                               s_scale_stride, threadIdx.x, blockDim.x, true, pre_a, pre_b);
+    } else {
+        push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride,
+                         threadIdx.x, blockDim.x, true);
+    }
 }
 
 // Routing pass and dispatch pack in ONE launch for steps of ONE source with
@@ -492,6 +560,7 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
     __shared__ uint64_t s_route_scale_ptr[kMaxGroupRoutes];
     __shared__ uint32_t s_route_scale_stride[kMaxGroupRoutes];
     __shared__ uint32_t s_route_expert[kMaxGroupRoutes];
+    __shared__ PushDst s_dst[kMaxWorld];                       // per receiver: its buffers
     __shared__ uint32_t scratch[kRouteWaves];
     __shared__ uint32_t s_carry;
 
@@ -509,6 +578,22 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
     // every token of mine is past the bound: nothing to send; the first workgroup stays (it publishes the totals)
     if (!receiver && blockIdx.x != 0 && first_token >= tokens) return;
 
+    // The first entries and the ids of my tokens' routes are asked for first of all: they travel
+    // while the tables are cleared and the receivers' descriptors copied to LDS.
+    constexpr uint32_t kBatch = 8;
+    uint32_t early[kBatch];
+#pragma unroll
+    for (uint32_t j = 0; j < kBatch; ++j) {
+        const uint32_t f = j * blockDim.x + tid;
+        early[j] = f < flat_entries ? (uint32_t)src.indices[f] : 0xFFFFFFFFu;
+    }
+    const uint32_t my_routes = per_group * K;    // one thread each
+    uint32_t my_expert = 0xFFFFFFFFu;
+    if (!receiver && tid < my_routes && my_first + tid < flat_entries) {
+        my_expert = (uint32_t)src.indices[my_first + tid];
+    }
+    if (!receiver && tid < ws.world) s_dst[tid] = args.dst[tid];
+
     uint32_t *cnt = s_tab;                 // [E] entries per expert; receivers: [G][Le]
     uint32_t *prior = s_tab + E;           // [E] entries per expert before my first token
     uint32_t *rows_before = prior + E;     // [E] padded rows of all experts before e
@@ -525,23 +610,16 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
             }
         }
     }
-    // The routes of my tokens: one thread each.
-    const uint32_t my_routes = per_group * K;
-    uint32_t my_expert = 0xFFFFFFFFu;
-    if (!receiver && tid < my_routes && my_first + tid < flat_entries) {
-        my_expert = (uint32_t)src.indices[my_first + tid];
-    }
     __syncthreads();
 
     // One pass over the entries of the step, kBatch loads in flight per lane.
-    constexpr uint32_t kBatch = 8;
     const uint32_t rank = blockIdx.x - token_groups;        // receivers only
     for (uint32_t f0 = 0; f0 < flat_entries; f0 += kBatch * blockDim.x) {
         uint32_t expert[kBatch];
 #pragma unroll
         for (uint32_t j = 0; j < kBatch; ++j) {
             const uint32_t f = f0 + j * blockDim.x + tid;
-            expert[j] = f < flat_entries ? (uint32_t)src.indices[f] : 0xFFFFFFFFu;
+            expert[j] = f0 == 0 ? early[j] : f < flat_entries ? (uint32_t)src.indices[f] : 0xFFFFFFFFu;
         }
 #pragma unroll
         for (uint32_t j = 0; j < kBatch; ++j) {
@@ -609,7 +687,7 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
             toff = prior[my_expert] + earlier;
             const uint32_t r = owner_of_expert(ws, my_expert);
             const uint32_t row = rows_before[my_expert] - rows_before[r * Le];
-            slot = resolve_copy(args.dst[r], ws, row + toff, true, &row_ptr, &scale_ptr, &scale_stride);
+            slot = resolve_copy(s_dst[r], ws, row + toff, true, &row_ptr, &scale_ptr, &scale_stride);
         } else {
             atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
         }

@@ -43,10 +43,25 @@ __device__ __forceinline__ uint32_t block_inclusive_scan(uint32_t v, uint32_t *s
     return before + incl;
 }
 
+// The order in which receiver `r` lays out the sources (kMaxWorld bytes, four to
+// a word), asked for in one go: eight independent loads, so that whoever needs the
+// order later does not walk it source by source, one dependent trip each.
+struct OrderWords {
+    uint32_t w[kMaxWorld / 4];
+};
+
+__device__ __forceinline__ OrderWords load_order_words(const Workspace &ws, uint32_t r) {
+    OrderWords o;
+#pragma unroll
+    for (uint32_t i = 0; i < (uint32_t)kMaxWorld / 4; ++i) o.w[i] = ws.order[r * (kMaxWorld / 4) + i];
+    return o;
+}
+
 // Rows of receiver `r` from `tot[g * Le + le]`, the number of copies source g
-// sends to local expert le.  Whole workgroup.
+// sends to local expert le.  `order` = load_order_words(ws, r), asked for by the
+// caller as early as it can.  Whole workgroup.
 __device__ inline void layout_from_totals(const FinalizeArgs &args, const Workspace &ws, uint32_t r,
-                                   const uint32_t *tot, uint32_t *scratch) {
+                                          const uint32_t *tot, uint32_t *scratch, const OrderWords &order) {
     const uint32_t N = ws.num_groups, E = ws.num_experts, Le = ws.experts_per_rank;
     const uint32_t tid = threadIdx.x;
     const uint32_t pad = ws.expert_padding;
@@ -66,12 +81,20 @@ __device__ inline void layout_from_totals(const FinalizeArgs &args, const Worksp
         // Sources in the order the reference's host worker visits them
         // (a2a_worker.rs:681-694); each gets a contiguous run of rows.
         uint32_t running = poff;
-        for (uint32_t i = 0; i < N; ++i) {
-            const uint32_t g = source_order_lookup(ws.order, r, i);
-            ws.slot_base[g * E + e] = running;
-            running += tot[g * Le + tid];
+#pragma unroll
+        for (uint32_t i = 0; i < (uint32_t)kMaxWorld; ++i) {
+            if (i < N) {
+                const uint32_t g = order.w[i / 4] >> (8 * (i % 4)) & 0xFFu;
+                ws.slot_base[g * E + e] = running;
+                running += tot[g * Le + tid];
+            }
         }
     }
+}
+
+__device__ inline void layout_from_totals(const FinalizeArgs &args, const Workspace &ws, uint32_t r,
+                                          const uint32_t *tot, uint32_t *scratch) {
+    layout_from_totals(args, ws, r, tot, scratch, load_order_words(ws, r));
 }
 
 }  // namespace a2a
