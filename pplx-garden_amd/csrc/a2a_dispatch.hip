@@ -281,6 +281,9 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     __shared__ uint32_t s_carry;
 
     const uint32_t tid = threadIdx.x;
+    // read once: used after LDS atomics and barriers, the compiler would fetch it again from the
+    // launch's implicit arguments each time, a trip to memory in the middle of the chain
+    const uint32_t nthreads = blockDim.x;
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
     const uint32_t G = ws.num_groups, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
@@ -295,35 +298,31 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     uint32_t early[kBatch];
     uint32_t early_mine = 0xFFFFFFFFu;
     if constexpr (SINGLE) {
+        // Without a branch around any of them (an address inside the array for every lane; which of the
+        // values count is decided where they are used), so that all of them are in flight together and
+        // each is waited for by itself.
         const PushSrc &one = args.single;
-        const uint32_t entries = effective_tokens(one.bound_m, one.num_tokens) * K;
+        const uint32_t entries = one.num_tokens * K;   // > 0: the one source has tokens
 #pragma unroll
         for (uint32_t j = 0; j < kBatch; ++j) {
-            const uint32_t f = j * blockDim.x + tid;
-            early[j] = f < entries ? (uint32_t)one.indices[f] : 0xFFFFFFFFu;
+            const uint32_t f = j * nthreads + tid;
+            early[j] = (uint32_t)one.indices[f < entries ? f : entries - 1];
         }
-        if (!receiver && lane < K) early_mine = (uint32_t)one.indices[(size_t)blockIdx.x * one.indices_stride + lane];
+        early_mine = (uint32_t)one.indices[(size_t)(receiver ? 0 : blockIdx.x) * one.indices_stride + (lane < K ? lane : 0)];
     }
     // A receiver workgroup also asks for the order in which it lays out the sources, a token
-    // workgroup for its row (after the entries: what the chain waits for first goes first).  A step
+    // workgroup, further down, for its row (what the chain waits for first goes first).  A step
     // this small leaves the memory system idle, so the row is there when the routes are known; in
     // the larger steps of the other dispatch kernels the same early request delays the entries.
     OrderWords my_order = {};
     if (receiver) my_order = load_order_words(ws, blockIdx.x - total_tokens);
-    u32x4 pre_a = {0, 0, 0, 0}, pre_b = {0, 0, 0, 0};
-    bool pre_live = false;
-    if constexpr (SINGLE) {
-        const PushSrc &one = args.single;
-        pre_live = !receiver && blockIdx.x < effective_tokens(one.bound_m, one.num_tokens);
-        first_piece<QUANT>(args, one, blockIdx.x, tid, pre_live, &pre_a, &pre_b);
-    }
 
     // Per token of the step (all sources, in grid order): where its K expert ids
     // are, with the source in the top byte; 0 for tokens past their source's
     // bound.  This is what the counting pass below looks up per entry.
     const uint32_t table_words = ((G + 3) * E + 1) & ~1u;
     uint64_t *tok_ids = reinterpret_cast<uint64_t *>(s_dyn + table_words);
-    for (uint32_t ft = tid; !SINGLE && ft < total_tokens; ft += blockDim.x) {
+    for (uint32_t ft = tid; !SINGLE && ft < total_tokens; ft += nthreads) {
         // token_start is non-decreasing and equals the total from G on, so the
         // fixed trip count is safe and lets the loads go out together
         uint32_t g = 0, start = 0;
@@ -347,9 +346,9 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     uint32_t *copies_before = rows_before + E;              // [E] copies of the sources laid out before mine
     const uint32_t table = receiver ? G * Le : G * E + E;
     if (SINGLE && !receiver) {
-        for (uint32_t i = tid; i < 2 * E; i += blockDim.x) s_dyn[i] = 0;   // cnt and prior
+        for (uint32_t i = tid; i < 2 * E; i += nthreads) s_dyn[i] = 0;   // cnt and prior
     } else {
-        for (uint32_t i = tid; i < table; i += blockDim.x) s_dyn[i] = 0;
+        for (uint32_t i = tid; i < table; i += nthreads) s_dyn[i] = 0;
     }
     uint32_t my_g = 0, token = 0;
     if constexpr (SINGLE) {
@@ -359,13 +358,30 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
         while (my_g + 1 < G && blockIdx.x >= args.token_start[my_g + 1]) ++my_g;
         token = blockIdx.x - args.token_start[my_g];
     }
-    if (!receiver && tid < ws.world) s_dst[tid] = args.dst[tid];
+    // The receivers' descriptors are asked for here and written to LDS after the counting: written
+    // here, the wait for them would also wait for the entries and the row asked for above.
+    // (field by field and without a branch, so that they stay in registers and nothing waits for them
+    // before their use)
+    const PushDst &dst_of_tid = args.dst[tid < ws.world ? tid : 0];
+    uint8_t *const my_out_x = dst_of_tid.out_x;
+    float *const my_out_scale = dst_of_tid.out_scale;
+    const uint64_t my_out_stride = dst_of_tid.out_stride;
+    const uint32_t my_os_elem = dst_of_tid.os_stride_elem, my_os_token = dst_of_tid.os_stride_token;
+    const uint32_t my_out_rows = dst_of_tid.out_rows;
+    // The row comes last: the chain needs it last, and what is asked for later is waited for later.
+    u32x4 pre_a = {0, 0, 0, 0}, pre_b = {0, 0, 0, 0};
+    bool pre_live = false;
+    if constexpr (SINGLE) {
+        const PushSrc &one = args.single;
+        pre_live = !receiver && blockIdx.x < effective_tokens(one.bound_m, one.num_tokens);
+        first_piece<QUANT>(args, one, blockIdx.x, tid, pre_live, &pre_a, &pre_b);
+    }
     // Sources without tokens have no workgroup of their own: the first receiver
     // workgroup (the first workgroup, if nobody receives) clears their tables.
     if (blockIdx.x == (fin.recv_mask != 0 ? total_tokens : 0)) {
         for (uint32_t g = 0; g < G; ++g) {
             if (args.src[g].num_tokens != 0) continue;
-            for (uint32_t e = tid; e < E; e += blockDim.x) {
+            for (uint32_t e = tid; e < E; e += nthreads) {
                 ws.num_routed[g * E + e] = 0;
                 ws.expert_offsets[g * E + e] = 0;
             }
@@ -384,35 +400,8 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     const uint32_t order_words = receiver || SINGLE ? 0 : ws.world * (kMaxWorld / 4);
     const uint32_t order_word = tid < order_words ? ws.order[tid] : 0;
     const uint32_t flat_entries = SINGLE ? effective_tokens(src.bound_m, src.num_tokens) * K : 0;
-    for (uint32_t f0 = 0; f0 < total_entries || f0 == 0; f0 += kBatch * blockDim.x) {
-        uint32_t expert[kBatch], src_of[kBatch];
-#pragma unroll
-        for (uint32_t j = 0; j < kBatch; ++j) {
-            const uint32_t f = f0 + j * blockDim.x + tid;
-            expert[j] = 0xFFFFFFFFu;
-            src_of[j] = SINGLE ? my_g : 0;
-            if constexpr (SINGLE) {
-                if (f0 == 0) {
-                    expert[j] = early[j];
-                } else if (f < flat_entries) {
-                    expert[j] = (uint32_t)src.indices[f];
-                }
-            } else if (f < total_entries) {
-                const uint32_t flat_token = K > 1 ? __umulhi(f, args.topk_magic) : f;
-                const uint64_t ids = tok_ids[flat_token];
-                src_of[j] = (uint32_t)(ids >> 56);
-                if (ids != 0) {
-                    expert[j] = (uint32_t) reinterpret_cast<const int32_t *>(ids & 0x00FFFFFFFFFFFFFFull)[f - flat_token * K];
-                }
-            }
-        }
-        if (f0 == 0 && !receiver) {
-            if constexpr (SINGLE) {
-                my_expert = early_mine;
-            } else if (lane < K) {
-                my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
-            }
-        }
+    // counts one batch of entries: entry j of the batch is f0 + j * nthreads + tid
+    auto count_batch = [&](const uint32_t (&expert)[kBatch], const uint32_t (&src_of)[kBatch], uint32_t f0) {
 #pragma unroll
         for (uint32_t j = 0; j < kBatch; ++j) {
             const uint32_t x = expert[j];
@@ -422,13 +411,55 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
                 if (le < Le) atomicAdd(&cnt[src_of[j] * Le + le], 1u);
             } else {
                 atomicAdd(&cnt[(SINGLE ? 0 : src_of[j]) * E + x], 1u);
-                const uint32_t f = f0 + j * blockDim.x + tid;
+                const uint32_t f = f0 + j * nthreads + tid;
                 if (src_of[j] == my_g && f < my_first) atomicAdd(&prior[x], 1u);
             }
         }
+    };
+    uint32_t f_begin = 0;
+    if constexpr (SINGLE) {
+        // The first batch was asked for at the head.  It is counted here in straight-line code, outside
+        // the loop: each of its values is then waited for by itself, and the row and the descriptors
+        // asked for after them stay in flight meanwhile.
+        uint32_t expert[kBatch], src_of[kBatch];
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t f = j * nthreads + tid;
+            expert[j] = f < flat_entries ? early[j] : 0xFFFFFFFFu;
+            src_of[j] = my_g;
+        }
+        if (!receiver && lane < K) my_expert = early_mine;
+        count_batch(expert, src_of, 0);
+        f_begin = kBatch * nthreads;
+    }
+    for (uint32_t f0 = f_begin; f0 < total_entries || (!SINGLE && f0 == 0); f0 += kBatch * nthreads) {
+        uint32_t expert[kBatch], src_of[kBatch];
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t f = f0 + j * nthreads + tid;
+            expert[j] = 0xFFFFFFFFu;
+            src_of[j] = SINGLE ? my_g : 0;
+            if constexpr (SINGLE) {
+                if (f < flat_entries) expert[j] = (uint32_t)src.indices[f];
+            } else if (f < total_entries) {
+                const uint32_t flat_token = K > 1 ? __umulhi(f, args.topk_magic) : f;
+                const uint64_t ids = tok_ids[flat_token];
+                src_of[j] = (uint32_t)(ids >> 56);
+                if (ids != 0) {
+                    expert[j] = (uint32_t) reinterpret_cast<const int32_t *>(ids & 0x00FFFFFFFFFFFFFFull)[f - flat_token * K];
+                }
+            }
+        }
+        if (!SINGLE && f0 == 0 && !receiver && lane < K) {
+            my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
+        }
+        count_batch(expert, src_of, f0);
+    }
+    if (!receiver && tid < ws.world) {
+        s_dst[tid] = PushDst{my_out_x, my_out_scale, my_out_stride, my_os_elem, my_os_token, my_out_rows, 0};
     }
     if (tid < order_words) s_order[tid] = order_word;
-    for (uint32_t i = tid + blockDim.x; i < order_words; i += blockDim.x) s_order[i] = ws.order[i];
+    for (uint32_t i = tid + nthreads; i < order_words; i += nthreads) s_order[i] = ws.order[i];
     __syncthreads();
 
     if (receiver) {
@@ -441,7 +472,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     // the scan at the first expert of a receiver is the expert's first row there)
     // and the copies of the sources its receiver lays out before mine.
     uint32_t carry = 0;
-    for (uint32_t e0 = 0; e0 < E; e0 += blockDim.x) {
+    for (uint32_t e0 = 0; e0 < E; e0 += nthreads) {
         const uint32_t e = e0 + tid;
         uint32_t total = 0, before = 0;
         if (SINGLE) {
@@ -473,8 +504,8 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
             rows_before[e] = incl - padded;
             copies_before[e] = before;
         }
-        if (e0 + blockDim.x < E) {   // uniform: another round follows
-            if (tid == blockDim.x - 1) s_carry = incl;
+        if (e0 + nthreads < E) {   // uniform: another round follows
+            if (tid == nthreads - 1) s_carry = incl;
             __syncthreads();
             carry = s_carry;
         }
@@ -482,7 +513,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     __syncthreads();
 
     // The first token's workgroup publishes its source's totals (last wavefront).
-    if (token == 0 && wave == blockDim.x / kWave - 1) {
+    if (token == 0 && wave == nthreads / kWave - 1) {
         uint32_t run = 0;
         for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
             const uint32_t e = e0 + lane;
@@ -524,10 +555,10 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     }
     if constexpr (SINGLE) {
         push_rows<QUANT, true>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr,
-                               s_scale_stride, threadIdx.x, blockDim.x, true, pre_a, pre_b);
+                               s_scale_stride, threadIdx.x, nthreads, true, pre_a, pre_b);
     } else {
         push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale, s_scale_ptr, s_scale_stride,
-                         threadIdx.x, blockDim.x, true);
+                         threadIdx.x, nthreads, true);
     }
 }
 
