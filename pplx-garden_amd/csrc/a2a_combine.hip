@@ -158,6 +158,30 @@ template <typename T, typename U, int KFIX, bool ONE_RANK>
 __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(const CombArgs args,
                                                                               const Workspace ws) {
     constexpr int V = vec_elems<T>();
+    if constexpr (ONE_RANK) {
+        // everything the head of a wavefront needs from the argument block, asked for in one go
+        A2A_PIN(args.token_start[kMaxWorld]);
+        A2A_PIN(args.single_rank);
+        A2A_PIN(args.hidden_dim);
+        A2A_PIN(args.accumulate);
+        A2A_PIN(args.staged_base);
+        A2A_PIN(args.single.out);
+        A2A_PIN(args.single.indices);
+        A2A_PIN(args.single.weights);
+        A2A_PIN(args.single.bound_m);
+        A2A_PIN(args.single.out_stride);
+        A2A_PIN(args.single.indices_stride);
+        A2A_PIN(args.single.weights_stride);
+        A2A_PIN(args.single.num_tokens);
+        A2A_PIN(ws.world);
+        A2A_PIN(ws.dp_size);
+        A2A_PIN(ws.num_experts);
+        A2A_PIN(ws.experts_per_rank);
+        A2A_PIN(ws.le_magic);
+        A2A_PIN(ws.max_tk);
+        A2A_PIN(ws.route_slot);
+        A2A_PIN(ws.err);
+    }
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
     const uint32_t E = ws.num_experts;

@@ -270,6 +270,36 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
 template <bool QUANT, bool SINGLE>
 __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs args, const FinalizeArgs fin,
                                                               const Workspace ws) {
+    if constexpr (SINGLE) {
+        // everything the head of a workgroup needs from the argument block, asked for in one go; the
+        // same in the kernel of a larger single source gained nothing and is left out there
+        A2A_PIN(args.token_start[kMaxWorld]);
+        A2A_PIN(args.single_source);
+        A2A_PIN(args.hidden_dim);
+        A2A_PIN(args.hidden_dim_scale);
+        A2A_PIN(args.row_bytes);
+        A2A_PIN(args.single.x);
+        A2A_PIN(args.single.indices);
+        A2A_PIN(args.single.bound_m);
+        A2A_PIN(args.single.x_stride);
+        A2A_PIN(args.single.indices_stride);
+        A2A_PIN(args.single.num_tokens);
+        A2A_PIN(fin.recv_mask);
+        A2A_PIN(ws.world);
+        A2A_PIN(ws.num_groups);
+        A2A_PIN(ws.num_experts);
+        A2A_PIN(ws.topk);
+        A2A_PIN(ws.experts_per_rank);
+        A2A_PIN(ws.le_magic);
+        A2A_PIN(ws.expert_padding);
+        A2A_PIN(ws.max_tk);
+        A2A_PIN(ws.order);
+        A2A_PIN(ws.num_routed);
+        A2A_PIN(ws.expert_offsets);
+        A2A_PIN(ws.route_slot);
+        A2A_PIN(ws.token_offset);
+        A2A_PIN(ws.err);
+    }
     extern __shared__ uint64_t s_dyn64[];
     uint32_t *s_dyn = reinterpret_cast<uint32_t *>(s_dyn64);
     __shared__ float s_scale[QUANT ? kMaxLdsScales : 1];
