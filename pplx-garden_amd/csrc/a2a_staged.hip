@@ -106,7 +106,32 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
     extern __shared__ uint32_t s_send[];
     __shared__ uint32_t scratch[kRouteWaves];
     __shared__ uint32_t s_carry;
+    // everything the head of a workgroup takes from the argument block, asked for in one go
+    A2A_PIN(args.src.x);
+    A2A_PIN(args.src.indices);
+    A2A_PIN(args.src.bound_m);
+    A2A_PIN(args.src.x_stride);
+    A2A_PIN(args.src.indices_stride);
+    A2A_PIN(args.src.num_tokens);
+    A2A_PIN(args.rank);
+    A2A_PIN(args.hidden_dim);
+    A2A_PIN(args.row_bytes);
+    A2A_PIN(args.topk_magic);
+    A2A_PIN(ws.num_experts);
+    A2A_PIN(ws.topk);
+    A2A_PIN(ws.dp_size);
+    A2A_PIN(ws.max_tk);
+    A2A_PIN(ws.num_routed);
+    A2A_PIN(ws.expert_offsets);
+    A2A_PIN(ws.token_offset);
+    A2A_PIN(ws.err);
+    A2A_PIN(st.send_buf);
+    A2A_PIN(st.pos_token);
+    A2A_PIN(st.disp_stride);
+    A2A_PIN(st.payload_bytes);
+    A2A_PIN(st.max_tokens);
     const uint32_t tid = threadIdx.x;
+    const uint32_t nthreads = blockDim.x;   // read once: used after LDS atomics it is fetched again every time
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
     const uint32_t E = ws.num_experts;
@@ -121,37 +146,46 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
     uint32_t *prior = cnt + E;       // [E] those of the tokens before mine
     uint32_t *excl = prior + E;      // [E] exclusive scan of cnt
 
-    for (uint32_t i = tid; i < 2 * E; i += blockDim.x) s_send[i] = 0;
-    __syncthreads();
-
-    uint32_t my_expert = 0xFFFFFFFFu;
-    for (uint32_t f0 = 0; f0 < entries || f0 == 0; f0 += 8 * blockDim.x) {
-        uint32_t expert[8];
+    // The first batch of entries is asked for before the tables are cleared and counted in
+    // straight-line code, each entry waited for by itself.
+    auto load_batch = [&](uint32_t f0, uint32_t (&expert)[8]) {
 #pragma unroll
         for (uint32_t j = 0; j < 8; ++j) {
-            const uint32_t f = f0 + j * blockDim.x + tid;
+            const uint32_t f = f0 + j * nthreads + tid;
             expert[j] = 0xFFFFFFFFu;
             if (f < entries) {
                 const uint32_t t = K > 1 ? __umulhi(f, args.topk_magic) : f;
                 expert[j] = (uint32_t)src.indices[(size_t)t * src.indices_stride + (f - t * K)];
             }
         }
-        if (f0 == 0 && lane < K) {
-            my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
-        }
+    };
+    auto count_batch = [&](uint32_t f0, const uint32_t (&expert)[8]) {
 #pragma unroll
         for (uint32_t j = 0; j < 8; ++j) {
             const uint32_t x = expert[j];
             if (x >= E) continue;
             atomicAdd(&cnt[x], 1u);
-            if (f0 + j * blockDim.x + tid < my_first) atomicAdd(&prior[x], 1u);
+            if (f0 + j * nthreads + tid < my_first) atomicAdd(&prior[x], 1u);
         }
+    };
+    uint32_t first_batch[8];
+    load_batch(0, first_batch);
+    uint32_t my_expert = 0xFFFFFFFFu;
+    if (lane < K) my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
+
+    for (uint32_t i = tid; i < 2 * E; i += nthreads) s_send[i] = 0;
+    __syncthreads();
+    count_batch(0, first_batch);
+    for (uint32_t f0 = 8 * nthreads; f0 < entries; f0 += 8 * nthreads) {
+        uint32_t expert[8];
+        load_batch(f0, expert);
+        count_batch(f0, expert);
     }
     __syncthreads();
 
     // Scan over the experts (a2a_dispatch_send.cu:236-242); token 0 publishes.
     uint32_t carry = 0;
-    for (uint32_t e0 = 0; e0 < E; e0 += blockDim.x) {
+    for (uint32_t e0 = 0; e0 < E; e0 += nthreads) {
         const uint32_t e = e0 + tid;
         const uint32_t c = e < E ? cnt[e] : 0;
         const uint32_t incl = carry + block_inclusive_scan(c, scratch);
@@ -162,8 +196,8 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
                 ws.expert_offsets[g * E + e] = incl;
             }
         }
-        if (e0 + blockDim.x < E) {   // uniform: another round follows
-            if (tid == blockDim.x - 1) s_carry = incl;
+        if (e0 + nthreads < E) {   // uniform: another round follows
+            if (tid == nthreads - 1) s_carry = incl;
             __syncthreads();
             carry = s_carry;
         }
@@ -190,7 +224,7 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
             ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
         }
     }
-    stage_row<QUANT>(args, st, g, token, blockDim.x);
+    stage_row<QUANT>(args, st, g, token, nthreads);
 }
 
 // The send of a large step, after a routing launch that left the chunk counts,
@@ -525,6 +559,20 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(1024) void combine_send_kernel(const CombineSendArgs args,
                                                             const Workspace ws, const Staging st) {
+    // everything a wavefront takes from the argument block, asked for in one go
+    A2A_PIN(args.y);
+    A2A_PIN(args.y_stride);
+    A2A_PIN(args.y_rows);
+    A2A_PIN(args.row_bytes);
+    A2A_PIN(args.team_waves);
+    A2A_PIN(ws.dp_size);
+    A2A_PIN(ws.max_tk);
+    A2A_PIN(st.comb_buf);
+    A2A_PIN(st.padded_index);
+    A2A_PIN(st.source_rank);
+    A2A_PIN(st.source_position);
+    A2A_PIN(st.comb_stride);
+    A2A_PIN(st.max_recv);
     const uint32_t r = args.rank;
     uint32_t total = st.num_recv[2 * r];
     if (total > st.max_recv) total = st.max_recv;
