@@ -355,7 +355,9 @@ __device__ __forceinline__ void copy_row_by_team(const u32x4 *src, u32x4 *dst, u
 // worker does, a2a_worker.rs:577-606,621-694): rows per expert, padded first
 // row of every expert, first row of every (source, expert) run inside it, and
 // the order in which the runs ARRIVE (sources in the worker's order, experts
-// inside a source).  Workgroup 0 publishes those tables.  Then the workgroups
+// inside a source).  Two wavefronts of a workgroup do that, each by itself;
+// a workgroup that has no row leaves before.  Workgroup 0 publishes those
+// tables.  Then the workgroups
 // share the received rows between them, one team of wavefronts per row: its metadata (padded_index,
 // source_rank, source position: a2a_worker.rs:636-671) is written and payload
 // and scales are copied from the sender's staged token
@@ -366,8 +368,6 @@ __device__ __forceinline__ void copy_row_by_team(const u32x4 *src, u32x4 *dst, u
 __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs args, const Workspace ws,
                                                           const Staging st) {
     extern __shared__ uint32_t s_recv[];
-    __shared__ uint32_t scratch[kRouteWaves];
-    __shared__ uint32_t s_carry;
     __shared__ uint8_t s_order[kMaxWorld];
     const uint32_t G = ws.num_groups, E = ws.num_experts, Le = ws.experts_per_rank;
     const uint32_t r = args.rank;
@@ -375,6 +375,8 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     const uint32_t n_local = first >= E ? 0 : (E - first < Le ? E - first : Le);
     const uint32_t items = G * Le;
     const uint32_t tid = threadIdx.x;
+    const uint32_t nthreads = blockDim.x;
+    const uint32_t lane = tid & (kWave - 1);
     const bool publish = blockIdx.x == 0;
     uint32_t *tot = s_recv;              // [g][le]  copies source g sends to local expert le
     uint32_t *excl = tot + items;        // [g][le]  position of the run in the sender's expert-sorted order
@@ -386,9 +388,9 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
 
     // The order in which this receiver lays out its sources (one byte per source, from the table the
     // context computed once) travels with the counts and is read from LDS from then on: looked up in
-    // memory where it is used, it put a dependent trip into both scans and one in front of every row.
+    // memory where it is used, it put a dependent trip into the layout and one in front of every row.
     if (tid < G) s_order[tid] = (uint8_t)source_order_lookup(ws.order, r, tid);
-    for (uint32_t w = tid; w < items; w += blockDim.x) {
+    for (uint32_t w = tid; w < items; w += nthreads) {
         const uint32_t g = Le > 1 ? __umulhi(w, ws.le_magic) : w;
         const uint32_t le = w - g * Le;
         const uint32_t e = first + le;
@@ -397,84 +399,106 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
         excl[w] = live && e > 0 ? ws.expert_offsets[g * E + e - 1] : 0;
     }
     __syncthreads();
-    // Per source: where its rows for this receiver begin in its own send order (dst_group_offset,
-    // a2a_worker.rs:571-575) and how many rows the lower-numbered sources send here
-    // (src_group_offset, a2a_worker.rs:582-590: numeric order, not the order of arrival).
-    // (one wavefront per source adds up its row of `tot` here; the short sum over the sources below
-    // it follows after the barriers of the next scan)
-    for (uint32_t g = tid / kWave; g < G; g += blockDim.x / kWave) {
-        uint32_t part = 0;
-        for (uint32_t le = tid & (kWave - 1); le < Le; le += kWave) part += tot[g * Le + le];
-        for (int off = kWave / 2; off > 0; off >>= 1) part += __shfl_down(part, off);
-        if ((tid & (kWave - 1)) == 0) {
-            grp_dst[g] = excl[g * Le];
-            grp_cnt[g] = part;
+
+    // Rows this receiver gets from source g (lane g; there are at most kMaxWorld <= 64 sources): the
+    // sender's scan over its experts gives them without a sum.  Every wavefront adds them up by itself,
+    // and a workgroup whose first row lies beyond the rows received leaves here: the host sizes the
+    // grid for an upper bound, a receiver typically gets 1/N of it, and the layout below is the
+    // expensive part of a workgroup without rows.
+    uint32_t from_source = 0;
+    if (lane < G && n_local != 0) {
+        const uint32_t last = lane * Le + n_local - 1;
+        from_source = excl[last] + tot[last] - excl[lane * Le];
+    }
+    const uint32_t from_lower = wave_inclusive_scan(from_source, lane);   // inclusive over the sources
+    const uint32_t rows = (uint32_t)__builtin_amdgcn_readlane((int)from_lower, kWave - 1);
+    const uint32_t team_threads = args.team_waves * kWave;
+    if (!publish && blockIdx.x * (nthreads / team_threads) >= rows) return;   // uniform
+
+    // The layout is the work of two wavefronts, each by itself (scans on the DPP path, no barrier
+    // inside); the others wait for them.  Done by every wavefront of every workgroup, with workgroup
+    // scans, it was most of the kernel's instructions.
+    const uint32_t wave = tid / kWave;
+    if (wave == 0) {
+        // Per source: where its rows for this receiver begin in its own send order (dst_group_offset,
+        // a2a_worker.rs:571-575) and how many rows the lower-numbered sources send here
+        // (src_group_offset, a2a_worker.rs:582-590: numeric order, not the order of arrival).
+        if (lane < G) {
+            grp_dst[lane] = excl[lane * Le];
+            grp_cnt[lane] = from_source;
+            grp_src[lane] = from_lower - from_source;
+        }
+
+        // Rows per expert, padded offsets, first row of every run.
+        const uint32_t visited = lane < G ? s_order[lane] : 0;   // lane i: the i-th source in the order of the layout
+        const uint32_t pad = ws.expert_padding;
+        uint32_t carry = 0;
+        for (uint32_t l0 = 0; l0 < Le; l0 += kWave) {
+            const uint32_t le = l0 + lane;
+            const bool mine = le < n_local;
+            uint32_t tpe = 0;
+            if (mine) {
+                for (uint32_t g = 0; g < G; ++g) tpe += tot[g * Le + le];
+            }
+            const uint32_t padded = (tpe + pad - 1) / pad * pad;
+            const uint32_t scan = wave_inclusive_scan(mine ? padded : 0, lane);
+            if (mine) {
+                const uint32_t poff = carry + scan - padded;
+                const uint32_t e = first + le;
+                uint32_t running = poff;
+                uint32_t g = (uint32_t)__builtin_amdgcn_readlane((int)visited, 0);
+                uint32_t next = tot[g * Le + le];
+                for (uint32_t i = 0; i < G; ++i) {
+                    // the count of the source after this one is asked for before this one's is used
+                    const uint32_t count = next;
+                    const uint32_t g_next = (uint32_t)__builtin_amdgcn_readlane((int)visited, (int)(i + 1 < G ? i + 1 : i));
+                    next = tot[g_next * Le + le];
+                    run_row[i * Le + le] = running;
+                    if (publish) ws.slot_base[g * E + e] = running;
+                    running += count;
+                    g = g_next;
+                }
+                if (publish) {
+                    ws.tokens_per_expert[e] = tpe;
+                    ws.padded_offset[e] = poff;
+                    if (args.out_num_tokens != nullptr) args.out_num_tokens[le] = (int32_t)tpe;
+                    if (poff + tpe > args.dst.out_rows) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+                }
+            }
+            carry += (uint32_t)__builtin_amdgcn_readlane((int)scan, kWave - 1);
         }
     }
-
-    // Rows per expert, padded offsets, first row of every run.
-    const uint32_t pad = ws.expert_padding;
-    uint32_t carry = 0;
-    for (uint32_t l0 = 0; l0 < Le; l0 += blockDim.x) {
-        const uint32_t le = l0 + tid;
-        const bool mine = le < n_local;
-        uint32_t tpe = 0;
-        if (mine) {
-            for (uint32_t g = 0; g < G; ++g) tpe += tot[g * Le + le];
-        }
-        const uint32_t padded = (tpe + pad - 1) / pad * pad;
-        const uint32_t incl = carry + block_inclusive_scan(mine ? padded : 0, scratch);
-        if (mine) {
-            const uint32_t poff = incl - padded;
-            const uint32_t e = first + le;
-            uint32_t running = poff;
-            for (uint32_t i = 0; i < G; ++i) {
+    if (wave == (nthreads > kWave ? 1u : 0u)) {
+        // Arrival order: sources as the worker visits them, local experts inside a source.  Lane i has
+        // the rows that arrive before those of the i-th source visited; inside a source the sender's
+        // scan over its experts says how many rows precede those of a local expert.  No sum, no scan
+        // over the runs.
+        const uint32_t visited = lane < G ? s_order[lane] : 0;
+        const uint32_t theirs = (uint32_t)__shfl((int)from_source, (int)visited);   // every lane takes part
+        const uint32_t arrive = lane < G ? theirs : 0;
+        const uint32_t before = wave_inclusive_scan(arrive, lane) - arrive;
+        for (uint32_t b = 0; b < items; b += kWave) {
+            const uint32_t s = b + lane;
+            const uint32_t i = s < items ? (Le > 1 ? __umulhi(s, ws.le_magic) : s) : 0;
+            const uint32_t base = (uint32_t)__shfl((int)before, (int)i);
+            const uint32_t count = (uint32_t)__shfl((int)arrive, (int)i);
+            if (s < items) {
+                const uint32_t le = s - i * Le;
                 const uint32_t g = s_order[i];
-                run_row[i * Le + le] = running;
-                if (publish) ws.slot_base[g * E + e] = running;
-                running += tot[g * Le + le];
+                seg[s] = base + (le < n_local ? excl[g * Le + le] - excl[g * Le] : count);
             }
+        }
+        if (lane == 0) {
+            seg[items] = rows;
             if (publish) {
-                ws.tokens_per_expert[e] = tpe;
-                ws.padded_offset[e] = poff;
-                if (args.out_num_tokens != nullptr) args.out_num_tokens[le] = (int32_t)tpe;
-                if (poff + tpe > args.dst.out_rows) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+                if (rows > st.max_recv) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+                st.num_recv[2 * r] = rows;
             }
         }
-        if (l0 + blockDim.x < Le) {   // uniform: another round follows
-            if (tid == blockDim.x - 1) s_carry = incl;
-            __syncthreads();
-            carry = s_carry;
-        }
     }
-
-    if (tid < G) {   // grp_cnt was written before the barriers of the scan above
-        uint32_t rows_below = 0;
-        for (uint32_t g = 0; g < tid; ++g) rows_below += grp_cnt[g];
-        grp_src[tid] = rows_below;
-    }
-
-    // Arrival order: sources as the worker visits them, local experts inside a source.
-    carry = 0;
-    for (uint32_t b = 0; b < items; b += blockDim.x) {
-        const uint32_t s = b + tid;
-        uint32_t cnt = 0;
-        if (s < items) {
-            const uint32_t i = Le > 1 ? __umulhi(s, ws.le_magic) : s;
-            cnt = tot[s_order[i] * Le + (s - i * Le)];
-        }
-        const uint32_t incl = carry + block_inclusive_scan(cnt, scratch);
-        if (s < items) seg[s] = incl - cnt;
-        if (tid == blockDim.x - 1) s_carry = incl;
-        __syncthreads();
-        carry = s_carry;
-    }
-    const uint32_t total = carry;
-    if (tid == 0) seg[items] = total;
     __syncthreads();
+    const uint32_t total = rows;
     if (publish && tid == 0) {
-        if (total > st.max_recv) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
-        st.num_recv[2 * r] = total;
         // rows that come from other nodes (num_efa_tokens, a2a_worker.rs:681-687)
         const uint32_t remote_segs = (ws.world / ws.node_size - 1) * (ws.node_size / ws.dp_size) * Le;
         st.num_recv[2 * r + 1] = remote_segs < items ? seg[remote_segs] : total;
@@ -485,9 +509,8 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     // time.  Every wavefront of a team finds the row's run by itself.
     const PushDst &dst = args.dst;
     const uint32_t num_chunks = args.row_bytes / 16;
-    const uint32_t lane = tid & (kWave - 1);
-    const uint32_t team = args.team_waves * kWave;
-    const uint32_t teams = blockDim.x / team;
+    const uint32_t team = team_threads;
+    const uint32_t teams = nthreads / team;
     const uint32_t member = tid % team;
     for (uint32_t row = blockIdx.x * teams + tid / team; row < total; row += gridDim.x * teams) {
         // the run this arrival belongs to: the one non-empty run with seg[s] <= row < seg[s + 1]
