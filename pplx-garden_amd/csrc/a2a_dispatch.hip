@@ -641,7 +641,7 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
 
     // The first entries and the ids of my tokens' routes are asked for first of all: they travel
     // while the tables are cleared and the receivers' descriptors copied to LDS.
-    constexpr uint32_t kBatch = 8;
+    constexpr uint32_t kBatch = 10;   // 8192 entries over 896 threads in one batch: one trip to memory, not two
     uint32_t early[kBatch];
 #pragma unroll
     for (uint32_t j = 0; j < kBatch; ++j) {
