@@ -8,6 +8,13 @@ namespace a2a {
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
+// A barrier for data that wavefronts of a workgroup hand to each other through LDS: it waits for this
+// wavefront's LDS operations only.  Loads from memory that were asked for earlier stay in flight across
+// it (in front of its own barrier the compiler may wait for every outstanding access to memory).
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 template <int CTRL>
 __device__ __forceinline__ float dpp_move(float v) {
     return __int_as_float(

@@ -40,9 +40,10 @@ __device__ __forceinline__ void store_copy(u32x4 v, u32x4 *p) {
 
 // Moves the row of `token` to its copies.  Lanes 0..K-1 of EVERY wavefront hold
 // the row pointer, scale pointer and scale stride of route k (0 = no copy).
-// The row is loaded here, AFTER the routes are known: asking for it earlier to
-// hide its latency was measured slower at every size (4 us on the 4096-token
-// pack, 0.4 us on the 128-token one).
+// The row is loaded here, AFTER the routes are known, unless the caller passes
+// its first piece (PRE): in the bandwidth-bound pack of a large step asking for
+// it earlier was 4 us slower; the latency-bound one-launch kernels ask for it at
+// their head.
 // The work is done by a TEAM of `team_threads` threads (a multiple of 64), in
 // which the caller is thread `team_tid`; a workgroup is one team or several of
 // the same size, each with a token and LDS arrays of its own.  Every thread of
@@ -91,7 +92,7 @@ __device__ __forceinline__ void push_rows(const PushArgs &args, const PushSrc &s
             s_scale_ptr[lane] = live ? scale_ptr : 0;
             s_scale_stride[lane] = scale_stride;
         }
-        __syncthreads();
+        lds_barrier();   // (the row's stores and whatever the caller has asked for stay in flight)
         const uint32_t Hl = Hs < (uint32_t)kMaxLdsScales ? Hs : (uint32_t)kMaxLdsScales;
         for (uint32_t i = tid; i < K * Hl; i += team_threads) {
             const uint32_t k = i / Hl;
@@ -626,6 +627,7 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
     __shared__ uint32_t s_carry;
 
     const uint32_t tid = threadIdx.x;
+    const uint32_t nthreads = blockDim.x;
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t G = ws.num_groups, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
     const uint32_t my_g = args.single_source - 1;
@@ -639,13 +641,13 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
     // every token of mine is past the bound: nothing to send; the first workgroup stays (it publishes the totals)
     if (!receiver && blockIdx.x != 0 && first_token >= tokens) return;
 
-    // The first entries and the ids of my tokens' routes are asked for first of all: they travel
-    // while the tables are cleared and the receivers' descriptors copied to LDS.
+    // The first entries and the ids of my tokens' routes are asked for first of all, then the rows of the
+    // first round: they travel while the entries are counted and the routes resolved.
     constexpr uint32_t kBatch = 10;   // 8192 entries over 896 threads in one batch: one trip to memory, not two
     uint32_t early[kBatch];
 #pragma unroll
     for (uint32_t j = 0; j < kBatch; ++j) {
-        const uint32_t f = j * blockDim.x + tid;
+        const uint32_t f = j * nthreads + tid;
         early[j] = f < flat_entries ? (uint32_t)src.indices[f] : 0xFFFFFFFFu;
     }
     const uint32_t my_routes = per_group * K;    // one thread each
@@ -653,35 +655,61 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
     if (!receiver && tid < my_routes && my_first + tid < flat_entries) {
         my_expert = (uint32_t)src.indices[my_first + tid];
     }
-    if (!receiver && tid < ws.world) s_dst[tid] = args.dst[tid];
+    // The descriptor of receiver `tid` is asked for here too and written to LDS after the counting (written
+    // here, the wait for it would cover the entries; asked for later, it would cover the rows).
+    const PushDst &dst_of_tid = args.dst[tid < ws.world ? tid : 0];
+    uint8_t *const my_out_x = dst_of_tid.out_x;
+    float *const my_out_scale = dst_of_tid.out_scale;
+    const uint64_t my_out_stride = dst_of_tid.out_stride;
+    const uint32_t my_os_elem = dst_of_tid.os_stride_elem, my_os_token = dst_of_tid.os_stride_token;
+    const uint32_t my_out_rows = dst_of_tid.out_rows;
+    // (The rows without a condition: a thread that has no piece asks for one it ignores later, from a row
+    // that exists; a value picked by a condition would be waited for right here.  Every barrier between
+    // here and the rows' use is an lds_barrier, and nothing is stored to memory in front of them: the
+    // compiler's own barrier after such stores waits for every outstanding load.)
+    const uint32_t teams = nthreads / team_threads;
+    const uint32_t team = tid / team_threads;
+    const uint32_t team_tid = tid - team * team_threads;
+    u32x4 pre_a, pre_b = {0, 0, 0, 0};
+    {
+        const uint32_t any_token =
+            receiver ? 0 : (first_token + team < src.num_tokens ? first_token + team : src.num_tokens - 1);
+        const uint8_t *x_row = src.x + (size_t)any_token * src.x_stride;
+        if constexpr (QUANT) {
+            const uint32_t pieces = args.hidden_dim / 16;
+            const u32x4 *piece = reinterpret_cast<const u32x4 *>(x_row + (size_t)(team_tid < pieces ? team_tid : 0) * 32);
+            pre_a = __builtin_nontemporal_load(piece);
+            pre_b = __builtin_nontemporal_load(piece + 1);
+        } else {
+            const uint32_t pieces = args.row_bytes / 16;
+            pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + (team_tid < pieces ? team_tid : 0));
+        }
+    }
 
     uint32_t *cnt = s_tab;                 // [E] entries per expert; receivers: [G][Le]
     uint32_t *prior = s_tab + E;           // [E] entries per expert before my first token
     uint32_t *rows_before = prior + E;     // [E] padded rows of all experts before e
     const uint32_t table = receiver ? G * Le : 2 * E;
-    for (uint32_t i = tid; i < table; i += blockDim.x) s_tab[i] = 0;
+    for (uint32_t i = tid; i < table; i += nthreads) s_tab[i] = 0;
     // Sources without tokens have no workgroup of their own: the first receiver
-    // workgroup (the first workgroup, if nobody receives) clears their tables.
-    if (blockIdx.x == (fin.recv_mask != 0 ? token_groups : 0)) {
+    // workgroup (the first workgroup, if nobody receives) clears their tables, at the end of its work.
+    auto clear_empty_sources = [&]() {
+        if (blockIdx.x != (fin.recv_mask != 0 ? token_groups : 0)) return;
         for (uint32_t g = 0; g < G; ++g) {
             if (args.src[g].num_tokens != 0) continue;
-            for (uint32_t e = tid; e < E; e += blockDim.x) {
+            for (uint32_t e = tid; e < E; e += nthreads) {
                 ws.num_routed[g * E + e] = 0;
                 ws.expert_offsets[g * E + e] = 0;
             }
         }
-    }
-    __syncthreads();
+    };
+    lds_barrier();
 
     // One pass over the entries of the step, kBatch loads in flight per lane.
     const uint32_t rank = blockIdx.x - token_groups;        // receivers only
-    for (uint32_t f0 = 0; f0 < flat_entries; f0 += kBatch * blockDim.x) {
-        uint32_t expert[kBatch];
-#pragma unroll
-        for (uint32_t j = 0; j < kBatch; ++j) {
-            const uint32_t f = f0 + j * blockDim.x + tid;
-            expert[j] = f0 == 0 ? early[j] : f < flat_entries ? (uint32_t)src.indices[f] : 0xFFFFFFFFu;
-        }
+    // (the first batch in straight-line code: inside the loop the compiler waits for every outstanding
+    // load, the rows included, before it uses the first entry)
+    auto count_batch = [&](const uint32_t (&expert)[kBatch], uint32_t f0) {
 #pragma unroll
         for (uint32_t j = 0; j < kBatch; ++j) {
             const uint32_t x = expert[j];
@@ -691,15 +719,29 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
                 if (le < Le) atomicAdd(&cnt[my_g * Le + le], 1u);
             } else {
                 atomicAdd(&cnt[x], 1u);
-                if (f0 + j * blockDim.x + tid < my_first) atomicAdd(&prior[x], 1u);
+                if (f0 + j * nthreads + tid < my_first) atomicAdd(&prior[x], 1u);
             }
         }
+    };
+    count_batch(early, 0);
+    for (uint32_t f0 = kBatch * nthreads; f0 < flat_entries; f0 += kBatch * nthreads) {
+        uint32_t expert[kBatch];
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t f = f0 + j * nthreads + tid;
+            expert[j] = f < flat_entries ? (uint32_t)src.indices[f] : 0xFFFFFFFFu;
+        }
+        count_batch(expert, f0);
     }
     if (!receiver && tid < my_routes) s_route_expert[tid] = my_expert;
-    __syncthreads();
+    if (!receiver && tid < ws.world) {
+        s_dst[tid] = PushDst{my_out_x, my_out_scale, my_out_stride, my_os_elem, my_os_token, my_out_rows, 0};
+    }
+    lds_barrier();
 
     if (receiver) {
         if (fin.recv_mask >> rank & 1) layout_from_totals(fin, ws, rank, cnt, scratch);
+        clear_empty_sources();
         return;
     }
 
@@ -707,22 +749,22 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
     // at the first expert of a receiver is the expert's first row there).
     const uint32_t pad = ws.expert_padding;
     uint32_t carry = 0;
-    for (uint32_t e0 = 0; e0 < E; e0 += blockDim.x) {
+    for (uint32_t e0 = 0; e0 < E; e0 += nthreads) {
         const uint32_t e = e0 + tid;
         const uint32_t total = e < E ? cnt[e] : 0;
         const uint32_t padded = e < E ? (total + pad - 1) / pad * pad : 0;
-        const uint32_t incl = carry + block_inclusive_scan(padded, scratch);
+        const uint32_t incl = carry + block_inclusive_scan<true>(padded, scratch);
         if (e < E) rows_before[e] = incl - padded;
-        if (e0 + blockDim.x < E) {   // uniform: another round follows
-            if (tid == blockDim.x - 1) s_carry = incl;
-            __syncthreads();
+        if (e0 + nthreads < E) {   // uniform: another round follows
+            if (tid == nthreads - 1) s_carry = incl;
+            lds_barrier();
             carry = s_carry;
         }
     }
-    __syncthreads();
+    lds_barrier();
 
     // The first workgroup publishes the source's totals (last wavefront).
-    if (blockIdx.x == 0 && tid / kWave == blockDim.x / kWave - 1) {
+    if (blockIdx.x == 0 && tid / kWave == nthreads / kWave - 1) {
         uint32_t run = 0;
         for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
             const uint32_t e = e0 + lane;
@@ -758,14 +800,10 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
         s_route_scale_ptr[tid] = scale_ptr;
         s_route_scale_stride[tid] = scale_stride;
     }
-    __syncthreads();
+    lds_barrier();
 
-    // The teams move one token each per round.  The rows are asked for only now: asking for the
-    // first two rounds' rows before the entries, or between asking for the entries and counting
-    // them, made the 1024-token step 3 and 4 us slower.
-    const uint32_t teams = blockDim.x / team_threads;
-    const uint32_t team = tid / team_threads;
-    const uint32_t team_tid = tid - team * team_threads;
+    // The teams move one token each per round; the rows of the first round are on their way since the head.
+    // (Asking for the rows of the next round before a round stores made the 1024-token step 3.4 us slower.)
     for (uint32_t first = 0; first < per_group; first += teams) {
         const uint32_t mine = first + team;                  // which of the workgroup's tokens
         const uint32_t token = first_token + mine;
@@ -777,10 +815,17 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
             scale_ptr = s_route_scale_ptr[mine * K + lane];
             scale_stride = s_route_scale_stride[mine * K + lane];
         }
-        push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale[team], s_scale_ptr[team],
-                         s_scale_stride[team], team_tid, team_threads, live);
+        if (first == 0) {
+            push_rows<QUANT, true>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale[team],
+                                   s_scale_ptr[team], s_scale_stride[team], team_tid, team_threads, live, pre_a,
+                                   pre_b);
+        } else {
+            push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale[team],
+                             s_scale_ptr[team], s_scale_stride[team], team_tid, team_threads, live);
+        }
         __syncthreads();   // the team's LDS arrays are reused by the next round
     }
+    clear_empty_sources();
 }
 
 // Pack of a large group step, after a routing launch that left, per chunk, the

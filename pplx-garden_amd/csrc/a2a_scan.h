@@ -3,6 +3,7 @@
 // rows from per-source totals.
 #pragma once
 
+#include "a2a_device.h"
 #include "a2a_internal.h"
 
 namespace a2a {
@@ -31,13 +32,15 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan(uint32_t v, uint32_t lan
 
 // Inclusive scan over the first blockDim.x values (one per thread); `scratch`
 // holds one word per wavefront.  Every thread of the workgroup must call.
+// LDS_ONLY: with barriers that leave loads from memory in flight (lds_barrier).
+template <bool LDS_ONLY = false>
 __device__ __forceinline__ uint32_t block_inclusive_scan(uint32_t v, uint32_t *scratch) {
     const uint32_t lane = threadIdx.x & (kWave - 1);
     const uint32_t wave = threadIdx.x / kWave;
     const uint32_t incl = wave_inclusive_scan(v, lane);
-    __syncthreads();
+    if constexpr (LDS_ONLY) lds_barrier(); else __syncthreads();
     if (lane == kWave - 1) scratch[wave] = incl;
-    __syncthreads();
+    if constexpr (LDS_ONLY) lds_barrier(); else __syncthreads();
     uint32_t before = 0;
     for (uint32_t w = 0; w < wave; ++w) before += scratch[w];
     return before + incl;
