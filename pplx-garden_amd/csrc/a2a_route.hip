@@ -222,6 +222,21 @@ template <int MODE>
 __global__ __launch_bounds__(kRouteBlock) void route_hist_kernel(const RouteArgs args,
                                                                  const Workspace ws) {
     __shared__ uint16_t wave_hist[kRouteWaves][A2A_MAX_EXPERTS];
+    if constexpr (MODE == 1) {
+        // what the head of a workgroup takes from the argument block, asked for in one go
+        A2A_PIN(args.block_start[0]);
+        A2A_PIN(args.block_start[1]);
+        A2A_PIN(ws.num_groups);
+        A2A_PIN(ws.num_experts);
+        A2A_PIN(ws.topk);
+        A2A_PIN(ws.nb_max);
+        A2A_PIN(ws.max_tk);
+        A2A_PIN(ws.turn);
+        A2A_PIN(ws.totals);
+        A2A_PIN(ws.chunk_counts);
+        A2A_PIN(ws.local_rank);
+        A2A_PIN(ws.err);
+    }
     const uint32_t G = ws.num_groups, E = ws.num_experts;
     const uint32_t words = MODE == 2 ? E + ws.world : (G + 1) * E;
     uint32_t *totals = MODE == 2 ? ws.send_totals : ws.totals;

@@ -18,9 +18,11 @@ size_t align_up_sz(size_t n, size_t a) { return (n + a - 1) / a * a; }
 // ---------------------------------------------------------------------------
 
 // Stages the row of `token` (payload, then scales).  Whole workgroup.
-template <bool QUANT>
+// PRE: the thread's first piece of the row was asked for earlier and is passed in.
+template <bool QUANT, bool PRE = false>
 __device__ __forceinline__ void stage_row(const StageSendArgs &args, const Staging &st, uint32_t g, uint32_t token,
-                                          uint32_t staging_threads) {
+                                          uint32_t staging_threads, u32x4 pre_a = u32x4{0, 0, 0, 0},
+                                          u32x4 pre_b = u32x4{0, 0, 0, 0}) {
     const uint32_t tid = threadIdx.x;
     if (tid >= staging_threads) return;
     const uint32_t lane = tid & (kWave - 1);
@@ -36,7 +38,10 @@ __device__ __forceinline__ void stage_row(const StageSendArgs &args, const Stagi
             const uint32_t c = base + lane;
             const bool active = c < num_chunks;
             u32x4 a = {0, 0, 0, 0}, b = {0, 0, 0, 0};
-            if (active) {
+            if (PRE && base == wave * kWave) {
+                a = pre_a;
+                b = pre_b;
+            } else if (active) {
                 const u32x4 *p = reinterpret_cast<const u32x4 *>(x_row + (size_t)c * 32);
                 a = __builtin_nontemporal_load(p);
                 b = __builtin_nontemporal_load(p + 1);
@@ -52,7 +57,7 @@ __device__ __forceinline__ void stage_row(const StageSendArgs &args, const Stagi
         const uint32_t num_chunks = args.row_bytes / 16;
         for (uint32_t c = tid; c < num_chunks; c += staging_threads) {
             reinterpret_cast<u32x4 *>(row)[c] =
-                __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
+                PRE && c == tid ? pre_a : __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + c);
         }
         if (src.x_scale != nullptr) {
             const float *xs = src.x_scale + (size_t)token * src.xs_stride_token;
@@ -172,23 +177,39 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
     load_batch(0, first_batch);
     uint32_t my_expert = 0xFFFFFFFFu;
     if (lane < K) my_expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
+    // The row is asked for here, after the entries, and travels while they are counted.  Without a
+    // condition (a thread without a piece asks for one it ignores), and every barrier up to its use
+    // waits for LDS only: otherwise something on the way would wait for it by accident.
+    u32x4 pre_a, pre_b = {0, 0, 0, 0};
+    {
+        const uint8_t *x_row = src.x + (size_t)token * src.x_stride;
+        if constexpr (QUANT) {
+            const uint32_t pieces = args.hidden_dim / 16;
+            const u32x4 *piece = reinterpret_cast<const u32x4 *>(x_row + (size_t)(tid < pieces ? tid : 0) * 32);
+            pre_a = __builtin_nontemporal_load(piece);
+            pre_b = __builtin_nontemporal_load(piece + 1);
+        } else {
+            const uint32_t pieces = args.row_bytes / 16;
+            pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + (tid < pieces ? tid : 0));
+        }
+    }
 
     for (uint32_t i = tid; i < 2 * E; i += nthreads) s_send[i] = 0;
-    __syncthreads();
+    lds_barrier();
     count_batch(0, first_batch);
     for (uint32_t f0 = 8 * nthreads; f0 < entries; f0 += 8 * nthreads) {
         uint32_t expert[8];
         load_batch(f0, expert);
         count_batch(f0, expert);
     }
-    __syncthreads();
+    lds_barrier();
 
     // Scan over the experts (a2a_dispatch_send.cu:236-242); token 0 publishes.
     uint32_t carry = 0;
     for (uint32_t e0 = 0; e0 < E; e0 += nthreads) {
         const uint32_t e = e0 + tid;
         const uint32_t c = e < E ? cnt[e] : 0;
-        const uint32_t incl = carry + block_inclusive_scan(c, scratch);
+        const uint32_t incl = carry + block_inclusive_scan<true>(c, scratch);
         if (e < E) {
             excl[e] = incl - c;
             if (token == 0) {
@@ -198,11 +219,11 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
         }
         if (e0 + nthreads < E) {   // uniform: another round follows
             if (tid == nthreads - 1) s_carry = incl;
-            __syncthreads();
+            lds_barrier();
             carry = s_carry;
         }
     }
-    __syncthreads();
+    lds_barrier();
     if (token >= eff) return;   // past bound_m: nothing to stage (uniform)
 
     if (wave == 0) {
@@ -224,7 +245,7 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
             ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
         }
     }
-    stage_row<QUANT>(args, st, g, token, nthreads);
+    stage_row<QUANT, true>(args, st, g, token, nthreads, pre_a, pre_b);
 }
 
 // The send of a large step, after a routing launch that left the chunk counts,
