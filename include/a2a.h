@@ -130,7 +130,12 @@ int a2a_ctx_status(a2a_ctx *ctx, void *stream, uint32_t *flags);
  *                         1: rows are bf16; they are quantised to fp8 e4m3 with
  *                            one float scale per 128 elements (needs
  *                            in_elemsize 1, hidden_dim_scale = hidden_dim/128,
- *                            x_scale_ptr NULL)
+ *                            x_scale_ptr NULL).  Per group of 128: amax =
+ *                            max(max|x|, 1e-4), scale = amax / 448, code =
+ *                            e4m3(x * (448 / amax)), round to nearest even.  A NaN
+ *                            in a group makes its scale NaN and its 128 codes
+ *                            0x7F; an infinity makes its scale +inf, the code of
+ *                            an infinite value 0x7F, of a finite one a signed zero
  *   x_scale_*             optional float scales [T, Hs], strides in ELEMENTS
  *   indices               [T, K] expert ids, row stride in elements
  *   weights               unused by dispatch, as in the reference
@@ -256,7 +261,10 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
  *     dropped silently as described at those bits.
  *   - The first call on a GPU also looks up where that GPU holds the array
  *     (hipGetSymbolAddress, once per device): make one call outside any
- *     stream capture before capturing calls into a graph.
+ *     stream capture before capturing calls into a graph.  A first call on a
+ *     stream that is being captured is refused with A2A_ERR_BAD_ORDER.
+ *   - A refused call enqueues nothing: every check of the step runs before the
+ *     first launch.
  *   - The routing of the step stays inside the library: a2a_combine needs a
  *     context and the a2a_dispatch that goes with it.
  * Error text: a2a_last_error(NULL) on the calling thread.

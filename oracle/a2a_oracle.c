@@ -142,13 +142,25 @@ void oracle_layout(const uint32_t *num_routed, uint32_t N, uint32_t E, uint32_t 
  * reference; the rule (all float32, separately rounded operations):
  *   amax = max(max|x|, 1e-4); scale = amax / 448;
  *   q = e4m3fn(clamp(x * (448 / amax), -448, 448))
+ * with maxima that propagate NaN and one spelling of NaN on output: a NaN in
+ * the group gives scale 0x7FC00000 and 128 codes 0x7F; an infinity (no NaN)
+ * gives scale +inf, code 0x7F for an infinite value (inf * 0) and a zero with
+ * its sign for a finite one (x * 0).
  */
 void oracle_quantize_row(const uint16_t *x, uint32_t H, uint8_t *q, float *scale) {
     for (uint32_t g = 0; g < H / 128; ++g) {
         float amax = 0.0f;
+        int has_nan = 0;
         for (uint32_t i = 0; i < 128; ++i) {
             const float a = fabsf(bf16_to_f32(x[g * 128 + i]));
+            if (a != a) has_nan = 1;
             if (a > amax) amax = a;
+        }
+        if (has_nan) {
+            const uint32_t quiet = 0x7FC00000u;
+            memcpy(&scale[g], &quiet, 4);
+            memset(q + g * 128, 0x7F, 128);
+            continue;
         }
         if (!(amax > 1e-4f)) amax = 1e-4f;
         volatile float inv = 448.0f / amax;
@@ -158,7 +170,8 @@ void oracle_quantize_row(const uint16_t *x, uint32_t H, uint8_t *q, float *scale
             float c = v;
             if (c > 448.0f) c = 448.0f;
             if (c < -448.0f) c = -448.0f;
-            q[g * 128 + i] = oracle_e4m3fn_encode(c);
+            const uint8_t code = oracle_e4m3fn_encode(c);
+            q[g * 128 + i] = (code & 0x7F) == 0x7F ? 0x7F : code;
         }
     }
 }

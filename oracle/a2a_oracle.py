@@ -420,6 +420,10 @@ AMAX_FLOOR = np.float32(1e-4)
 QUANT_GROUP = 128
 
 
+NAN_CODE = np.uint8(0x7F)
+QUIET_NAN_BITS = np.uint32(0x7FC00000)
+
+
 def quantize_block128(x_bf16: np.ndarray):
     """bf16 rows -> (fp8 e4m3fn codes [T,H], float32 scales [T,H/128]).
 
@@ -430,23 +434,42 @@ def quantize_block128(x_bf16: np.ndarray):
         q_i   = e4m3fn_rne(clamp(x_i * (448 / amax), -448, 448))
     The multiply and the two divisions are separate correctly rounded float32
     operations (no fused multiply-add, no reciprocal approximation).
+
+    Non-finite values follow from the same arithmetic with NaN-propagating
+    maxima (numpy's, torch's), and NaN has ONE spelling on output (code 0x7F,
+    scale bits 0x7FC00000; which NaN an operation returns differs between
+    machines):
+      * a NaN in the group: amax, scale and every product are NaN, so the
+        scale is NaN and all 128 codes are 0x7F;
+      * an infinity and no NaN: amax = scale = +inf, 448 / amax = 0, so a
+        finite value becomes a zero with its sign (0x00 / 0x80) and an infinite
+        one (inf * 0 = NaN) the code 0x7F.
+    Either way the group dequantises to NaN throughout: a bad activation stays
+    visible, as it does in the reference, which moves the caller's bytes
+    untouched (a2a_dispatch_send.cu:341-367).
     """
     x = bf16_to_f32(x_bf16)
     T, H = x.shape
     assert H % QUANT_GROUP == 0
     g = x.reshape(T, H // QUANT_GROUP, QUANT_GROUP)
-    amax = np.maximum(np.abs(g).max(axis=2), AMAX_FLOOR).astype(np.float32)
-    inv = (FP8_MAX / amax).astype(np.float32)
-    scale = (amax / FP8_MAX).astype(np.float32)
-    y = (g * inv[:, :, None]).astype(np.float32)
-    y = np.clip(y, -FP8_MAX, FP8_MAX)
-    return e4m3fn_encode(y).reshape(T, H), scale
+    with np.errstate(invalid="ignore", over="ignore"):
+        amax = np.maximum(np.abs(g).max(axis=2), AMAX_FLOOR).astype(np.float32)
+        inv = (FP8_MAX / amax).astype(np.float32)
+        scale = (amax / FP8_MAX).astype(np.float32)
+        y = (g * inv[:, :, None]).astype(np.float32)
+        y = np.clip(y, -FP8_MAX, FP8_MAX)
+    codes = e4m3fn_encode(y).reshape(T, H)
+    codes = np.where((codes & 0x7F) == 0x7F, NAN_CODE, codes).astype(np.uint8)
+    scale_bits = scale.view(np.uint32)
+    scale = np.where(np.isnan(scale), QUIET_NAN_BITS, scale_bits).astype(np.uint32).view(np.float32)
+    return codes, scale
 
 
 def dequantize_block128(q: np.ndarray, scale: np.ndarray) -> np.ndarray:
     T, H = q.shape
     v = e4m3fn_decode(q).reshape(T, H // QUANT_GROUP, QUANT_GROUP)
-    return (v * scale[:, :, None]).astype(np.float32).reshape(T, H)
+    with np.errstate(invalid="ignore"):
+        return (v * scale[:, :, None]).astype(np.float32).reshape(T, H)
 
 
 # ---------------------------------------------------------------------------

@@ -55,14 +55,20 @@ def source_order(rank: int, world_size: int, node_size: int) -> List[int]:
 
 
 def quantize_block128(x: torch.Tensor):
-    """bf16 [T, H] -> (fp8 e4m3 codes uint8 [T, H], float32 scales [T, H / 128])."""
+    """bf16 [T, H] -> (fp8 e4m3 codes uint8 [T, H], float32 scales [T, H / 128]).
+
+    A NaN or an infinity in a group goes through the same operations (torch's maxima propagate
+    NaN); on output NaN has one spelling: code 0x7F, scale bits 0x7FC00000."""
     T, H = x.shape
     f = x.to(torch.float32).reshape(T, H // QUANT_GROUP, QUANT_GROUP)
     amax = f.abs().amax(dim=-1, keepdim=True).clamp_min(1e-4)
     inv = torch.tensor(FP8_MAX, dtype=torch.float32) / amax
     q = (f * inv).clamp(-FP8_MAX, FP8_MAX).to(torch.float8_e4m3fn)
     scale = (amax / torch.tensor(FP8_MAX, dtype=torch.float32)).reshape(T, H // QUANT_GROUP)
-    return q.reshape(T, H).view(torch.uint8), scale
+    codes = q.reshape(T, H).view(torch.uint8)
+    codes = torch.where((codes & 0x7F) == 0x7F, torch.full_like(codes, 0x7F), codes)
+    scale = torch.where(scale.isnan(), torch.full_like(scale, float("nan")), scale)
+    return codes, scale
 
 
 def dispatch_world(xs: Sequence[torch.Tensor], indices: Sequence[torch.Tensor], *, num_experts: int,

@@ -376,12 +376,22 @@ size_t carve_workspace(const a2a_config &c, uint32_t max_tokens, uint8_t *base, 
     return off;
 }
 
-// The group dispatch on the tables of `ws`: argument checks, then the launches.  `ctx` only
-// receives error texts and may be null (then they go where a2a_last_error(NULL) finds them).
-// `num_tokens_out[g]`, if not null, gets the tokens of every source.
-int dispatch_group(a2a_ctx *ctx, const a2a_config &c, const Workspace &ws, const a2a_dispatch_args *args,
-                   uint32_t quantize, hipStream_t s, KernelTiming pack_timing, KernelTiming route_timing,
-                   uint32_t *num_tokens_out) {
+// Everything the launches of a group dispatch take, built from the callers' arguments.
+struct GroupPlan {
+    RouteArgs ra;
+    FinalizeArgs fa;
+    PushArgs pa;
+    uint32_t blocks = 0;                  // routing chunks of all sources
+    uint32_t tokens = 0;                  // tokens of all sources
+    uint32_t num_tokens[kMaxWorld] = {};  // per source
+};
+
+// First half of a group dispatch: every argument check, and the plan.  Enqueues nothing and
+// changes nothing: a refused call leaves the stream, the tables and the context as they were.
+// `ctx` only receives error texts and may be null (then they go where a2a_last_error(NULL)
+// finds them).
+int plan_dispatch_group(a2a_ctx *ctx, const a2a_config &c, const a2a_dispatch_args *args, uint32_t quantize,
+                        GroupPlan &plan) {
     const uint32_t N = c.world_size, K = c.num_experts_per_token;
     for (uint32_t r = 0; r < N; ++r) {
         const a2a_dispatch_args &a = args[r];
@@ -393,9 +403,9 @@ int dispatch_group(a2a_ctx *ctx, const a2a_config &c, const Workspace &ws, const
             return rc;
     }
 
-    RouteArgs ra;
-    FinalizeArgs fa;
-    PushArgs pa;
+    RouteArgs &ra = plan.ra;
+    FinalizeArgs &fa = plan.fa;
+    PushArgs &pa = plan.pa;
     memset(&ra, 0, sizeof ra);
     memset(&fa, 0, sizeof fa);
     memset(&pa, 0, sizeof pa);
@@ -427,7 +437,7 @@ int dispatch_group(a2a_ctx *ctx, const a2a_config &c, const Workspace &ws, const
         ps.num_tokens = T;
         pa.token_start[g] = tokens;
         tokens += T;
-        if (num_tokens_out != nullptr) num_tokens_out[g] = T;
+        plan.num_tokens[g] = T;
     }
     for (uint32_t g = G; g <= (uint32_t)kMaxWorld; ++g) {
         ra.block_start[g] = blocks;
@@ -453,7 +463,19 @@ int dispatch_group(a2a_ctx *ctx, const a2a_config &c, const Workspace &ws, const
     pa.hidden_dim = c.hidden_dim;
     pa.hidden_dim_scale = c.hidden_dim_scale;
     pa.topk_magic = K > 1 ? (uint32_t)((0x100000000ull + K - 1) / K) : 0;
+    plan.blocks = blocks;
+    plan.tokens = tokens;
+    return A2A_OK;
+}
 
+// Second half: the launches of an accepted plan on the tables of `ws`.
+int launch_dispatch_group(a2a_ctx *ctx, const a2a_config &c, const Workspace &ws, const GroupPlan &plan,
+                          uint32_t quantize, hipStream_t s, KernelTiming pack_timing, KernelTiming route_timing) {
+    const RouteArgs &ra = plan.ra;
+    const FinalizeArgs &fa = plan.fa;
+    const PushArgs &pa = plan.pa;
+    const uint32_t blocks = plan.blocks, tokens = plan.tokens;
+    const uint32_t G = c.world_size / c.dp_size;
     hipError_t e;
     if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && dispatch_small_fits(pa, ws, quantize != 0, tokens)) {
         e = launch_dispatch_small(pa, fa, ws, quantize != 0, tokens, s, pack_timing);
@@ -491,16 +513,23 @@ constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
 uint8_t *g_scratch_ptr[kMaxDevices] = {};
 
-hipError_t static_scratch_of(int dev, uint8_t **out) {
+int static_scratch_of(int dev, hipStream_t stream, uint8_t **out) {
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (g_scratch_ptr[dev] == nullptr) {
+        // The look-up loads the symbol's module on this device: not a call to make while `stream`
+        // is being captured into a graph.
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(stream, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone)
+            return fail(nullptr, A2A_ERR_BAD_ORDER,
+                        "the first a2a_dispatch_static on a GPU looks up where that GPU holds the library's array, "
+                        "which a stream capture forbids: make one call on device %d outside the capture first", dev);
         void *ptr = nullptr;
         const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-        if (e != hipSuccess) return e;
+        if (e != hipSuccess) return hip_fail(nullptr, e, "hipGetSymbolAddress(scratch)");
         g_scratch_ptr[dev] = static_cast<uint8_t *>(ptr);
     }
     *out = g_scratch_ptr[dev];
-    return hipSuccess;
+    return A2A_OK;
 }
 
 // What a step on tables that hold another step's leftovers needs before its
@@ -668,9 +697,13 @@ int a2a_dispatch(a2a_ctx *ctx, const a2a_dispatch_args *args, uint32_t quantize,
     const KernelTiming route_timing = ctx->timing[A2A_KERNEL_ROUTE];
     ctx->timing[A2A_KERNEL_PACK] = KernelTiming();
     ctx->timing[A2A_KERNEL_ROUTE] = KernelTiming();
-    if (int rc = dispatch_group(ctx, ctx->cfg, ctx->ws, args, quantize, static_cast<hipStream_t>(stream), pack_timing,
-                                route_timing, ctx->num_tokens))
+    GroupPlan plan;
+    if (int rc = plan_dispatch_group(ctx, ctx->cfg, args, quantize, plan)) return rc;
+    if (int rc = launch_dispatch_group(ctx, ctx->cfg, ctx->ws, plan, quantize, static_cast<hipStream_t>(stream),
+                                       pack_timing, route_timing))
         return rc;
+    // only an accepted step replaces what the context knows of the previous one
+    memcpy(ctx->num_tokens, plan.num_tokens, sizeof ctx->num_tokens);
     ctx->group_routing = true;
     ctx->step_open = false;
     ctx->sent_mask = 0;
@@ -706,20 +739,22 @@ int a2a_dispatch_static(const a2a_config *config, const a2a_dispatch_args *args,
                     "a2a_dispatch_static has %zu (use a2a_ctx_create and a2a_dispatch for larger steps)",
                     c.world_size, (unsigned long long)max_tokens, c.num_experts_per_token, c.num_experts, need,
                     (size_t)A2A_STATIC_SCRATCH_BYTES);
+    // Every check of the step before anything is enqueued: a refused call does nothing.
+    GroupPlan plan;
+    if (int rc = plan_dispatch_group(nullptr, c, args, quantize, plan)) return rc;
     DeviceGuard guard(c.device);
     if (!guard.ok) return fail(nullptr, A2A_ERR_INVALID_ARGUMENT, "cannot select device %d", c.device);
+    hipStream_t s = static_cast<hipStream_t>(stream);
     uint8_t *base = nullptr;
-    hipError_t e = static_scratch_of(c.device, &base);
-    if (e != hipSuccess) return hip_fail(nullptr, e, "hipGetSymbolAddress(scratch)");
+    if (int rc = static_scratch_of(c.device, s, &base)) return rc;
     carve_workspace(c, (uint32_t)max_tokens, base, ws);
     if (device_flags != nullptr) ws.err = device_flags;
-    hipStream_t s = static_cast<hipStream_t>(stream);
     const uint32_t words = 2 * (ws.num_groups + 1) * ws.num_experts;
     const uint32_t blocks = words > 8 * 1024 ? 8 : 1;
     hipLaunchKernelGGL(static_prepare_kernel, dim3(blocks), dim3(1024), 0, s, ws, device_flags == nullptr ? 1u : 0u);
-    e = hipGetLastError();
+    const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return hip_fail(nullptr, e, "launch static_prepare");
-    return dispatch_group(nullptr, c, ws, args, quantize, s, KernelTiming(), KernelTiming(), nullptr);
+    return launch_dispatch_group(nullptr, c, ws, plan, quantize, s, KernelTiming(), KernelTiming());
 }
 
 int a2a_combine(a2a_ctx *ctx, const a2a_combine_args *args, uint32_t expert_y_dtype,

@@ -293,6 +293,26 @@ int main() {
             d2[r].out_x = ox2[r];
             d2[r].out_x_scale = (float *)os2[r];
         }
+        // The FIRST call on a GPU looks up the library's array there, which a stream capture forbids:
+        // it is refused, and the refusal leaves nothing in the graph.
+        auto captured = [&](const a2a_dispatch_args *args, int *rc_out, size_t *nodes_out) -> int {
+            hipGraph_t graph = nullptr;
+            HIP_OK(hipStreamBeginCapture(stream, hipStreamCaptureModeRelaxed));
+            *rc_out = a2a_dispatch_static(&cfg, args, /*quantize=*/1, d_flags, stream);
+            HIP_OK(hipStreamEndCapture(stream, &graph));
+            *nodes_out = 99;
+            HIP_OK(hipGraphGetNodes(graph, nullptr, nodes_out));
+            HIP_OK(hipGraphDestroy(graph));
+            return 0;
+        };
+        int rc_cap = 0;
+        size_t nodes = 0;
+        if (int e = captured(d2, &rc_cap, &nodes)) return e;
+        const bool first_refused = rc_cap == A2A_ERR_BAD_ORDER && nodes == 0;
+        std::printf("static dispatch, first call under capture: %s (%d, %zu nodes)\n",
+                    first_refused ? "refused" : "NOT REFUSED", rc_cap, nodes);
+        if (!first_refused) ++failures;
+
         A2A_OK_OR_FAIL(a2a_dispatch(ctx, d, /*quantize=*/1, stream));
         const int rc = a2a_dispatch_static(&cfg, d2, /*quantize=*/1, d_flags, stream);
         if (rc != 0) {
@@ -318,6 +338,19 @@ int main() {
         }
         std::printf("static dispatch: %s\n", same ? "identical to a2a_dispatch" : "DIFFERS from a2a_dispatch");
         if (!same) ++failures;
+        // After that eager call a capture takes the launches; a call that is refused (tokens without
+        // rows) still records none: every check runs before the first launch.
+        a2a_dispatch_args bad[N];
+        std::memcpy(bad, d2, sizeof bad);
+        bad[N - 1].x_ptr = nullptr;
+        if (int e = captured(bad, &rc_cap, &nodes)) return e;
+        const bool clean_refusal = rc_cap == A2A_ERR_INVALID_ARGUMENT && nodes == 0;
+        if (int e = captured(d2, &rc_cap, &nodes)) return e;
+        const bool recorded = rc_cap == 0 && nodes >= 2;
+        std::printf("static dispatch under capture: refused call %s, accepted call %s (%zu nodes)\n",
+                    clean_refusal ? "recorded nothing" : "LEFT NODES BEHIND", recorded ? "recorded" : "NOT RECORDED",
+                    nodes);
+        if (!clean_refusal || !recorded) ++failures;
         for (uint32_t r = 0; r < N; ++r) {
             (void)hipFree(n2[r]);
             (void)hipFree(ox2[r]);

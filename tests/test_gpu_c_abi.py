@@ -24,6 +24,9 @@ def test_cpp_caller_of_the_c_abi():
     assert "selftest passed" in done.stdout
     assert "group calls" in done.stdout and "split calls" in done.stdout
     assert "static dispatch: identical to a2a_dispatch" in done.stdout
+    # a first call under stream capture is refused; a refused call leaves no node in the caller's graph
+    assert "first call under capture: refused" in done.stdout
+    assert "refused call recorded nothing, accepted call recorded" in done.stdout
 
 
 def test_memory_ceilings_program_runs():

@@ -58,6 +58,62 @@ def test_quantiser_on_every_bf16_value_and_many_scales():
 
 
 @pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
+@pytest.mark.parametrize("repeat", [1, 110, 450], ids=["one_launch_small", "one_launch_single", "two_launch"])
+def test_quantiser_on_nan_infinity_and_the_largest_bf16_value(repeat, split):
+    """A NaN poisons its group of 128 (scale NaN, every code the NaN code), an infinity makes the
+    scale infinite: bit for bit what the oracle says (which the CPU tests pin against a hand-written
+    expectation and torch's operations), in every dispatch kernel that quantises (10, 1100 and 4500
+    tokens take the three paths of the group call and of the split send)."""
+    from a2a_nonfinite import bad_rows, expected_special_groups
+
+    bits, kinds = bad_rows()
+    H = bits.shape[1]
+    x_codes = np.tile(bits, (repeat, 1))
+    T = x_codes.shape[0]
+    case = replace(C0, name="quant_bad", num_tokens=T, hidden_dim=H, topk=2, num_experts=8, world_size=2)
+    x = torch.from_numpy(x_codes.view(np.int16).copy()).view(torch.bfloat16)
+    gen = torch.Generator().manual_seed(5)
+    idx = torch.rand((T, 8), generator=gen).topk(2, dim=-1).indices.to(torch.int32)
+    w = torch.full((T, 2), 0.5, dtype=torch.float32)
+    empty = dict(x=torch.zeros((0, H), dtype=torch.bfloat16), idx=torch.zeros((0, 2), dtype=torch.int32),
+                 w=torch.zeros((0, 2), dtype=torch.float32))
+    ins = [dict(x=x, idx=idx, w=w), empty]
+    want = oracle.dispatch_world(
+        [oracle.RankInput(x=bf16_codes(i["x"]), indices=i["idx"].numpy()) for i in ins],
+        num_experts=8, world_size=2, node_size=2, expert_padding=1, out_rows=2 * T, quantize=True)
+    _, ops = make_ops(case, DEV, max_num_tokens=T)
+    try:
+        outs = [dict(n=torch.full((4,), -1, dtype=torch.int32, device=DEV),
+                     x=torch.full((2 * T, H), SENTINEL, dtype=torch.uint8, device=DEV).view(torch.float8_e4m3fn),
+                     s=torch.full((2 * T, H // 128), -7.0, dtype=torch.float32, device=DEV)) for _ in range(2)]
+        phases = [dict(do_send=True, do_recv=False), dict(do_send=False, do_recv=True)] if split else [dict()]
+        for kw in phases:
+            for r in range(2):
+                ops[r].dispatch(out_expert_num_tokens=outs[r]["n"], out_expert_x=outs[r]["x"],
+                                out_expert_x_scale=outs[r]["s"], dp_x=ins[r]["x"].to(DEV), dp_x_scale=None,
+                                indices=ins[r]["idx"].view(torch.uint32).to(DEV), weights=ins[r]["w"].to(DEV), **kw)
+        torch.cuda.synchronize(DEV)
+        assert ops[0].context.status() == 0
+        for r in range(2):
+            wr = want[r].written
+            np.testing.assert_array_equal(outs[r]["n"].cpu().numpy(), want[r].num_tokens)
+            np.testing.assert_array_equal(outs[r]["x"].view(torch.uint8).cpu().numpy()[wr], want[r].x[wr])
+            np.testing.assert_array_equal(outs[r]["s"].cpu().numpy().view(np.uint32)[wr],
+                                          want[r].x_scale.view(np.uint32)[wr])
+        # and against the hand-written expectation directly, on the copies of the first ten tokens
+        slots = want[0].slots[0]
+        for row, group, codes, scale_bits in expected_special_groups(bits, kinds):
+            for k in range(2):
+                r, slot = int(idx[row, k]) // 4, int(slots[row, k])
+                got = outs[r]["x"].view(torch.uint8)[slot, group * 128:(group + 1) * 128].cpu().numpy()
+                np.testing.assert_array_equal(got, codes)
+                assert int(outs[r]["s"][slot, group].view(torch.int32).item()) & 0xFFFFFFFF == scale_bits
+    finally:
+        for op in ops:
+            op.destroy()
+
+
+@pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
 @pytest.mark.parametrize("case", [C0, scaled(C0, 1200)], ids=["one_launch", "two_launch"])
 def test_bound_m_limits_the_tokens(case, split):
     world = make_world(case, "all")
@@ -135,8 +191,18 @@ def _check_split_combine_refuses_narrow_rows(in_dtype, out_dtype):
         with pytest.raises(RuntimeError, match="element size of out_dtype"):
             ops[0].combine(out_tokens=t[0]["o"], indices=t[0]["idx"], weights=t[0]["w"], expert_y=t[0]["y"],
                            do_send=True, do_recv=False)
-        with pytest.raises(RuntimeError, match="as wide as out_dtype"):
-            ops[0].context.combine_send(0, t[0]["y"].data_ptr(), cfg.hidden_dim * in_dtype.itemsize, rows, 0)
+        if in_dtype.itemsize < out_dtype.itemsize:
+            with pytest.raises(RuntimeError, match="as wide as out_dtype"):
+                ops[0].context.combine_send(0, t[0]["y"].data_ptr(), cfg.hidden_dim * in_dtype.itemsize, rows, 0)
+        else:
+            # wider rows can be copied (their first bytes), but the recv is told the type and refuses
+            # to read staging rows sized for 2-byte elements as 4-byte ones
+            for r in range(4):
+                ops[r].context.combine_send(r, t[r]["y"].data_ptr(), cfg.hidden_dim * in_dtype.itemsize, rows, 0)
+            with pytest.raises(RuntimeError, match="does not have the 2-byte elements"):
+                ops[0].context.combine_recv(0, cfg.max_num_tokens, rows, in_dtype, t[0]["o"].data_ptr(),
+                                            cfg.hidden_dim, t[0]["idx"].data_ptr(), cfg.num_experts_per_token,
+                                            t[0]["w"].data_ptr(), cfg.num_experts_per_token, None, False, 0)
         torch.cuda.synchronize(DEV)
         assert ops[0].context.status() == 0
     finally:
@@ -148,11 +214,14 @@ def _check_split_combine_refuses_narrow_rows(in_dtype, out_dtype):
 @pytest.mark.parametrize("in_dtype,out_dtype", [
     (torch.bfloat16, torch.bfloat16), (torch.float32, torch.float32), (torch.float16, torch.float16),
     (torch.bfloat16, torch.float32), (torch.float16, torch.float32),
+    (torch.bfloat16, torch.float16), (torch.float16, torch.bfloat16),
+    (torch.float32, torch.bfloat16), (torch.float32, torch.float16),
 ], ids=lambda d: str(d).split(".")[-1])
 def test_combine_types_and_accumulate(in_dtype, out_dtype, split):
-    """expert_y in {f16, bf16, f32} x out in {f16, bf16, f32} (launch_utils.cuh:183-194), with and
-    without accumulate (a2a_combine_recv.cu:132).  The split calls stage rows sized for the
-    output type, so there expert_y has the output's element size."""
+    """All nine pairs expert_y in {f16, bf16, f32} x out in {f16, bf16, f32} that the reference
+    instantiates (a2a_combine_recv.cu:237-238, launch_utils.cuh:183-194), with and without accumulate
+    (a2a_combine_recv.cu:132).  The split calls stage rows sized for the output type, so there
+    expert_y has the output's element size (seven pairs through the group call only)."""
     if split and in_dtype.itemsize != out_dtype.itemsize:
         _check_split_combine_refuses_narrow_rows(in_dtype, out_dtype)
         return

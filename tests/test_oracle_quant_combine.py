@@ -52,6 +52,57 @@ def test_quantize_special_groups():
     np.testing.assert_array_equal(cs, s)
 
 
+def test_quantize_non_finite_groups():
+    """NaN, infinities and the largest bf16 value inside ordinary rows: the hand-written
+    expectation, torch's library operations (NaN spelled one way), and the C restatement."""
+    from a2a_nonfinite import BF16_MAX, bad_rows, expected_special_groups
+
+    bits, kinds = bad_rows()
+    q, s = oracle.quantize_block128(bits)
+    sb = s.view(np.uint32)
+    special = expected_special_groups(bits, kinds)
+    assert len(special) == len([k for k in kinds.values() if k != "max"])
+    for row, group, codes, scale_bits in special:
+        np.testing.assert_array_equal(q[row, group * 128:(group + 1) * 128], codes, err_msg=f"row {row} group {group}")
+        assert sb[row, group] == scale_bits, (row, group, hex(sb[row, group]))
+    # every other group is what it is without the special value next door: groups are independent
+    clean = bits.copy()
+    for (row, group), kind in kinds.items():
+        if kind != "max":
+            clean[row, group * 128:(group + 1) * 128] = 0
+    cq, cs = oracle.quantize_block128(clean)
+    for row in range(bits.shape[0]):
+        for group in range(bits.shape[1] // 128):
+            if kinds.get((row, group)) in ("nan", "inf"):
+                continue
+            np.testing.assert_array_equal(q[row, group * 128:(group + 1) * 128], cq[row, group * 128:(group + 1) * 128])
+            assert sb[row, group] == cs.view(np.uint32)[row, group]
+    assert np.isfinite(cs).all() and not ((cq & 0x7F) == 0x7F).any()
+    # the largest finite bf16 value is an ordinary maximum: +-448 exactly, scale = value / 448
+    big = np.float32(oracle.bf16_to_f32(np.array([BF16_MAX], dtype=np.uint16))[0])
+    assert q[5, 384 + 77] == 0x7E and q[5, 512 + 1] == 0xFE
+    assert s[5, 3] == big / np.float32(448) and s[5, 4] == big / np.float32(448)
+    # a poisoned group dequantises to NaN throughout: the bad activation stays visible
+    deq = oracle.dequantize_block128(q, s)
+    for row, group, _, _ in special:
+        assert np.isnan(deq[row, group * 128:(group + 1) * 128]).all()
+    # torch's library operations on the same rows, NaN spelled one way
+    xb = torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16)
+    tq, ts = _torch_quantize(xb)
+    tq = np.where((tq & 0x7F) == 0x7F, 0x7F, tq).astype(np.uint8)
+    tsb = np.where(np.isnan(ts), 0x7FC00000, ts.view(np.uint32)).astype(np.uint32)
+    np.testing.assert_array_equal(q, tq)
+    np.testing.assert_array_equal(sb, tsb)
+    # the C restatement and the torch twin of the benchmark's CPU baseline
+    c_q, c_s = c_oracle.quantize(bits)
+    np.testing.assert_array_equal(c_q, q)
+    np.testing.assert_array_equal(c_s.view(np.uint32), sb)
+    import a2a_oracle_torch
+    t2q, t2s = a2a_oracle_torch.quantize_block128(xb)
+    np.testing.assert_array_equal(t2q.numpy(), q)
+    np.testing.assert_array_equal(t2s.numpy().view(np.uint32), sb)
+
+
 def test_dequantised_value_is_within_half_a_grid_step():
     rd = make_rank(C2, 0, 64)                                # 1 % outliers x50 stress the scales
     x = oracle.bf16_to_f32(bf16_codes(rd.x))

@@ -71,6 +71,25 @@ def test_source_order_known_answers(world, node, rank, expected):
     assert sorted(expected) == list(range(world))
 
 
+@pytest.mark.parametrize("world,node,dp,rank,expected", [
+    # Worked by hand through the three loops of a2a_worker.rs:681-694 (groups, not ranks, are visited).
+    # 2 nodes of 4 ranks, groups of 2: rank 5 is on node 1 in group 2; node 0's groups 0, 1 first,
+    # then the other group of its node (3), then its own.
+    (8, 4, 2, 5, [0, 1, 3, 2]),
+    (8, 4, 2, 2, [2, 3, 0, 1]),
+    # one node, four groups of two: rank 2 is in group 1; the groups after it, wrapping, then its own
+    (8, 8, 2, 2, [2, 3, 0, 1]),
+    # a group is a whole node: only the other node's group, then the own
+    (8, 4, 4, 6, [0, 1]),
+    # three nodes: nodes 1 and 2 in turn, then the node neighbour, then the own group
+    (12, 4, 2, 1, [2, 3, 4, 5, 1, 0]),
+    (12, 4, 2, 10, [0, 1, 2, 3, 4, 5]),
+])
+def test_source_order_known_answers_with_dp_groups(world, node, dp, rank, expected):
+    assert oracle.source_order(rank, world, node, dp) == expected
+    assert sorted(expected) == list(range(world // dp))
+
+
 @pytest.mark.parametrize("N,E,node,pad,maxpriv", [(4, 32, 4, 1, 3), (4, 32, 2, 4, 0), (8, 64, 4, 16, 5),
                                                   (2, 16, 2, 1, 8), (3, 10, 3, 2, 1)])
 def test_receiver_layout_invariants_and_closed_form(N, E, node, pad, maxpriv):

@@ -168,3 +168,108 @@ def test_static_dispatch_can_be_captured_in_a_hip_graph():
         graph.replay()
         assert_dispatch_equal(case, b.result(), want)
         del scratch
+
+
+def _raw_step(N, H, Hs, K, E, Le, tokens, rows, *, in_elemsize, seed, dp_size=1, scale_transposed=False):
+    """Inputs and sentinel-filled outputs of one step without quantisation (rows travel as bytes,
+    scales are the caller's): returns (keep-alive list, args, output tensors)."""
+    keep, args, outs = [], [], []
+    for r in range(N):
+        g = r // dp_size                                     # the members of a dp group pass the same tokens
+        gg = torch.Generator().manual_seed(seed + 31 * g)
+        T = tokens[g]
+        x = torch.randn((T, H), generator=gg).to(torch.bfloat16 if in_elemsize == 2 else torch.float32).to(DEV)
+        idx = torch.rand((T, E), generator=gg).topk(K, dim=-1).indices.to(torch.int32).to(DEV)
+        xs = None
+        if Hs:
+            xs = torch.randn((Hs, T) if scale_transposed else (T, Hs), generator=gg).to(DEV)
+        n = torch.full((Le,), -1, dtype=torch.int32, device=DEV)
+        ox = torch.full((rows, H * in_elemsize), SENTINEL, dtype=torch.uint8, device=DEV)
+        os_ = torch.full((rows, max(Hs, 1)), -7.0, dtype=torch.float32, device=DEV)
+        keep.append((x, idx, xs))
+        outs.append((n, ox, os_))
+        args.append(native.A2ADispatchArgs(
+            num_tokens=T, x_ptr=x.data_ptr() if T else None, x_stride=H * in_elemsize,
+            x_scale_ptr=xs.data_ptr() if Hs and T else None,
+            x_scale_stride_elem=(T if scale_transposed else 1) if Hs else 0,
+            x_scale_stride_token=(1 if scale_transposed else Hs) if Hs else 0,
+            indices=idx.data_ptr() if T else None, indices_stride=K, weights=None, weights_stride=K, bound_m=None,
+            out_num_tokens=n.data_ptr(), out_x=ox.data_ptr(), out_x_stride=H * in_elemsize, out_x_rows=rows,
+            out_x_scale=os_.data_ptr() if Hs else None, out_x_scale_stride_elem=1 if Hs else 0,
+            out_x_scale_stride_token=Hs))
+    return keep, args, outs
+
+
+@pytest.mark.parametrize("name,N,node,dp,H,Hs,in_elemsize,steps", [
+    # rows that travel as bytes with the caller's scales (the x_scale copy of the kernels), scales transposed
+    ("bf16_with_scales", 4, 4, 1, 384, 3, 2, [[300, 0, 41, 299], [5, 6, 0, 1], [0, 1400, 0, 0]]),
+    # dp groups of two on two nodes of two: the on-device source order and the masks of the sources laid
+    # out earlier are only computed by this entry point's own prepare kernel
+    ("dp2_two_nodes", 4, 2, 2, 256, 0, 4, [[700, 650], [3, 9], [1300, 0]]),
+    ("dp2_three_nodes", 12, 4, 2, 128, 0, 2, [[40, 0, 33, 1, 60, 17], [600, 580, 0, 640, 1, 333]]),
+], ids=lambda v: v if isinstance(v, str) else None)
+def test_static_dispatch_without_quantisation_and_with_dp_groups(name, N, node, dp, H, Hs, in_elemsize, steps):
+    """Byte for byte what a2a_dispatch on a context writes (that path is checked against the oracle by
+    the reference-matrix and dp-group tests), over consecutive steps of different sizes."""
+    E, K, pad = 24, 3, 2
+    Le = -(-E // N)
+    max_tokens = max(max(s) for s in steps)
+    stream = torch.cuda.current_stream(DEV).cuda_stream
+    common = dict(hidden_dim=H, hidden_dim_scale=Hs, in_elemsize=in_elemsize, out_elemsize=2,
+                  scale_elemsize=4 if Hs else 0, max_num_tokens=max_tokens, max_recv_tokens=max_tokens * K * N,
+                  max_private_tokens=0, num_experts=E, expert_padding=pad, num_experts_per_token=K, dp_size=dp,
+                  node_size=node, world_size=N, device=0)
+    cfg = native.A2AConfig(struct_size=ctypes.sizeof(native.A2AConfig), out_dtype=native.SCALAR_TYPE[torch.bfloat16],
+                           flags=0, **common)
+    ctx = native.AllToAllContext.create(out_dtype=torch.bfloat16, **common)
+    flags = torch.zeros(1, dtype=torch.int32, device=DEV)
+    try:
+        for i, tokens in enumerate(steps):
+            print(f"{name} step {i}: tokens per group={tokens}", flush=True)
+            rows = max(sum(tokens) * K + pad * Le, 1)
+            ka, a, out_a = _raw_step(N, H, Hs, K, E, Le, tokens, rows, in_elemsize=in_elemsize, seed=70 + i,
+                                     dp_size=dp, scale_transposed=True)
+            kb, b, out_b = _raw_step(N, H, Hs, K, E, Le, tokens, rows, in_elemsize=in_elemsize, seed=70 + i,
+                                     dp_size=dp, scale_transposed=True)
+            ctx.dispatch(a, False, stream)
+            assert ctx.status(stream) == 0
+            native.dispatch_static(cfg, b, False, flags.data_ptr(), stream)
+            torch.cuda.synchronize(DEV)
+            assert int(flags.item()) == 0
+            wrote = 0
+            for r in range(N):
+                for ta, tb in zip(out_a[r], out_b[r]):
+                    assert torch.equal(ta.view(torch.uint8), tb.view(torch.uint8)), f"rank {r}"
+                wrote += int((out_a[r][0].clamp_min(0)).sum().item())
+            assert wrote == sum(tokens) * K                    # every copy arrived: nothing compared is vacuous
+            del ka, kb
+    finally:
+        ctx.destroy()
+
+
+def test_static_dispatch_refusals_enqueue_nothing():
+    """Steps whose tables do not fit the fixed array, more tokens than max_num_tokens, and flags are refused
+    on the host with the status and a text that names the sizes; a refused call records no node when a
+    stream is being captured (the C++ self-test counts the nodes of such a graph)."""
+    case = Case("static_refusals", 16, 256, 256, 8, 8, 9400)
+    world = [make_rank(case, r, 16) for r in range(8)]
+    b = _Buffers(case, world, 256)
+    stream = torch.cuda.current_stream(DEV).cuda_stream
+    big = _config(case, 40000)                                   # 8 ranks x 40000 tokens x 8 routes: tables beyond 8 MiB
+    args = list(b.args)
+    args[0] = native.A2ADispatchArgs.from_buffer_copy(args[0])
+    args[0].num_tokens = 40000
+    with pytest.raises(RuntimeError, match="bytes of routing tables"):
+        native.dispatch_static(big, args, True, None, stream)
+    with pytest.raises(RuntimeError, match="exceeds maximum"):
+        native.dispatch_static(_config(case, 16), args, True, None, stream)
+    flagged = _config(case, 16)
+    flagged.flags = native.FLAG_SEPARATE_ROUTING
+    with pytest.raises(RuntimeError, match="takes no flags"):
+        native.dispatch_static(flagged, b.args, True, None, stream)
+    # the refused calls left the outputs alone, and the same buffers still take an accepted call
+    torch.cuda.synchronize(DEV)
+    assert all((t == SENTINEL).all() for t in b.x)
+    native.dispatch_static(_config(case, 16), b.args, True, None, stream)
+    want = _oracle(case, world, 256)
+    assert_dispatch_equal(case, b.result(), want)
