@@ -156,6 +156,10 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens,
  * sends of this step routed to `rank` and copies them into out_x / out_x_scale;
  * writes the per-local-expert counts.  `out_x_rows` (rows of out_x) is an
  * addition: copies that would land beyond it are dropped and flagged.
+ * The first recv of a step also enqueues, in front of its own copy, the layout
+ * of EVERY receiver (once per step, as the reference's worker runs once per
+ * rank and step): the recvs of the other ranks must be ordered after it, as
+ * they must be ordered after the sends (same stream, or events).
  */
 int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens,
                       void *out_x, size_t out_x_stride, size_t out_x_rows,

@@ -1032,7 +1032,6 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
     StageRecvArgs rv;
     memset(&rv, 0, sizeof rv);
     rv.rank = rank;
-    rv.valid_mask = ctx->sent_mask & ~ctx->empty_mask;
     rv.dst.out_x = static_cast<uint8_t *>(out_x);
     rv.dst.out_scale = out_x_scale;
     rv.dst.out_stride = out_x_stride;
@@ -1043,8 +1042,11 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
     rv.row_bytes = (uint32_t)row_bytes_of(c);
     rv.hidden_dim_scale = c.hidden_dim_scale;
     rv.max_rows = rows_upper_bound(ctx);
+    // The first recv of a step lays out every receiver: once per step, as the reference's host
+    // worker does (a2a_worker.rs:526-703), not once per recv launch.
+    rv.valid_mask = ctx->sent_mask & ~ctx->empty_mask;
     rv.max_private = c.max_private_tokens;
-    hipError_t e = launch_stage_recv(rv, ctx->ws, ctx->staging, s);
+    const hipError_t e = launch_stage_recv(rv, ctx->ws, ctx->staging, !ctx->recv_seen, s);
     if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_recv");
     ctx->recv_seen = true;
     ctx->staging.recv_mask |= 1u << rank;

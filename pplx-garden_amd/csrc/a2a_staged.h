@@ -32,6 +32,7 @@ struct Staging {
     uint32_t *source_position = nullptr; // [N][max_recv]
     uint32_t *source_dispatch_offset = nullptr;  // [N][max_recv]  a2a_worker.rs:636-656
     uint32_t *combine_send_offset = nullptr;     // [N][max_recv]  a2a_worker.rs:659-667
+    uint32_t *source_row = nullptr;      // [N][max_recv]: staged row a received row is copied from (sender * max_tokens + token)
     uint32_t *num_recv = nullptr;        // [N][2]: received rows, rows from other nodes
     size_t disp_stride = 0;
     size_t comb_stride = 0;
@@ -56,12 +57,15 @@ struct StageRecvArgs {
     PushDst dst;
     int32_t *out_num_tokens;  // rows per local expert for the caller, may be null
     uint32_t rank;
-    uint32_t valid_mask;
     uint32_t row_bytes;
     uint32_t hidden_dim_scale;
     uint32_t max_rows;        // upper bound of received rows known to the host
     uint32_t team_waves;      // wavefronts that share a row (set by the launcher)
+    // the first recv of a step only: it lays out every receiver
+    uint32_t valid_mask;      // sources that sent tokens in this step (the others count as empty)
     uint32_t max_private;     // rows per source in the private part of a receive region (a2a_worker.rs:646-656)
+    uint32_t copy_blocks;     // workgroups that serve the caller's rank; the others lay out the other receivers (launcher)
+    uint32_t slices;          // workgroups per other receiver (set by the launcher)
 };
 
 struct CombineSendArgs {
@@ -96,7 +100,8 @@ hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &w
 // The send of a large step after launch_route_accumulate(..., for_send = true).
 hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                                      bool quantize, hipStream_t stream);
-hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st,
+// `first_of_step`: no recv has run since the step's sends; this launch also lays out the other receivers.
+hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st, bool first_of_step,
                              hipStream_t stream);
 hipError_t launch_combine_send(const CombineSendArgs &args, const Workspace &ws, const Staging &st,
                                hipStream_t stream);

@@ -365,47 +365,72 @@ __device__ __forceinline__ void copy_row_by_team(const u32x4 *src, u32x4 *dst, u
 #pragma unroll
         for (uint32_t u = 0; u < 8; ++u) {
             const uint32_t c = c0 + u * team + member;
-            if (c < num_chunks) __builtin_nontemporal_store(v[u], dst + c);
+            if (c < num_chunks) dst[c] = v[u];
         }
     }
 }
 
 // ---------------------------------------------------------------------------
-// dispatch recv, one launch.  Every workgroup first lays out the receiver from
-// the published per-source counts of its experts (what the reference's host
-// worker does, a2a_worker.rs:577-606,621-694): rows per expert, padded first
-// row of every expert, first row of every (source, expert) run inside it, and
-// the order in which the runs ARRIVE (sources in the worker's order, experts
-// inside a source).  Two wavefronts of a workgroup do that, each by itself;
-// a workgroup that has no row leaves before.  Workgroup 0 publishes those
-// tables.  Then the workgroups
-// share the received rows between them, one team of wavefronts per row: its metadata (padded_index,
-// source_rank, source position: a2a_worker.rs:636-671) is written and payload
-// and scales are copied from the sender's staged token
-// (a2a_dispatch_recv.cu:139-155).
+// dispatch recv.  The receivers of a step are laid out ONCE per step, by the
+// launch of the step's first recv (the reference's host worker runs
+// process_routing_info once per rank and step, a2a_worker.rs:526-703).
 //
-// Dynamic LDS: 4 * G * Le + 1 + 3 * G words.
+// stage_recv_first_kernel is that launch.  Its first workgroups serve the rank
+// that called: each lays the receiver out in LDS from the published per-source
+// counts of its experts (a2a_worker.rs:577-606,621-694: rows per expert, padded
+// first row of every expert, first row of every (source, expert) run inside it,
+// and the order in which the runs ARRIVE: sources in the worker's order,
+// experts inside a source), then teams of wavefronts share the received rows:
+// the row's metadata is written (padded_index, source_rank, source position and
+// the two offset tables: a2a_worker.rs:636-671) and payload and scales are
+// copied from the sender's staged token (a2a_dispatch_recv.cu:139-155).  A rank
+// on a GPU of its own would launch only these.  The workgroups behind them lay
+// out the OTHER receivers, in the shadow of that copy: the same layout in LDS,
+// then one thread per received row writes the row's metadata and the staged row
+// it comes from (the token behind its position in the sender's order).
+//
+// stage_recv_kernel is the launch of every later recv of the step.  It only
+// copies: a team of wavefronts per received row reads where the row comes from
+// and where it goes (one trip for both) and moves payload and scales; its first
+// workgroup hands the receiver's counts to the caller.
+//
+// Dynamic LDS of a layout: 4 * G * Le + 1 + 3 * G words.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs args, const Workspace ws,
-                                                          const Staging st) {
-    extern __shared__ uint32_t s_recv[];
-    __shared__ uint8_t s_order[kMaxWorld];
+struct ReceiverTables {   // in LDS, see lay_out_receiver
+    uint32_t *tot;       // [g][le]  copies source g sends to local expert le
+    uint32_t *excl;      // [g][le]  position of the run in the sender's expert-sorted order
+    uint32_t *run_row;   // [i][le]  first row of the run in the receiver's buffer (i = order index)
+    uint32_t *seg;       // [i][le]  first ARRIVAL index of the run; seg[items] = rows received
+    uint32_t *grp_dst;   // [g]      position of source g's first row for this receiver in g's send order
+    uint32_t *grp_src;   // [g]      rows this receiver gets from the sources numbered below g
+    uint32_t *grp_cnt;   // [g]      rows this receiver gets from source g
+    const uint8_t *order;  // [i]    the i-th source this receiver lays out
+    uint32_t rows;       // rows received
+};
+
+// Lays out receiver `r` in LDS.  Whole workgroup.  `publish`: this workgroup also writes the
+// receiver's tables to memory and (if given) its counts to the caller.  Returns false, before the
+// expensive part, when the workgroup's first row `first_row` lies beyond the rows received and it
+// does not publish: the host sizes grids for an upper bound, a receiver typically gets 1/N of it.
+__device__ __forceinline__ bool lay_out_receiver(uint32_t valid_mask, const Workspace &ws, const Staging &st, uint32_t r,
+                                                 bool publish, uint32_t first_row, int32_t *out_num_tokens,
+                                                 uint32_t out_rows, uint32_t *s_recv, uint8_t *s_order,
+                                                 ReceiverTables &t) {
     const uint32_t G = ws.num_groups, E = ws.num_experts, Le = ws.experts_per_rank;
-    const uint32_t r = args.rank;
     const uint32_t first = r * Le;
     const uint32_t n_local = first >= E ? 0 : (E - first < Le ? E - first : Le);
     const uint32_t items = G * Le;
     const uint32_t tid = threadIdx.x;
     const uint32_t nthreads = blockDim.x;
     const uint32_t lane = tid & (kWave - 1);
-    const bool publish = blockIdx.x == 0;
-    uint32_t *tot = s_recv;              // [g][le]  copies source g sends to local expert le
-    uint32_t *excl = tot + items;        // [g][le]  position of the run in the sender's expert-sorted order
-    uint32_t *run_row = excl + items;    // [i][le]  first row of the run in the receiver's buffer (i = order index)
-    uint32_t *seg = run_row + items;     // [i][le]  first ARRIVAL index of the run; seg[items] = rows received
-    uint32_t *grp_dst = seg + items + 1; // [g]      position of source g's first row for this receiver in g's send order
-    uint32_t *grp_src = grp_dst + G;     // [g]      rows this receiver gets from the sources numbered below g
-    uint32_t *grp_cnt = grp_src + G;     // [g]      rows this receiver gets from source g
+    uint32_t *tot = t.tot = s_recv;
+    uint32_t *excl = t.excl = tot + items;
+    uint32_t *run_row = t.run_row = excl + items;
+    uint32_t *seg = t.seg = run_row + items;
+    uint32_t *grp_dst = t.grp_dst = seg + items + 1;
+    uint32_t *grp_src = t.grp_src = grp_dst + G;
+    uint32_t *grp_cnt = t.grp_cnt = grp_src + G;
+    t.order = s_order;
 
     // The order in which this receiver lays out its sources (one byte per source, from the table the
     // context computed once) travels with the counts and is read from LDS from then on: looked up in
@@ -415,26 +440,22 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
         const uint32_t g = Le > 1 ? __umulhi(w, ws.le_magic) : w;
         const uint32_t le = w - g * Le;
         const uint32_t e = first + le;
-        const bool live = le < n_local && (args.valid_mask >> g & 1);
+        const bool live = le < n_local && (valid_mask >> g & 1);
         tot[w] = live ? ws.num_routed[g * E + e] : 0;
         excl[w] = live && e > 0 ? ws.expert_offsets[g * E + e - 1] : 0;
     }
     __syncthreads();
 
     // Rows this receiver gets from source g (lane g; there are at most kMaxWorld <= 64 sources): the
-    // sender's scan over its experts gives them without a sum.  Every wavefront adds them up by itself,
-    // and a workgroup whose first row lies beyond the rows received leaves here: the host sizes the
-    // grid for an upper bound, a receiver typically gets 1/N of it, and the layout below is the
-    // expensive part of a workgroup without rows.
+    // sender's scan over its experts gives them without a sum.  Every wavefront adds them up by itself.
     uint32_t from_source = 0;
     if (lane < G && n_local != 0) {
         const uint32_t last = lane * Le + n_local - 1;
         from_source = excl[last] + tot[last] - excl[lane * Le];
     }
     const uint32_t from_lower = wave_inclusive_scan(from_source, lane);   // inclusive over the sources
-    const uint32_t rows = (uint32_t)__builtin_amdgcn_readlane((int)from_lower, kWave - 1);
-    const uint32_t team_threads = args.team_waves * kWave;
-    if (!publish && blockIdx.x * (nthreads / team_threads) >= rows) return;   // uniform
+    const uint32_t rows = t.rows = (uint32_t)__builtin_amdgcn_readlane((int)from_lower, kWave - 1);
+    if (!publish && first_row >= rows) return false;   // uniform
 
     // The layout is the work of two wavefronts, each by itself (scans on the DPP path, no barrier
     // inside); the others wait for them.  Done by every wavefront of every workgroup, with workgroup
@@ -482,8 +503,8 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
                 if (publish) {
                     ws.tokens_per_expert[e] = tpe;
                     ws.padded_offset[e] = poff;
-                    if (args.out_num_tokens != nullptr) args.out_num_tokens[le] = (int32_t)tpe;
-                    if (poff + tpe > args.dst.out_rows) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+                    if (out_num_tokens != nullptr) out_num_tokens[le] = (int32_t)tpe;
+                    if (poff + tpe > out_rows) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
                 }
             }
             carry += (uint32_t)__builtin_amdgcn_readlane((int)scan, kWave - 1);
@@ -518,81 +539,225 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
         }
     }
     __syncthreads();
-    const uint32_t total = rows;
     if (publish && tid == 0) {
         // rows that come from other nodes (num_efa_tokens, a2a_worker.rs:681-687)
         const uint32_t remote_segs = (ws.world / ws.node_size - 1) * (ws.node_size / ws.dp_size) * Le;
-        st.num_recv[2 * r + 1] = remote_segs < items ? seg[remote_segs] : total;
+        st.num_recv[2 * r + 1] = remote_segs < items ? seg[remote_segs] : rows;
+    }
+    return true;
+}
+
+// What the receiver's tables say of arrival `row` of run `s` (seg[s] <= row < seg[s + 1]).
+struct RowMeta {
+    uint32_t g;        // source (dp group)
+    uint32_t pos;      // position in the source's expert-sorted order
+    uint32_t dst_row;  // row in the receiver's buffer
+};
+
+__device__ __forceinline__ RowMeta row_of_run(const ReceiverTables &t, const Workspace &ws, uint32_t s, uint32_t row) {
+    const uint32_t Le = ws.experts_per_rank;
+    const uint32_t i = Le > 1 ? __umulhi(s, ws.le_magic) : s;
+    const uint32_t le = s - i * Le;
+    RowMeta m;
+    m.g = t.order[i];
+    const uint32_t j = row - t.seg[s];
+    m.pos = t.excl[m.g * Le + le] + j;
+    m.dst_row = t.run_row[s] + j;
+    return m;
+}
+
+// Writes the five per-row tables of the reference's host worker for arrival `row` of receiver `r`
+// (a2a_worker.rs:633-671).  One thread.
+__device__ __forceinline__ void write_row_tables(const ReceiverTables &t, const Workspace &ws, const Staging &st,
+                                                 uint32_t r, uint32_t row, const RowMeta &m, uint32_t max_private) {
+    const uint32_t G = ws.num_groups;
+    const size_t at = (size_t)r * st.max_recv + row;
+    st.padded_index[at] = m.dst_row;
+    // the member of the group that sends to this rank (a2a_worker.rs:633)
+    const uint32_t peer = m.g * ws.dp_size + r % ws.dp_size;
+    st.source_rank[at] = peer;
+    st.source_position[at] = m.pos;
+    // How the reference addresses the row on its way in and on its way back (a2a_worker.rs:636-667).
+    // Nothing here reads these two: they are what a rank on a GPU of its own would consume.
+    const uint32_t index_on_rank = m.pos - t.grp_dst[m.g];     // rows of this source before this one
+    const bool same_node = peer / ws.node_size == r / ws.node_size;
+    uint32_t sdo = m.pos, cso = m.pos;                         // own rows: the sender's position
+    if (peer != r) {
+        if (index_on_rank < max_private) {
+            sdo = max_private * m.g + index_on_rank;                               // private region
+        } else if (same_node) {
+            sdo = m.pos | 0x80000000u;                                             // read from the peer's send buffer
+        } else {
+            sdo = t.grp_src[m.g] + index_on_rank + max_private * (G - 1);          // overflow region
+        }
+    }
+    if ((peer != r || ws.dp_size > 1) && !same_node) cso = t.grp_src[m.g] + index_on_rank;
+    st.source_dispatch_offset[at] = sdo;
+    st.combine_send_offset[at] = cso;
+}
+
+__global__ __launch_bounds__(1024) void stage_recv_first_kernel(const StageRecvArgs args, const Workspace ws,
+                                                                const Staging st) {
+    extern __shared__ uint32_t s_recv[];
+    __shared__ uint8_t s_order[kMaxWorld];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nthreads = blockDim.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t items = ws.num_groups * ws.experts_per_rank;
+    ReceiverTables t;
+
+    if (blockIdx.x >= args.copy_blocks) {
+        // ---- one of the other receivers: layout, then one thread per received row ----
+        const uint32_t w = blockIdx.x - args.copy_blocks;
+        uint32_t r = w / args.slices;
+        const uint32_t slice = w - r * args.slices;
+        if (r >= args.rank) ++r;   // the caller's rank is served by the first workgroups
+        if (!lay_out_receiver(args.valid_mask, ws, st, r, slice == 0, slice * nthreads, nullptr, 0xFFFFFFFFu, s_recv,
+                              s_order, t))
+            return;
+        const uint32_t total = t.rows < st.max_recv ? t.rows : st.max_recv;   // beyond: flagged and dropped
+        for (uint32_t row = slice * nthreads + tid; row < total; row += args.slices * nthreads) {
+            // the run this arrival belongs to: the last one with seg[s] <= row (runs without rows share
+            // their first arrival with the run after them, so the last such run is the one with rows)
+            uint32_t lo = 0, hi = items;   // seg[lo] <= row < seg[hi]
+            while (hi - lo > 1) {
+                const uint32_t mid = (lo + hi) / 2;
+                if (t.seg[mid] <= row) lo = mid; else hi = mid;
+            }
+            const RowMeta m = row_of_run(t, ws, lo, row);
+            // the token behind the position: asked for first, used last
+            const uint32_t token = m.pos < ws.max_tk ? st.pos_token[(size_t)m.g * ws.max_tk + m.pos] : 0;
+            write_row_tables(t, ws, st, r, row, m, args.max_private);
+            st.source_row[(size_t)r * st.max_recv + row] = m.g * st.max_tokens + token;
+        }
+        return;
     }
 
-    // From here on the workgroup is split into teams of args.team_waves
-    // wavefronts that work alone (no barrier): one received row per team at a
-    // time.  Every wavefront of a team finds the row's run by itself.
+    // ---- the caller's rank: layout, then a team of wavefronts per received row ----
+    const uint32_t r = args.rank;
+    const uint32_t team_threads = args.team_waves * kWave;
+    const uint32_t teams = nthreads / team_threads;
+    if (!lay_out_receiver(args.valid_mask, ws, st, r, blockIdx.x == 0, blockIdx.x * teams, args.out_num_tokens,
+                          args.dst.out_rows, s_recv, s_order, t))
+        return;
+    // From here on the workgroup is split into teams that work alone (no barrier): one received row
+    // per team at a time.  Every wavefront of a team finds the row's run by itself.
     const PushDst &dst = args.dst;
     const uint32_t num_chunks = args.row_bytes / 16;
-    const uint32_t team = team_threads;
-    const uint32_t teams = nthreads / team;
-    const uint32_t member = tid % team;
-    for (uint32_t row = blockIdx.x * teams + tid / team; row < total; row += gridDim.x * teams) {
+    const uint32_t member = tid % team_threads;
+    for (uint32_t row = blockIdx.x * teams + tid / team_threads; row < t.rows; row += args.copy_blocks * teams) {
         // the run this arrival belongs to: the one non-empty run with seg[s] <= row < seg[s + 1]
         uint32_t s = 0;
         for (uint32_t s0 = 0; s0 < items; s0 += kWave) {
             const uint32_t cand = s0 + lane;
-            const uint64_t hit = __ballot(cand < items && seg[cand] <= row && row < seg[cand + 1]);
+            const uint64_t hit = __ballot(cand < items && t.seg[cand] <= row && row < t.seg[cand + 1]);
             if (hit != 0) {
                 s = s0 + (uint32_t)__builtin_ctzll(hit);
                 break;
             }
         }
-        const uint32_t i = Le > 1 ? __umulhi(s, ws.le_magic) : s;
-        const uint32_t le = s - i * Le;
-        const uint32_t g = s_order[i];
-        const uint32_t j = row - seg[s];
-        const uint32_t pos = excl[g * Le + le] + j;
-        const uint32_t dst_row = run_row[s] + j;
-        if (row >= st.max_recv) continue;   // flagged above: more rows than the receive region was sized for
+        const RowMeta m = row_of_run(t, ws, s, row);
+        if (row >= st.max_recv) continue;   // flagged by the layout: more rows than the receive region was sized for
+        const uint32_t token = st.pos_token[(size_t)m.g * ws.max_tk + m.pos];
         if (member == 0) {
-            st.padded_index[(size_t)r * st.max_recv + row] = dst_row;
-            // the member of the group that sends to this rank (a2a_worker.rs:633)
-            st.source_rank[(size_t)r * st.max_recv + row] = g * ws.dp_size + r % ws.dp_size;
-            st.source_position[(size_t)r * st.max_recv + row] = pos;
-            // How the reference addresses the row on its way in and on its way back
-            // (a2a_worker.rs:636-667).  Nothing here reads these two: they are what a rank on a
-            // GPU of its own would consume.
-            const uint32_t peer = g * ws.dp_size + r % ws.dp_size;
-            const uint32_t index_on_rank = pos - grp_dst[g];       // rows of this source before this one
-            const bool same_node = peer / ws.node_size == r / ws.node_size;
-            uint32_t sdo = pos, cso = pos;                         // own rows: the sender's position
-            if (peer != r) {
-                if (index_on_rank < args.max_private) {
-                    sdo = args.max_private * g + index_on_rank;                        // private region
-                } else if (same_node) {
-                    sdo = pos | 0x80000000u;                                           // read from the peer's send buffer
-                } else {
-                    sdo = grp_src[g] + index_on_rank + args.max_private * (G - 1);     // overflow region
-                }
-            }
-            if ((peer != r || ws.dp_size > 1) && !same_node) cso = grp_src[g] + index_on_rank;
-            st.source_dispatch_offset[(size_t)r * st.max_recv + row] = sdo;
-            st.combine_send_offset[(size_t)r * st.max_recv + row] = cso;
+            write_row_tables(t, ws, st, r, row, m, args.max_private);
+            st.source_row[(size_t)r * st.max_recv + row] = m.g * st.max_tokens + token;
         }
         if (dst.out_x == nullptr) continue;
-        if (dst_row >= dst.out_rows) {
+        if (m.dst_row >= dst.out_rows) {
             if (member == 0) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
             continue;
         }
-        const uint32_t token = st.pos_token[(size_t)g * ws.max_tk + pos];
-        const uint8_t *src = st.send_buf + ((size_t)g * st.max_tokens + token) * st.disp_stride;
+        const uint8_t *src = st.send_buf + ((size_t)m.g * st.max_tokens + token) * st.disp_stride;
         copy_row_by_team(reinterpret_cast<const u32x4 *>(src),
-                         reinterpret_cast<u32x4 *>(dst.out_x + (size_t)dst_row * dst.out_stride), num_chunks, member,
-                         team);
+                         reinterpret_cast<u32x4 *>(dst.out_x + (size_t)m.dst_row * dst.out_stride), num_chunks, member,
+                         team_threads);
         if (dst.out_scale != nullptr) {
             const float *ss = reinterpret_cast<const float *>(src + st.payload_bytes);
-            float *os = dst.out_scale + (size_t)dst_row * dst.os_stride_token;
-            for (uint32_t q = member; q < args.hidden_dim_scale; q += team) {
+            float *os = dst.out_scale + (size_t)m.dst_row * dst.os_stride_token;
+            for (uint32_t q = member; q < args.hidden_dim_scale; q += team_threads) {
                 os[(size_t)q * dst.os_stride_elem] = ss[q];
             }
         }
+    }
+}
+
+__global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs args, const Workspace ws,
+                                                          const Staging st) {
+    // everything a wavefront takes from the argument block, asked for in one go
+    A2A_PIN(args.dst.out_x);
+    A2A_PIN(args.dst.out_scale);
+    A2A_PIN(args.dst.out_stride);
+    A2A_PIN(args.dst.os_stride_elem);
+    A2A_PIN(args.dst.os_stride_token);
+    A2A_PIN(args.dst.out_rows);
+    A2A_PIN(args.rank);
+    A2A_PIN(args.row_bytes);
+    A2A_PIN(args.hidden_dim_scale);
+    A2A_PIN(args.team_waves);
+    A2A_PIN(st.send_buf);
+    A2A_PIN(st.padded_index);
+    A2A_PIN(st.source_row);
+    A2A_PIN(st.num_recv);
+    A2A_PIN(st.disp_stride);
+    A2A_PIN(st.payload_bytes);
+    A2A_PIN(st.max_recv);
+    const uint32_t r = args.rank;
+    const uint32_t tid = threadIdx.x;
+    const PushDst &dst = args.dst;
+    const uint32_t num_chunks = args.row_bytes / 16;
+    const uint32_t team = args.team_waves * kWave;   // threads that share a row
+    const uint32_t teams = blockDim.x / team;
+    const uint32_t member = tid % team;
+    const uint32_t *padded_index = st.padded_index + (size_t)r * st.max_recv;
+    const uint32_t *source_row = st.source_row + (size_t)r * st.max_recv;
+    // The first row's two table words are asked for together with the number of rows received
+    // (a row index the tables do not hold reads entry 0 and is dropped by the loop's bound).
+    uint32_t row = blockIdx.x * teams + tid / team;
+    const uint32_t probe = row < st.max_recv ? row : 0;
+    uint32_t dst_row = padded_index[probe];
+    uint32_t from = source_row[probe];
+    uint32_t total = st.num_recv[2 * r];
+    if (total > st.max_recv) total = st.max_recv;   // flagged by the layout: more rows than the region was sized for
+
+    if (blockIdx.x == 0) {
+        // the receiver's counts for the caller (a2a_dispatch_recv.cu:220-224)
+        const uint32_t E = ws.num_experts, Le = ws.experts_per_rank;
+        const uint32_t first = r * Le;
+        const uint32_t n_local = first >= E ? 0 : (E - first < Le ? E - first : Le);
+        for (uint32_t le = tid; le < n_local; le += blockDim.x) {
+            const uint32_t tpe = ws.tokens_per_expert[first + le];
+            if (args.out_num_tokens != nullptr) args.out_num_tokens[le] = (int32_t)tpe;
+            if (ws.padded_offset[first + le] + tpe > dst.out_rows) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+        }
+    }
+    if (dst.out_x == nullptr) return;
+
+    const uint32_t stride = gridDim.x * teams;
+    while (row < total) {
+        // the next row's words travel while this one is copied
+        const uint32_t next = row + stride;
+        const uint32_t next_probe = next < total ? next : row;
+        const uint32_t next_dst = padded_index[next_probe];
+        const uint32_t next_from = source_row[next_probe];
+        if (dst_row >= dst.out_rows) {
+            if (member == 0) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+        } else {
+            const uint8_t *src = st.send_buf + (size_t)from * st.disp_stride;
+            copy_row_by_team(reinterpret_cast<const u32x4 *>(src),
+                             reinterpret_cast<u32x4 *>(dst.out_x + (size_t)dst_row * dst.out_stride), num_chunks,
+                             member, team);
+            if (dst.out_scale != nullptr) {
+                const float *ss = reinterpret_cast<const float *>(src + st.payload_bytes);
+                float *os = dst.out_scale + (size_t)dst_row * dst.os_stride_token;
+                for (uint32_t q = member; q < args.hidden_dim_scale; q += team) {
+                    os[(size_t)q * dst.os_stride_elem] = ss[q];
+                }
+            }
+        }
+        row = next;
+        dst_row = next_dst;
+        from = next_from;
     }
 }
 
@@ -698,6 +863,10 @@ int staging_allocate(Staging &st, const a2a_config &cfg, std::string *error) {
         return A2A_ERR_UNSUPPORTED;
     }
     st.max_recv = (uint32_t)max_recv;
+    if (N * cfg.max_num_tokens > 0xFFFFFFFFull) {   // a staged row is named by sender * max_num_tokens + token
+        if (error) *error = "world_size * max_num_tokens too large";
+        return A2A_ERR_UNSUPPORTED;
+    }
 
     size_t off = 0;
     auto carve = [&off](size_t bytes) {
@@ -713,6 +882,7 @@ int staging_allocate(Staging &st, const a2a_config &cfg, std::string *error) {
     const size_t o_spos = carve(N * max_recv * sizeof(uint32_t));
     const size_t o_sdo = carve(N * max_recv * sizeof(uint32_t));
     const size_t o_cso = carve(N * max_recv * sizeof(uint32_t));
+    const size_t o_srow = carve(N * max_recv * sizeof(uint32_t));
     const size_t o_nrecv = carve(N * 2 * sizeof(uint32_t));
     hipError_t e = hipMalloc(&st.arena, off);
     if (e != hipSuccess) {
@@ -731,6 +901,7 @@ int staging_allocate(Staging &st, const a2a_config &cfg, std::string *error) {
     st.source_position = reinterpret_cast<uint32_t *>(base + o_spos);
     st.source_dispatch_offset = reinterpret_cast<uint32_t *>(base + o_sdo);
     st.combine_send_offset = reinterpret_cast<uint32_t *>(base + o_cso);
+    st.source_row = reinterpret_cast<uint32_t *>(base + o_srow);
     st.num_recv = reinterpret_cast<uint32_t *>(base + o_nrecv);
     // Tables are read before they are written only through misuse; start from zero.
     e = hipMemset(base + o_pos, 0, o_comb - o_pos);
@@ -831,14 +1002,26 @@ hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace 
     return hipGetLastError();
 }
 
-hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st,
+hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st, bool first_of_step,
                              hipStream_t stream) {
     RowLaunch l = row_launch(args.max_rows, args.row_bytes / 16);
-    if (l.blocks == 0) l.blocks = 1;    // the layout is published even when nothing was sent
+    if (l.blocks == 0) l.blocks = 1;    // the counts are handed over even when nothing was sent
     StageRecvArgs a = args;
     a.team_waves = l.team_waves;
+    if (!first_of_step) {
+        hipLaunchKernelGGL(stage_recv_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, a, ws, st);
+        return hipGetLastError();
+    }
+    // Behind the caller's workgroups: a few per other receiver, enough threads for the rows a receiver
+    // typically gets (1/N of the host's upper bound); each repeats that receiver's layout in LDS.
+    a.copy_blocks = l.blocks;
+    const uint32_t typical = (args.max_rows + ws.world - 1) / ws.world;
+    a.slices = (typical + l.threads - 1) / l.threads;
+    if (a.slices < 1) a.slices = 1;
+    if (a.slices > 16) a.slices = 16;
+    const uint32_t blocks = l.blocks + (ws.world - 1) * a.slices;
     const size_t lds = (4 * (size_t)ws.num_groups * ws.experts_per_rank + 1 + 3 * (size_t)ws.num_groups) * sizeof(uint32_t);
-    hipLaunchKernelGGL(stage_recv_kernel, dim3(l.blocks), dim3(l.threads), lds, stream, a, ws, st);
+    hipLaunchKernelGGL(stage_recv_first_kernel, dim3(blocks), dim3(l.threads), lds, stream, a, ws, st);
     return hipGetLastError();
 }
 
