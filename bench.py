@@ -387,14 +387,195 @@ def other_shape(case, device, routings: int, steps: int, warmup: int, ctx_flags:
     return out
 
 
+def split_calls(case, device, routings: int, steps: int, warmup: int, label: str):
+    """The four split calls (`a2a_dispatch_send / _recv`, `a2a_combine_send / _recv`: the calls the
+    reference's FFI binds, a2a_context.rs:275-487) at the headline's shape, rank 0 holding the tokens.
+    Rows move twice here (sender -> staging -> receiver, and back), so the bytes are two-hop bytes.
+
+    Three passes: (1) whole steps (the send, every rank's recv, every rank's combine-send, rank 0's
+    combine-recv) in which every kernel records events at its own start and end: the kernels' own
+    durations, per kernel; (2) the same steps between two synchronisations, no events: wall time of the
+    work of the whole group on this GPU; (3) only rank 0's four calls per step, no events: what a rank
+    on a GPU of its own runs (its combine-recv reads the rows the other ranks' combine-sends of the
+    passes before left in the staging buffer)."""
+    import numpy as np
+    import torch
+    from pplx_garden_amd.native import p2p_all_to_all as native
+    from pplx_garden_amd.utils.math import Statistics
+
+    wl = Workload(case, device, routings, native.FLAG_PREALLOC_STAGING)
+    ctx = wl.ctx
+    N, H, Hs, K, T = case.world_size, case.hidden_dim, case.hidden_dim_scale, case.topk, case.num_tokens
+    Le = case.experts_per_rank
+    stream = torch.cuda.current_stream(device).cuda_stream
+    rows_of = []                           # [routing][rank]: rows a rank receives
+    for routing in wl.routings:
+        owner = routing[0].indices.numpy().reshape(-1) // Le
+        rows_of.append(np.bincount(owner, minlength=N)[:N])
+
+    def send(j):
+        ctx.dispatch_send(0, T, wl.x[0].data_ptr(), 2 * H, None, 0, 0, wl.idx[j][0].data_ptr(), K,
+                          wl.w[j][0].data_ptr(), K, None, stream, quantize=True)
+
+    def empty_send(r):
+        ctx.dispatch_send(r, 0, None, 2 * H, None, 0, 0, None, K, None, K, None, stream, quantize=True)
+
+    def recv(r):
+        ctx.dispatch_recv(r, wl.out_n[r].data_ptr(), wl.out_x[r].data_ptr(), H, wl.rows, wl.out_s[r].data_ptr(), 1, Hs,
+                          stream)
+
+    def combine_send(r):
+        ctx.combine_send(r, wl.y[r].data_ptr(), 2 * H, wl.rows, stream)
+
+    def combine_recv(j):
+        ctx.combine_recv(0, T, wl.rows, torch.bfloat16, wl.out_tokens[0].data_ptr(), H, wl.idx[j][0].data_ptr(), K,
+                         wl.w[j][0].data_ptr(), K, None, False, stream)
+
+    def whole_step(i, timed=None):
+        j = i % len(wl.routings)
+
+        def own(which, key):
+            if timed is not None:
+                pair = [torch.cuda.Event(enable_timing=True) for _ in range(2)]
+                for ev in pair:
+                    ev.record()             # an event gets its handle when it is first recorded
+                ctx.time_next_kernel(which, pair[0].cuda_event, pair[1].cuda_event)
+                timed.append((key, j, pair))
+
+        own(native.KERNEL_ROUTE, "route")
+        own(native.KERNEL_STAGE_SEND, "send")
+        send(j)
+        for r in range(1, N):
+            empty_send(r)
+        for r in range(N):
+            own(native.KERNEL_STAGE_RECV, ("recv", r))
+            recv(r)
+        for r in range(N):
+            own(native.KERNEL_COMBINE_SEND, ("combine_send", r))
+            combine_send(r)
+        own(native.KERNEL_GATHER, "combine_recv")
+        combine_recv(j)
+
+    def one_rank_step(i):
+        j = i % len(wl.routings)
+        send(j)
+        recv(0)
+        combine_send(0)
+        combine_recv(j)
+
+    def wall(step_fn, n):
+        for i in range(warmup):
+            step_fn(i)
+        torch.cuda.synchronize(device)
+        t0 = time.perf_counter()
+        for i in range(n):
+            step_fn(warmup + i)
+        torch.cuda.synchronize(device)
+        dt = time.perf_counter() - t0
+        flags = ctx.status(stream)
+        if flags:
+            raise RuntimeError(f"device error flags {flags}")
+        return dt / n * 1e6
+
+    # (1) the kernels' own durations
+    timed = []
+    sample_steps = min(steps, 100)
+    for i in range(min(warmup, 20)):
+        whole_step(i)
+    torch.cuda.synchronize(device)
+    for i in range(sample_steps):
+        whole_step(i, timed)
+    torch.cuda.synchronize(device)
+    if ctx.status(stream):
+        raise RuntimeError("device error flags in the split calls")
+    us = {}
+    for key, j, (a, b) in timed:
+        us.setdefault(key, []).append((a.elapsed_time(b) * 1e3, j))
+    # (2), (3) wall time without events
+    whole_us = wall(whole_step, steps)
+    one_rank_us = wall(one_rank_step, steps)
+    wl.close()
+
+    row_d = H + 4 * Hs                     # a dispatched row: fp8 payload and its float scales
+    row_c = 2 * H                          # a combined row: bf16
+
+    def kernel(name, samples, bytes_of):
+        if not samples:
+            return None
+        t = [x for x, _ in samples]
+        total_bytes = sum(bytes_of(j) for _, j in samples)
+        st = Statistics.create(t)
+        out = {"kernel": name, "avg_us": round(st.mean, 2), "p50_us": round(st.p50, 2), "samples": len(t)}
+        if total_bytes:
+            rate = total_bytes / (sum(t) * 1e-6) / 1e9
+            out.update({"bytes_per_launch": int(total_bytes / len(t)), "achieved_gbs": round(rate, 1),
+                        "frac_of_hbm_peak": round(rate / HBM_PEAK_GBS, 4)})
+        return out
+
+    d_bytes, c_bytes = algorithmic_bytes(T, H, K)
+    later = [x for r in range(1, N) for x in us.get(("recv", r), [])]
+    # bytes of the later recvs: per sample, in the order the samples were taken
+    later_seq = [2 * int(rows_of[j][r]) * row_d for r in range(1, N) for _, j in us.get(("recv", r), [])]
+    csend = [x for r in range(N) for x in us.get(("combine_send", r), [])]
+    csend_seq = [2 * int(rows_of[j][r]) * row_c for r in range(N) for _, j in us.get(("combine_send", r), [])]
+
+    def seq_kernel(name, samples, byte_seq):
+        if not samples:
+            return None
+        t = [x for x, _ in samples]
+        st = Statistics.create(t)
+        rate = sum(byte_seq) / (sum(t) * 1e-6) / 1e9
+        return {"kernel": name, "avg_us": round(st.mean, 2), "p50_us": round(st.p50, 2), "samples": len(t),
+                "bytes_per_launch": int(sum(byte_seq) / len(t)), "achieved_gbs": round(rate, 1),
+                "frac_of_hbm_peak": round(rate / HBM_PEAK_GBS, 4)}
+
+    kernels = {
+        "dispatch_send": [
+            kernel("route_hist_kernel", us.get("route", []), lambda j: 0),
+            kernel("stage_send_resolve_kernel", us.get("send", []), lambda j: T * (2 * H + 4 * K) + T * row_d),
+        ],
+        "dispatch_recv": [
+            kernel("stage_recv_first_kernel", us.get(("recv", 0), []), lambda j: 2 * int(rows_of[j][0]) * row_d),
+            seq_kernel("stage_recv_kernel", later, later_seq),
+        ],
+        "combine_send": [seq_kernel("combine_send_kernel", csend, csend_seq)],
+        "combine_recv": [kernel("combine_gather_kernel", us.get("combine_recv", []), lambda j: c_bytes)],
+    }
+    one_rank_kernels = sum(k["avg_us"] for k in (kernels["dispatch_send"] + kernels["dispatch_recv"][:1]
+                                                 + kernels["combine_send"] + kernels["combine_recv"]) if k)
+    return {
+        "workload": label,
+        "one_rank_step_us_wall": round(one_rank_us, 2),
+        "one_rank_step_us_kernels": round(one_rank_kernels, 2),
+        "all_ranks_step_us_wall": round(whole_us, 2),
+        "kernels": kernels,
+        "rows_received_per_rank_first_routing": [int(v) for v in rows_of[0]],
+        "note": "two-hop bytes: a send reads 4096 bf16 rows and their index rows and stages one fp8 row with its "
+                "scales per token; a recv reads and writes the rows its rank receives; a combine-send reads and "
+                "writes the bf16 rows of its rank; the combine-recv is the gather of the group call over the "
+                "staging buffer.  one_rank_step = rank 0's four calls (what a rank on a GPU of its own runs; "
+                "its recv is the step's first and also lays out the other receivers); all_ranks_step = the "
+                "send, every rank's recv, every rank's combine-send and rank 0's combine-recv (the work of "
+                "the whole group for one sender's tokens, on this GPU).  Kernel durations come from events "
+                f"the launches record themselves, over {sample_steps} steps; wall times from {steps} steps "
+                "without events.",
+    }
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--routings", type=int, default=4, help="distinct routings cycled over the steps")
+    ap.add_argument("--regions", type=int, default=5,
+                    help="repetitions of the timed region (warm-up, then K steps without events); the line's "
+                         "value is the median region")
     ap.add_argument("--cpu-reps", type=int, default=3, help="repetitions of the CPU baseline (0 = skip)")
     ap.add_argument("--no-decode", action="store_true", help="skip the shapes other than the 4096-token one")
+    ap.add_argument("--no-split", action="store_true", help="skip the pass through the four split calls")
+    ap.add_argument("--split-only", action="store_true",
+                    help="time only the four split calls at the headline's shape (for a kernel trace of them alone)")
     ap.add_argument("--decode-only", action="store_true",
                     help="time only the 128-token shape (for a kernel trace of the decode step alone)")
     ap.add_argument("--only-shape", choices=("decode_128", "qwen3_decode_128", "kimi_1024"), default=None,
@@ -448,6 +629,11 @@ def main() -> int:
                   "receive slots padded to 128 per expert")
     others = {"decode_128": (C2, decode_label, None), "qwen3_decode_128": (C1, qwen_label, None),
               "kimi_1024": (C4, kimi_label, 37.0)}
+    if args.split_only:
+        print(json.dumps({"split_calls_4096_only": split_calls(
+            C3, device, args.routings, side_steps, args.warmup,
+            "DeepSeek-V3 prefill through the four split calls, rank 0 holds the 4096 tokens")}))
+        return 0
     if args.decode_only:
         args.only_shape = "decode_128"
     if args.only_shape is not None:
@@ -463,8 +649,10 @@ def main() -> int:
     #    record their own start and end instead: the samples of the roofline figures.
     _, disp, comb, both, pack, gather, route = time_workload(wl, side_steps, args.warmup, kernel_every=4,
                                                              call_every=1, route_events=True)
-    # 2. The timed region: no events.
-    wall_s, _, _, _, _, _, _ = time_workload(wl, args.steps, args.warmup)
+    # 2. The timed region: W warm-up steps, then exactly K steps between two synchronisations, no events.
+    #    Run `regions` times over; the line's value is the MEDIAN region, the spread is reported.
+    region_s = sorted(time_workload(wl, args.steps, args.warmup)[0] for _ in range(args.regions))
+    wall_s = region_s[len(region_s) // 2]
     # 3. The same as graph replays.
     graph_step_s, graph_steps = time_graph_replay(wl, args.steps, args.warmup)
     rows = wl.rows
@@ -497,7 +685,11 @@ def main() -> int:
     dominant, other = ((combine_roof, dispatch_roof) if g_stats.mean >= p_stats.mean
                        else (dispatch_roof, combine_roof))
 
-    decode = qwen = kimi = whole_group = None
+    decode = qwen = kimi = whole_group = split = None
+    if not args.no_split:
+        split = split_calls(C3, device, args.routings, side_steps, args.warmup,
+                            "DeepSeek-V3 prefill through the four split calls (send, recv, combine-send, "
+                            "combine-recv), rank 0 holds the 4096 tokens")
     if not args.no_decode:
         decode = other_shape(C2, device, args.routings, side_steps, args.warmup, ctx_flags, decode_label)
         decode["note"] = ("working set (26 MB) fits the 256 MB Infinity Cache and is not flushed between steps; "
@@ -568,6 +760,19 @@ def main() -> int:
             "routings_cycled": args.routings,
         },
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
+        "pct_of_hbm_peak_p50_with_events": round(
+            100.0 * (d_bytes + c_bytes) / (Statistics.create(both).p50 * 1e-6) / 1e9 / HBM_PEAK_GBS, 2),
+        "timed_regions": {
+            "regions": len(region_s), "steps_each": args.steps, "warmup_each": args.warmup,
+            "us_per_step": {"min": round(region_s[0] / args.steps * 1e6, 2),
+                            "median": round(wall_s / args.steps * 1e6, 2),
+                            "max": round(region_s[-1] / args.steps * 1e6, 2)},
+            "note": "each region: W warm-up steps, then exactly K steps between two synchronisations, no event in "
+                    "between; `value`, `ms_per_step` and `pct_of_hbm_peak` are the median region; "
+                    "`pct_of_hbm_peak_p50_with_events` is the same bytes over the p50 of the per-step time of the "
+                    "pass that records events around each phase of every step (the reference benchmark's method: "
+                    "every event idles the queue for about 3 us)",
+        },
         "prefill_4096": {
             "step_us_wall": round(ms_per_step * 1e3, 2),
             "graph_replay": {"step_us_wall": round(graph_step_s * 1e6, 2), "steps": graph_steps,
@@ -589,6 +794,7 @@ def main() -> int:
                 "total_us": stats_dict(both),
             },
         },
+        "split_calls_4096": split,
         "decode_128": decode,
         "qwen3_decode_128": qwen,
         "kimi_1024": kimi,

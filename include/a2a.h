@@ -309,20 +309,32 @@ typedef enum a2a_table {
 int a2a_ctx_read_table(a2a_ctx *ctx, uint32_t rank, uint32_t which,
                        uint32_t *out, size_t count, void *stream);
 
-/* Measuring aid, no counterpart in the reference.  The next a2a_dispatch (which =
- * A2A_KERNEL_PACK or A2A_KERNEL_ROUTE) or a2a_combine (A2A_KERNEL_GATHER) on
- * this context launches that kernel so that `start_event` and `stop_event`
- * (hipEvent_t, created by the caller with timing enabled) are recorded when the
- * kernel itself begins and ends; hipEventElapsedTime between them is the
- * kernel's duration, without the queue packets and idle time that events
- * recorded around a call add.  A2A_KERNEL_ROUTE is the routing launch that
- * precedes the pack of a large step; a step that counts its routing inside the
- * pack (a small one, or one source alone with up to 8192 copies) or runs several
- * routing kernels (A2A_FLAG_SEPARATE_ROUTING) has no such launch and leaves
- * those events alone.  One-shot: the request is
- * consumed by that call.  Pass two nulls to withdraw it.  The stop event must
- * have completed before its time is read (synchronise the stream or the event). */
-enum { A2A_KERNEL_PACK = 0, A2A_KERNEL_GATHER = 1, A2A_KERNEL_ROUTE = 2 };
+/* Measuring aid, no counterpart in the reference.  The next call on this context
+ * that launches the named kernel launches it so that `start_event` and
+ * `stop_event` (hipEvent_t, created by the caller with timing enabled) are
+ * recorded when the kernel itself begins and ends; hipEventElapsedTime between
+ * them is the kernel's duration, without the queue packets and idle time that
+ * events recorded around a call add.
+ *   A2A_KERNEL_PACK          the pack of the next a2a_dispatch
+ *   A2A_KERNEL_ROUTE         the routing launch that precedes the pack of a large
+ *                            step (a2a_dispatch) or the staging of a large send
+ *                            (a2a_dispatch_send); a step that counts its routing
+ *                            inside the pack or the staging launch (a small one,
+ *                            or one source alone with up to 8192 copies) or runs
+ *                            several routing kernels (A2A_FLAG_SEPARATE_ROUTING)
+ *                            has no such launch and leaves those events alone
+ *   A2A_KERNEL_GATHER        the gather of the next a2a_combine or a2a_combine_recv
+ *   A2A_KERNEL_STAGE_SEND    the staging launch of the next a2a_dispatch_send
+ *   A2A_KERNEL_STAGE_RECV    the copy launch of the next a2a_dispatch_recv
+ *   A2A_KERNEL_COMBINE_SEND  the copy launch of the next a2a_combine_send
+ * One-shot: the request is consumed by that call (a call that launches nothing,
+ * such as a send without tokens, consumes it too).  Pass two nulls to withdraw
+ * it.  The stop event must have completed before its time is read (synchronise
+ * the stream or the event). */
+enum {
+    A2A_KERNEL_PACK = 0, A2A_KERNEL_GATHER = 1, A2A_KERNEL_ROUTE = 2,
+    A2A_KERNEL_STAGE_SEND = 3, A2A_KERNEL_STAGE_RECV = 4, A2A_KERNEL_COMBINE_SEND = 5
+};
 int a2a_ctx_time_next_kernel(a2a_ctx *ctx, uint32_t which, void *start_event, void *stop_event);
 
 /* Row strides of the staging buffers (a2a_worker.rs:317-325). */

@@ -47,7 +47,7 @@ struct a2a_ctx {
 
     Staging staging;               // buffers and tables of the split calls
 
-    KernelTiming timing[3];        // one-shot events for the next pack / gather / routing launch of a group call
+    KernelTiming timing[6];        // one-shot events for the next launch of each kernel a2a_ctx_time_next_kernel names
 };
 
 // Device memory of a2a_dispatch_static: the routing tables of ONE step, in a
@@ -823,8 +823,7 @@ int a2a_combine(a2a_ctx *ctx, const a2a_combine_args *args, uint32_t expert_y_dt
 
 int a2a_ctx_time_next_kernel(a2a_ctx *ctx, uint32_t which, void *start_event, void *stop_event) {
     if (ctx == nullptr) return A2A_ERR_INVALID_ARGUMENT;
-    if (which != A2A_KERNEL_PACK && which != A2A_KERNEL_GATHER && which != A2A_KERNEL_ROUTE)
-        return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "unknown kernel %u", which);
+    if (which > A2A_KERNEL_COMBINE_SEND) return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "unknown kernel %u", which);
     if ((start_event == nullptr) != (stop_event == nullptr))
         return fail(ctx, A2A_ERR_INVALID_ARGUMENT, "pass both events or neither");
     ctx->timing[which].start = static_cast<hipEvent_t>(start_event);
@@ -933,6 +932,10 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     hipStream_t s = static_cast<hipStream_t>(stream);
     const uint32_t K = c.num_experts_per_token;
     const uint32_t T = (uint32_t)num_tokens;
+    const KernelTiming send_timing = ctx->timing[A2A_KERNEL_STAGE_SEND];
+    const KernelTiming route_timing = ctx->timing[A2A_KERNEL_ROUTE];
+    ctx->timing[A2A_KERNEL_STAGE_SEND] = KernelTiming();
+    ctx->timing[A2A_KERNEL_ROUTE] = KernelTiming();
 
     // The sender is the rank's dp group; when several members of a group send, each repeats
     // the same routing and stages the same rows.
@@ -967,7 +970,7 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
 
     hipError_t e;
     if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && stage_send_small_fits(sa, ctx->ws)) {
-        e = launch_stage_send_small(sa, ctx->ws, ctx->staging, quantize != 0, s);
+        e = launch_stage_send_small(sa, ctx->ws, ctx->staging, quantize != 0, s, send_timing);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send_small");
     } else {
         RouteArgs ra;
@@ -984,9 +987,9 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
         if (T != 0 && !(c.flags & A2A_FLAG_SEPARATE_ROUTING)) {
             // two launches: chunk histograms that also add up the sender's totals, then a staging
             // launch whose workgroups resolve their own positions from them
-            e = launch_route_accumulate(ra, ctx->ws, nb, s, true);
+            e = launch_route_accumulate(ra, ctx->ws, nb, s, true, route_timing);
             if (e != hipSuccess) return hip_fail(ctx, e, "launch route_hist (accumulating, send)");
-            e = launch_stage_send_resolve(sa, ctx->ws, ctx->staging, quantize != 0, s);
+            e = launch_stage_send_resolve(sa, ctx->ws, ctx->staging, quantize != 0, s, send_timing);
             if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send_resolve");
         } else {
             if (fused_routing_pays(fa, c.world_size / c.dp_size, nb)) {
@@ -998,7 +1001,7 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
                 e = launch_finalize(fa, ctx->ws, s);
                 if (e != hipSuccess) return hip_fail(ctx, e, "launch route_finalize");
             }
-            e = launch_stage_send(sa, ctx->ws, ctx->staging, quantize != 0, s);
+            e = launch_stage_send(sa, ctx->ws, ctx->staging, quantize != 0, s, send_timing);
             if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send");
         }
     }
@@ -1046,7 +1049,9 @@ int a2a_dispatch_recv(a2a_ctx *ctx, uint32_t rank, int32_t *out_num_tokens, void
     // worker does (a2a_worker.rs:526-703), not once per recv launch.
     rv.valid_mask = ctx->sent_mask & ~ctx->empty_mask;
     rv.max_private = c.max_private_tokens;
-    const hipError_t e = launch_stage_recv(rv, ctx->ws, ctx->staging, !ctx->recv_seen, s);
+    const KernelTiming recv_timing = ctx->timing[A2A_KERNEL_STAGE_RECV];
+    ctx->timing[A2A_KERNEL_STAGE_RECV] = KernelTiming();
+    const hipError_t e = launch_stage_recv(rv, ctx->ws, ctx->staging, !ctx->recv_seen, s, recv_timing);
     if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_recv");
     ctx->recv_seen = true;
     ctx->staging.recv_mask |= 1u << rank;
@@ -1082,7 +1087,9 @@ int a2a_combine_send(a2a_ctx *ctx, uint32_t rank, const void *expert_y, size_t e
     cs.y_rows = (uint32_t)(expert_y_rows > 0xFFFFFFFFull ? 0xFFFFFFFFull : expert_y_rows);
     cs.row_bytes = (uint32_t)((size_t)c.hidden_dim * c.out_elemsize);
     cs.max_rows = rows_upper_bound(ctx);
-    hipError_t e = launch_combine_send(cs, ctx->ws, ctx->staging, static_cast<hipStream_t>(stream));
+    const KernelTiming timing = ctx->timing[A2A_KERNEL_COMBINE_SEND];
+    ctx->timing[A2A_KERNEL_COMBINE_SEND] = KernelTiming();
+    hipError_t e = launch_combine_send(cs, ctx->ws, ctx->staging, static_cast<hipStream_t>(stream), timing);
     if (e != hipSuccess) return hip_fail(ctx, e, "launch combine_send");
     ctx->staging.combine_sent_mask |= 1u << rank;
     return A2A_OK;
@@ -1132,8 +1139,10 @@ int a2a_combine_recv(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, size_t num_
     cr.dst.num_tokens = (uint32_t)num_tokens;
     cr.hidden_dim = c.hidden_dim;
     cr.accumulate = accumulate ? 1 : 0;
+    const KernelTiming timing = ctx->timing[A2A_KERNEL_GATHER];
+    ctx->timing[A2A_KERNEL_GATHER] = KernelTiming();
     hipError_t e = launch_combine_recv(cr, ctx->ws, ctx->staging, expert_y_dtype, c.out_dtype,
-                                       static_cast<hipStream_t>(stream));
+                                       static_cast<hipStream_t>(stream), timing);
     if (e != hipSuccess) return hip_fail(ctx, e, "launch combine_recv");
     return A2A_OK;
 }

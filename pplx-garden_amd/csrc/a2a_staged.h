@@ -92,20 +92,21 @@ const uint32_t *staging_table(const Staging &st, const a2a_config &cfg, uint32_t
                               size_t *limit);
 
 hipError_t launch_stage_send(const StageSendArgs &args, const Workspace &ws, const Staging &st,
-                             bool quantize, hipStream_t stream);
+                             bool quantize, hipStream_t stream, KernelTiming timing = KernelTiming());
 // One-launch send (routing counted inside) for small steps: whether a step qualifies, and the launch.
 bool stage_send_small_fits(const StageSendArgs &args, const Workspace &ws);
 hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &ws, const Staging &st,
-                                   bool quantize, hipStream_t stream);
+                                   bool quantize, hipStream_t stream, KernelTiming timing = KernelTiming());
 // The send of a large step after launch_route_accumulate(..., for_send = true).
 hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace &ws, const Staging &st,
-                                     bool quantize, hipStream_t stream);
+                                     bool quantize, hipStream_t stream, KernelTiming timing = KernelTiming());
 // `first_of_step`: no recv has run since the step's sends; this launch also lays out the other receivers.
 hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st, bool first_of_step,
-                             hipStream_t stream);
+                             hipStream_t stream, KernelTiming timing = KernelTiming());
 hipError_t launch_combine_send(const CombineSendArgs &args, const Workspace &ws, const Staging &st,
-                               hipStream_t stream);
+                               hipStream_t stream, KernelTiming timing = KernelTiming());
 hipError_t launch_combine_recv(const CombineRecvArgs &args, const Workspace &ws, const Staging &st,
-                               uint32_t in_dtype, uint32_t out_dtype, hipStream_t stream);
+                               uint32_t in_dtype, uint32_t out_dtype, hipStream_t stream,
+                               KernelTiming timing = KernelTiming());
 
 }  // namespace a2a

@@ -951,15 +951,15 @@ const uint32_t *staging_table(const Staging &st, const a2a_config &cfg, uint32_t
 }
 
 hipError_t launch_stage_send(const StageSendArgs &args, const Workspace &ws, const Staging &st,
-                             bool quantize, hipStream_t stream) {
+                             bool quantize, hipStream_t stream, KernelTiming timing) {
     if (args.src.num_tokens == 0) return hipSuccess;
     const uint32_t threads = block_for_chunks(quantize ? args.hidden_dim / 16 : args.row_bytes / 16);
     if (quantize) {
-        hipLaunchKernelGGL(stage_send_kernel<true>, dim3(args.src.num_tokens), dim3(threads), 0, stream,
-                           args, ws, st);
+        hipExtLaunchKernelGGL(stage_send_kernel<true>, dim3(args.src.num_tokens), dim3(threads), 0, stream,
+                              timing.start, timing.stop, 0, args, ws, st);
     } else {
-        hipLaunchKernelGGL(stage_send_kernel<false>, dim3(args.src.num_tokens), dim3(threads), 0, stream,
-                           args, ws, st);
+        hipExtLaunchKernelGGL(stage_send_kernel<false>, dim3(args.src.num_tokens), dim3(threads), 0, stream,
+                              timing.start, timing.stop, 0, args, ws, st);
     }
     return hipGetLastError();
 }
@@ -971,21 +971,21 @@ bool stage_send_small_fits(const StageSendArgs &args, const Workspace &ws) {
 }
 
 hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &ws, const Staging &st,
-                                   bool quantize, hipStream_t stream) {
+                                   bool quantize, hipStream_t stream, KernelTiming timing) {
     const uint32_t threads = block_for_chunks(quantize ? args.hidden_dim / 16 : args.row_bytes / 16);
     const size_t lds = 3 * (size_t)ws.num_experts * sizeof(uint32_t);
     if (quantize) {
-        hipLaunchKernelGGL(stage_send_small_kernel<true>, dim3(args.src.num_tokens), dim3(threads), lds, stream,
-                           args, ws, st);
+        hipExtLaunchKernelGGL(stage_send_small_kernel<true>, dim3(args.src.num_tokens), dim3(threads), lds, stream,
+                              timing.start, timing.stop, 0, args, ws, st);
     } else {
-        hipLaunchKernelGGL(stage_send_small_kernel<false>, dim3(args.src.num_tokens), dim3(threads), lds, stream,
-                           args, ws, st);
+        hipExtLaunchKernelGGL(stage_send_small_kernel<false>, dim3(args.src.num_tokens), dim3(threads), lds, stream,
+                              timing.start, timing.stop, 0, args, ws, st);
     }
     return hipGetLastError();
 }
 
 hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace &ws, const Staging &st,
-                                     bool quantize, hipStream_t stream) {
+                                     bool quantize, hipStream_t stream, KernelTiming timing) {
     uint32_t threads = block_for_chunks(quantize ? args.hidden_dim / 16 : args.row_bytes / 16);
     const uint32_t blocks = args.src.num_tokens + 1;
     StageSendArgs a = args;
@@ -995,21 +995,24 @@ hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace 
         threads += kWave;
     }
     if (quantize) {
-        hipLaunchKernelGGL(stage_send_resolve_kernel<true>, dim3(blocks), dim3(threads), 0, stream, a, ws, st);
+        hipExtLaunchKernelGGL(stage_send_resolve_kernel<true>, dim3(blocks), dim3(threads), 0, stream, timing.start,
+                              timing.stop, 0, a, ws, st);
     } else {
-        hipLaunchKernelGGL(stage_send_resolve_kernel<false>, dim3(blocks), dim3(threads), 0, stream, a, ws, st);
+        hipExtLaunchKernelGGL(stage_send_resolve_kernel<false>, dim3(blocks), dim3(threads), 0, stream, timing.start,
+                              timing.stop, 0, a, ws, st);
     }
     return hipGetLastError();
 }
 
 hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st, bool first_of_step,
-                             hipStream_t stream) {
+                             hipStream_t stream, KernelTiming timing) {
     RowLaunch l = row_launch(args.max_rows, args.row_bytes / 16);
     if (l.blocks == 0) l.blocks = 1;    // the counts are handed over even when nothing was sent
     StageRecvArgs a = args;
     a.team_waves = l.team_waves;
     if (!first_of_step) {
-        hipLaunchKernelGGL(stage_recv_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, a, ws, st);
+        hipExtLaunchKernelGGL(stage_recv_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, timing.start, timing.stop,
+                              0, a, ws, st);
         return hipGetLastError();
     }
     // Behind the caller's workgroups: a few per other receiver, enough threads for the rows a receiver
@@ -1021,22 +1024,24 @@ hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, con
     if (a.slices > 16) a.slices = 16;
     const uint32_t blocks = l.blocks + (ws.world - 1) * a.slices;
     const size_t lds = (4 * (size_t)ws.num_groups * ws.experts_per_rank + 1 + 3 * (size_t)ws.num_groups) * sizeof(uint32_t);
-    hipLaunchKernelGGL(stage_recv_first_kernel, dim3(blocks), dim3(l.threads), lds, stream, a, ws, st);
+    hipExtLaunchKernelGGL(stage_recv_first_kernel, dim3(blocks), dim3(l.threads), lds, stream, timing.start,
+                          timing.stop, 0, a, ws, st);
     return hipGetLastError();
 }
 
 hipError_t launch_combine_send(const CombineSendArgs &args, const Workspace &ws, const Staging &st,
-                               hipStream_t stream) {
+                               hipStream_t stream, KernelTiming timing) {
     if (args.max_rows == 0) return hipSuccess;
     const RowLaunch l = row_launch(args.max_rows, args.row_bytes / 16);
     CombineSendArgs a = args;
     a.team_waves = l.team_waves;
-    hipLaunchKernelGGL(combine_send_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, a, ws, st);
+    hipExtLaunchKernelGGL(combine_send_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, timing.start, timing.stop,
+                          0, a, ws, st);
     return hipGetLastError();
 }
 
 hipError_t launch_combine_recv(const CombineRecvArgs &args, const Workspace &ws, const Staging &st,
-                               uint32_t in_dtype, uint32_t out_dtype, hipStream_t stream) {
+                               uint32_t in_dtype, uint32_t out_dtype, hipStream_t stream, KernelTiming timing) {
     CombArgs ca;
     std::memset(&ca, 0, sizeof ca);
     ca.dst[args.rank] = args.dst;
@@ -1047,7 +1052,7 @@ hipError_t launch_combine_recv(const CombineRecvArgs &args, const Workspace &ws,
     ca.accumulate = args.accumulate;
     ca.staged_base = st.comb_buf;
     ca.staged_stride = st.comb_stride;
-    return launch_combine_gather(ca, ws, in_dtype, out_dtype, args.dst.num_tokens, stream);
+    return launch_combine_gather(ca, ws, in_dtype, out_dtype, args.dst.num_tokens, stream, timing);
 }
 
 }  // namespace a2a

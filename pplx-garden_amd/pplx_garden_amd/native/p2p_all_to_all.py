@@ -50,6 +50,9 @@ FLAG_SEPARATE_ROUTING = 2   # never take the one-launch paths of small steps
 KERNEL_PACK = 0
 KERNEL_GATHER = 1
 KERNEL_ROUTE = 2
+KERNEL_STAGE_SEND = 3
+KERNEL_STAGE_RECV = 4
+KERNEL_COMBINE_SEND = 5
 
 
 class A2AConfig(ctypes.Structure):
@@ -331,10 +334,12 @@ class AllToAllContext:
         return torch.tensor(list(buf[:count]), dtype=torch.int64)
 
     def time_next_kernel(self, which: int, start_event: Optional[int], stop_event: Optional[int]) -> None:
-        """Have the next group dispatch (`KERNEL_PACK`, `KERNEL_ROUTE`) or combine (`KERNEL_GATHER`)
+        """Have the next call that launches kernel `which` (`KERNEL_PACK`, `KERNEL_ROUTE`: the group
+        dispatch; `KERNEL_GATHER`: the group combine or the split combine-recv; `KERNEL_STAGE_SEND`,
+        `KERNEL_ROUTE`: the split send; `KERNEL_STAGE_RECV`, `KERNEL_COMBINE_SEND`: those split calls)
         record the two events (raw `hipEvent_t` handles, e.g. `torch.cuda.Event.cuda_event`) at the
-        start and end of that kernel itself.  `KERNEL_ROUTE` is the routing launch before the pack of a
-        large step; a step without such a launch leaves those events alone."""
+        start and end of that kernel itself.  `KERNEL_ROUTE` is the routing launch before the pack or
+        the staging of a large step; a step without such a launch leaves those events alone."""
         self._require_open()
         self._check(self._lib.a2a_ctx_time_next_kernel(self._handle, which, _ptr(start_event), _ptr(stop_event)))
 
