@@ -371,13 +371,15 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
         tok_ids[ft] = t < effective_tokens(from.bound_m, from.num_tokens) ? ids : 0;
     }
     // SINGLE: a token workgroup keeps only the row of the one source, at the front
-    uint32_t *cnt = s_dyn;                                  // [G][E] (SINGLE: [E]) or, receivers, [G][Le]
-    uint32_t *prior = s_dyn + (SINGLE ? (size_t)E : (size_t)G * E);   // [E] own source, tokens before mine
-    uint32_t *rows_before = prior + E;                      // [E] padded rows of all experts before e
+    // [G][E] (SINGLE: [E]): low half of a word the entries of (source, expert), high half (own source only)
+    // those of the tokens before mine; receivers: [G][Le] plain counts.  A step of this kernel has at most
+    // kSmallMaxEntries < 2^16 entries.
+    uint32_t *cnt = s_dyn;
+    uint32_t *rows_before = s_dyn + (SINGLE ? (size_t)E : (size_t)G * E);   // [E] padded rows of all experts before e
     uint32_t *copies_before = rows_before + E;              // [E] copies of the sources laid out before mine
-    const uint32_t table = receiver ? G * Le : G * E + E;
+    const uint32_t table = receiver ? G * Le : G * E;
     if (SINGLE && !receiver) {
-        for (uint32_t i = tid; i < 2 * E; i += nthreads) s_dyn[i] = 0;   // cnt and prior
+        for (uint32_t i = tid; i < E; i += nthreads) s_dyn[i] = 0;
     } else {
         for (uint32_t i = tid; i < table; i += nthreads) s_dyn[i] = 0;
     }
@@ -441,9 +443,8 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
                 const uint32_t le = x - rank * Le;   // wraps for experts of lower ranks
                 if (le < Le) atomicAdd(&cnt[src_of[j] * Le + le], 1u);
             } else {
-                atomicAdd(&cnt[(SINGLE ? 0 : src_of[j]) * E + x], 1u);
                 const uint32_t f = f0 + j * nthreads + tid;
-                if (src_of[j] == my_g && f < my_first) atomicAdd(&prior[x], 1u);
+                atomicAdd(&cnt[(SINGLE ? 0 : src_of[j]) * E + x], src_of[j] == my_g && f < my_first ? 0x10001u : 1u);
             }
         }
     };
@@ -507,7 +508,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
         const uint32_t e = e0 + tid;
         uint32_t total = 0, before = 0;
         if (SINGLE) {
-            total = e < E ? cnt[e] : 0;   // nobody else sends: nothing is laid out before mine
+            total = e < E ? cnt[e] & 0xFFFFu : 0;   // nobody else sends: nothing is laid out before mine
         } else if (e < E) {
             const uint32_t r = owner_of_expert(ws, e);
             bool seen = false;
@@ -519,7 +520,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
 #pragma unroll
                 for (uint32_t j = 0; j < 8; ++j) {
                     g[j] = (j < 4 ? w0 >> (8 * j) : w1 >> (8 * (j - 4))) & 0xFFu;
-                    c[j] = i0 + j < G ? cnt[g[j] * E + e] : 0;
+                    c[j] = i0 + j < G ? cnt[g[j] * E + e] & 0xFFFFu : 0;
                 }
 #pragma unroll
                 for (uint32_t j = 0; j < 8; ++j) {
@@ -548,7 +549,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
         uint32_t run = 0;
         for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
             const uint32_t e = e0 + lane;
-            const uint32_t v = e < E ? cnt[(SINGLE ? 0 : my_g) * E + e] : 0;
+            const uint32_t v = e < E ? cnt[(SINGLE ? 0 : my_g) * E + e] & 0xFFFFu : 0;
             const uint32_t incl = run + wave_inclusive_scan(v, lane);
             if (e < E) {
                 ws.num_routed[my_g * E + e] = v;
@@ -572,7 +573,7 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
         uint32_t slot = kInvalidSlot, toff = 0;
         if (my_expert < E) {
             // copies of my source before this one: earlier tokens, then earlier k of this token
-            toff = prior[my_expert] + repeats;
+            toff = (cnt[(SINGLE ? 0 : my_g) * E + my_expert] >> 16) + repeats;
             const uint32_t r = owner_of_expert(ws, my_expert);
             const uint32_t row = rows_before[my_expert] - rows_before[r * Le] + copies_before[my_expert];
             slot = resolve_copy(s_dst[r], ws, row + toff, wave == 0, &row_ptr, &scale_ptr, &scale_stride);
@@ -606,12 +607,18 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
 // are the same: first row of the expert in its receiver + copies of earlier
 // tokens to the expert + copies of this token at an earlier k.
 //
-// Dynamic LDS: 3 * E words (or G * Le, if that is more: the receivers' table).
+// Dynamic LDS: 2 * E words (or G * Le, if that is more: the receivers' table).
+//
+// Two of these workgroups must fit a compute unit at once (the grid is one workgroup per
+// compute unit plus the receivers' ones, and a workgroup that has to wait for another to end starts
+// its whole chain a step late: 4 us on the 1024-token step).  With 14 wavefronts each that means at
+// most 64 vector registers a lane, which the kernel is held to (amdgpu_waves_per_eu): left to itself
+// the compiler moved between 62 and 75 with unrelated changes to the code.
 constexpr uint32_t kTokensPerGroup = 4;
 constexpr uint32_t kMaxGroupRoutes = kTokensPerGroup * A2A_MAX_EXPERTS_PER_TOKEN;
 
 template <bool QUANT>
-__global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs args, const FinalizeArgs fin,
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8))) void dispatch_single_kernel(const PushArgs args, const FinalizeArgs fin,
                                                                const Workspace ws, const uint32_t team_threads,
                                                                const uint32_t per_group) {
     extern __shared__ uint32_t s_tab[];
@@ -686,10 +693,10 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
         }
     }
 
-    uint32_t *cnt = s_tab;                 // [E] entries per expert; receivers: [G][Le]
-    uint32_t *prior = s_tab + E;           // [E] entries per expert before my first token
-    uint32_t *rows_before = prior + E;     // [E] padded rows of all experts before e
-    const uint32_t table = receiver ? G * Le : 2 * E;
+    uint32_t *cnt = s_tab;                 // [E] low half: entries per expert, high half: those before my first
+                                           // token; receivers: [G][Le] plain counts
+    uint32_t *rows_before = cnt + E;       // [E] padded rows of all experts before e
+    const uint32_t table = receiver ? G * Le : E;
     for (uint32_t i = tid; i < table; i += nthreads) s_tab[i] = 0;
     // Sources without tokens have no workgroup of their own: the first receiver
     // workgroup (the first workgroup, if nobody receives) clears their tables, at the end of its work.
@@ -718,8 +725,9 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
                 const uint32_t le = x - rank * Le;   // wraps for experts of lower ranks
                 if (le < Le) atomicAdd(&cnt[my_g * Le + le], 1u);
             } else {
-                atomicAdd(&cnt[x], 1u);
-                if (f0 + j * nthreads + tid < my_first) atomicAdd(&prior[x], 1u);
+                // one word per expert: low half all its entries, high half those before my first token
+                // (a step of this kernel has at most kSingleMaxEntries < 2^16 entries)
+                atomicAdd(&cnt[x], f0 + j * nthreads + tid < my_first ? 0x10001u : 1u);
             }
         }
     };
@@ -751,7 +759,7 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
     uint32_t carry = 0;
     for (uint32_t e0 = 0; e0 < E; e0 += nthreads) {
         const uint32_t e = e0 + tid;
-        const uint32_t total = e < E ? cnt[e] : 0;
+        const uint32_t total = e < E ? cnt[e] & 0xFFFFu : 0;
         const uint32_t padded = e < E ? (total + pad - 1) / pad * pad : 0;
         const uint32_t incl = carry + block_inclusive_scan<true>(padded, scratch);
         if (e < E) rows_before[e] = incl - padded;
@@ -768,7 +776,7 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
         uint32_t run = 0;
         for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
             const uint32_t e = e0 + lane;
-            const uint32_t v = e < E ? cnt[e] : 0;
+            const uint32_t v = e < E ? cnt[e] & 0xFFFFu : 0;
             const uint32_t incl = run + wave_inclusive_scan(v, lane);
             if (e < E) {
                 ws.num_routed[my_g * E + e] = v;
@@ -787,7 +795,7 @@ __global__ __launch_bounds__(1024) void dispatch_single_kernel(const PushArgs ar
             // copies of the source before this one: those of earlier workgroups' tokens, then mine
             uint32_t earlier = 0;
             for (uint32_t q = 0; q < tid; ++q) earlier += s_route_expert[q] == my_expert ? 1u : 0u;
-            toff = prior[my_expert] + earlier;
+            toff = (cnt[my_expert] >> 16) + earlier;
             const uint32_t r = owner_of_expert(ws, my_expert);
             const uint32_t row = rows_before[my_expert] - rows_before[r * Le];
             slot = resolve_copy(s_dst[r], ws, row + toff, true, &row_ptr, &scale_ptr, &scale_stride);
@@ -1104,7 +1112,7 @@ hipError_t launch_dispatch_single(const PushArgs &args, const FinalizeArgs &fin,
     const uint32_t per_group = single_tokens_per_group(total_tokens);
     const uint32_t threads = single_threads(team, per_group);
     const uint32_t blocks = (total_tokens + per_group - 1) / per_group + (fin.recv_mask != 0 ? ws.world : 0);
-    const size_t token_words = 3 * (size_t)ws.num_experts;
+    const size_t token_words = 2 * (size_t)ws.num_experts;
     const size_t receiver_words = (size_t)ws.num_groups * ws.experts_per_rank;
     const size_t lds = (token_words > receiver_words ? token_words : receiver_words) * sizeof(uint32_t);
     PushArgs a = args;
