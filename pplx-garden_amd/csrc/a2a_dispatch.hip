@@ -603,22 +603,24 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
 // token workgroups are about as many as the compute units): it is made of
 // teams of wavefronts, each as wide as a token row needs, that move one token
 // each per round.  As in dispatch_small_kernel no workgroup depends on another,
-// the receiver workgroups follow the token workgroups in the grid, and the rows
-// are the same: first row of the expert in its receiver + copies of earlier
-// tokens to the expert + copies of this token at an earlier k.
+// and the rows are the same: first row of the expert in its receiver + copies of
+// earlier tokens to the expert + copies of this token at an earlier k.  There are
+// no receiver workgroups: with one source a token workgroup's own tables hold
+// everything a receiver's layout needs, and the first workgroups write it.
 //
-// Dynamic LDS: 2 * E words (or G * Le, if that is more: the receivers' table).
+// Dynamic LDS: 2 * E words.
 //
-// Two of these workgroups must fit a compute unit at once (the grid is one workgroup per
-// compute unit plus the receivers' ones, and a workgroup that has to wait for another to end starts
-// its whole chain a step late: 4 us on the 1024-token step).  With 14 wavefronts each that means at
-// most 64 vector registers a lane, which the kernel is held to (amdgpu_waves_per_eu): left to itself
-// the compiler moved between 62 and 75 with unrelated changes to the code.
+// Two of these workgroups should fit a compute unit at once: where the grid has more workgroups than
+// the GPU has compute units, a workgroup that has to wait for another to end starts its whole chain
+// a step late (4 us on the 1024-token step when its grid still had the receivers' workgroups on top
+// of one token workgroup per compute unit).  With 14 wavefronts each that means at most 72 vector
+// registers a lane, which the kernel is held to (amdgpu_waves_per_eu): left to itself the compiler
+// moved between 62 and 75 with unrelated changes to the code.
 constexpr uint32_t kTokensPerGroup = 4;
 constexpr uint32_t kMaxGroupRoutes = kTokensPerGroup * A2A_MAX_EXPERTS_PER_TOKEN;
 
 template <bool QUANT>
-__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8))) void dispatch_single_kernel(const PushArgs args, const FinalizeArgs fin,
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(7))) void dispatch_single_kernel(const PushArgs args, const FinalizeArgs fin,
                                                                const Workspace ws, const uint32_t team_threads,
                                                                const uint32_t per_group) {
     extern __shared__ uint32_t s_tab[];
@@ -639,14 +641,16 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8))) void 
     const uint32_t G = ws.num_groups, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
     const uint32_t my_g = args.single_source - 1;
     const PushSrc &src = args.single;
-    const uint32_t token_groups = (src.num_tokens + per_group - 1) / per_group;
-    const bool receiver = blockIdx.x >= token_groups;
+    const uint32_t token_groups = gridDim.x;                            // every workgroup has tokens
     const uint32_t tokens = effective_tokens(src.bound_m, src.num_tokens);
     const uint32_t flat_entries = tokens * K;
-    const uint32_t first_token = blockIdx.x * per_group;                // token workgroups
+    const uint32_t first_token = blockIdx.x * per_group;
     const uint32_t my_first = first_token * K;                          // flat index of my first entry
-    // every token of mine is past the bound: nothing to send; the first workgroup stays (it publishes the totals)
-    if (!receiver && blockIdx.x != 0 && first_token >= tokens) return;
+    // Every token of mine is past the bound: nothing to send.  The first workgroups stay: they publish the
+    // totals, lay out the receivers and clear the tables of the sources without tokens (workgroup b:
+    // receivers and sources b, b + grid, ...).
+    const bool has_duty = blockIdx.x < ws.world;   // (there are at most as many sources as receivers)
+    if (!has_duty && first_token >= tokens) return;
 
     // The first entries and the ids of my tokens' routes are asked for first of all, then the rows of the
     // first round: they travel while the entries are counted and the routes resolved.
@@ -659,7 +663,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8))) void 
     }
     const uint32_t my_routes = per_group * K;    // one thread each
     uint32_t my_expert = 0xFFFFFFFFu;
-    if (!receiver && tid < my_routes && my_first + tid < flat_entries) {
+    if (tid < my_routes && my_first + tid < flat_entries) {
         my_expert = (uint32_t)src.indices[my_first + tid];
     }
     // The descriptor of receiver `tid` is asked for here too and written to LDS after the counting (written
@@ -677,43 +681,42 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8))) void 
     const uint32_t teams = nthreads / team_threads;
     const uint32_t team = tid / team_threads;
     const uint32_t team_tid = tid - team * team_threads;
+    // The same for the team's token of the SECOND round, asked for ahead of the first round's (it is
+    // needed later): a workgroup of two rounds then has all its rows on their way from the start and its
+    // rounds only store (1024 tokens: 41.3 -> 39.8 us per step).
     u32x4 pre_a, pre_b = {0, 0, 0, 0};
+    u32x4 next_a = {0, 0, 0, 0}, next_b = {0, 0, 0, 0};
     {
-        const uint32_t any_token =
-            receiver ? 0 : (first_token + team < src.num_tokens ? first_token + team : src.num_tokens - 1);
+        const uint32_t last_token = src.num_tokens - 1;
+        const uint32_t any_token = first_token + team < src.num_tokens ? first_token + team : last_token;
+        const uint32_t second = first_token + teams + team;
+        const uint32_t next_token = second < src.num_tokens ? second : last_token;
         const uint8_t *x_row = src.x + (size_t)any_token * src.x_stride;
+        const uint8_t *x_next = src.x + (size_t)next_token * src.x_stride;
+        const bool two_rounds = per_group > teams;   // uniform: a branch, not a select (nothing waits at its end)
         if constexpr (QUANT) {
             const uint32_t pieces = args.hidden_dim / 16;
-            const u32x4 *piece = reinterpret_cast<const u32x4 *>(x_row + (size_t)(team_tid < pieces ? team_tid : 0) * 32);
-            pre_a = __builtin_nontemporal_load(piece);
-            pre_b = __builtin_nontemporal_load(piece + 1);
+            const size_t at = (size_t)(team_tid < pieces ? team_tid : 0) * 32;
+            if (two_rounds) {
+                next_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_next + at));
+                next_b = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_next + at) + 1);
+            }
+            pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row + at));
+            pre_b = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row + at) + 1);
         } else {
             const uint32_t pieces = args.row_bytes / 16;
-            pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + (team_tid < pieces ? team_tid : 0));
+            const uint32_t at = team_tid < pieces ? team_tid : 0;
+            if (two_rounds) next_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_next) + at);
+            pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + at);
         }
     }
 
-    uint32_t *cnt = s_tab;                 // [E] low half: entries per expert, high half: those before my first
-                                           // token; receivers: [G][Le] plain counts
+    uint32_t *cnt = s_tab;                 // [E] low half: entries per expert, high half: those before my first token
     uint32_t *rows_before = cnt + E;       // [E] padded rows of all experts before e
-    const uint32_t table = receiver ? G * Le : E;
-    for (uint32_t i = tid; i < table; i += nthreads) s_tab[i] = 0;
-    // Sources without tokens have no workgroup of their own: the first receiver
-    // workgroup (the first workgroup, if nobody receives) clears their tables, at the end of its work.
-    auto clear_empty_sources = [&]() {
-        if (blockIdx.x != (fin.recv_mask != 0 ? token_groups : 0)) return;
-        for (uint32_t g = 0; g < G; ++g) {
-            if (args.src[g].num_tokens != 0) continue;
-            for (uint32_t e = tid; e < E; e += nthreads) {
-                ws.num_routed[g * E + e] = 0;
-                ws.expert_offsets[g * E + e] = 0;
-            }
-        }
-    };
+    for (uint32_t i = tid; i < E; i += nthreads) s_tab[i] = 0;
     lds_barrier();
 
     // One pass over the entries of the step, kBatch loads in flight per lane.
-    const uint32_t rank = blockIdx.x - token_groups;        // receivers only
     // (the first batch in straight-line code: inside the loop the compiler waits for every outstanding
     // load, the rows included, before it uses the first entry)
     auto count_batch = [&](const uint32_t (&expert)[kBatch], uint32_t f0) {
@@ -721,14 +724,9 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8))) void 
         for (uint32_t j = 0; j < kBatch; ++j) {
             const uint32_t x = expert[j];
             if (x >= E) continue;
-            if (receiver) {
-                const uint32_t le = x - rank * Le;   // wraps for experts of lower ranks
-                if (le < Le) atomicAdd(&cnt[my_g * Le + le], 1u);
-            } else {
-                // one word per expert: low half all its entries, high half those before my first token
-                // (a step of this kernel has at most kSingleMaxEntries < 2^16 entries)
-                atomicAdd(&cnt[x], f0 + j * nthreads + tid < my_first ? 0x10001u : 1u);
-            }
+            // one word per expert: low half all its entries, high half those before my first token
+            // (a step of this kernel has at most kSingleMaxEntries < 2^16 entries)
+            atomicAdd(&cnt[x], f0 + j * nthreads + tid < my_first ? 0x10001u : 1u);
         }
     };
     count_batch(early, 0);
@@ -741,17 +739,11 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8))) void 
         }
         count_batch(expert, f0);
     }
-    if (!receiver && tid < my_routes) s_route_expert[tid] = my_expert;
-    if (!receiver && tid < ws.world) {
+    if (tid < my_routes) s_route_expert[tid] = my_expert;
+    if (tid < ws.world) {
         s_dst[tid] = PushDst{my_out_x, my_out_scale, my_out_stride, my_os_elem, my_os_token, my_out_rows, 0};
     }
     lds_barrier();
-
-    if (receiver) {
-        if (fin.recv_mask >> rank & 1) layout_from_totals(fin, ws, rank, cnt, scratch);
-        clear_empty_sources();
-        return;
-    }
 
     // Per expert: padded rows of the experts before it (the difference to the scan
     // at the first expert of a receiver is the expert's first row there).
@@ -770,6 +762,43 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8))) void 
         }
     }
     lds_barrier();
+
+    // The receivers' layouts, by the last wavefront of the first workgroups (workgroup b: receivers b,
+    // b + grid, ...), beside the other wavefronts' work.  With one source everything a receiver needs
+    // is in this workgroup's tables: an expert's rows are its count, its first row the difference of two
+    // values of the scan, and of the other sources (all empty) those the receiver lays out after mine
+    // begin behind my rows (a2a_worker.rs:598-606,669-671,681-694).
+    if (has_duty && tid / kWave == nthreads / kWave - 1) {
+        // Sources without tokens have no workgroup of their own: their tables read as zeros.  (Early in
+        // the kernel's life and spread over workgroups: stores issued at the very end of a kernel delay
+        // the start of the next one.)
+        for (uint32_t g = blockIdx.x; g < G; g += token_groups) {
+            if (args.src[g].num_tokens != 0) continue;
+            for (uint32_t e = lane; e < E; e += kWave) {
+                ws.num_routed[g * E + e] = 0;
+                ws.expert_offsets[g * E + e] = 0;
+            }
+        }
+        for (uint32_t r = blockIdx.x; r < ws.world; r += token_groups) {
+            if (!(fin.recv_mask >> r & 1)) continue;
+            const uint32_t before_mine = ws.laid_before[r * G + my_g];   // sources receiver r lays out before mine
+            const uint32_t base = r * Le < E ? rows_before[r * Le] : 0;
+            for (uint32_t l0 = 0; l0 < Le; l0 += kWave) {
+                const uint32_t le = l0 + lane;
+                const uint32_t e = r * Le + le;
+                if (le >= Le || e >= E) continue;
+                const uint32_t tpe = cnt[e] & 0xFFFFu;
+                const uint32_t poff = rows_before[e] - base;
+                ws.tokens_per_expert[e] = tpe;
+                ws.padded_offset[e] = poff;
+                if (fin.out_num_tokens[r] != nullptr) fin.out_num_tokens[r][le] = (int32_t)tpe;
+                if (poff + tpe > fin.out_rows[r]) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+                for (uint32_t g = 0; g < G; ++g) {
+                    ws.slot_base[g * E + e] = g == my_g || (before_mine >> g & 1) ? poff : poff + tpe;
+                }
+            }
+        }
+    }
 
     // The first workgroup publishes the source's totals (last wavefront).
     if (blockIdx.x == 0 && tid / kWave == nthreads / kWave - 1) {
@@ -810,8 +839,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8))) void 
     }
     lds_barrier();
 
-    // The teams move one token each per round; the rows of the first round are on their way since the head.
-    // (Asking for the rows of the next round before a round stores made the 1024-token step 3.4 us slower.)
+    // The teams move one token each per round; the rows of the first two rounds are on their way since the head.
     for (uint32_t first = 0; first < per_group; first += teams) {
         const uint32_t mine = first + team;                  // which of the workgroup's tokens
         const uint32_t token = first_token + mine;
@@ -827,13 +855,16 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(8))) void 
             push_rows<QUANT, true>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale[team],
                                    s_scale_ptr[team], s_scale_stride[team], team_tid, team_threads, live, pre_a,
                                    pre_b);
+        } else if (first == teams) {
+            push_rows<QUANT, true>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale[team],
+                                   s_scale_ptr[team], s_scale_stride[team], team_tid, team_threads, live, next_a,
+                                   next_b);
         } else {
             push_rows<QUANT>(args, src, token, K, row_ptr, scale_ptr, scale_stride, s_scale[team],
                              s_scale_ptr[team], s_scale_stride[team], team_tid, team_threads, live);
         }
         __syncthreads();   // the team's LDS arrays are reused by the next round
     }
-    clear_empty_sources();
 }
 
 // Pack of a large group step, after a routing launch that left, per chunk, the
@@ -1111,10 +1142,8 @@ hipError_t launch_dispatch_single(const PushArgs &args, const FinalizeArgs &fin,
     const uint32_t team = push_threads(args, quantize);
     const uint32_t per_group = single_tokens_per_group(total_tokens);
     const uint32_t threads = single_threads(team, per_group);
-    const uint32_t blocks = (total_tokens + per_group - 1) / per_group + (fin.recv_mask != 0 ? ws.world : 0);
-    const size_t token_words = 2 * (size_t)ws.num_experts;
-    const size_t receiver_words = (size_t)ws.num_groups * ws.experts_per_rank;
-    const size_t lds = (token_words > receiver_words ? token_words : receiver_words) * sizeof(uint32_t);
+    const uint32_t blocks = (total_tokens + per_group - 1) / per_group;   // the receivers are laid out by the first of them
+    const size_t lds = 2 * (size_t)ws.num_experts * sizeof(uint32_t);
     PushArgs a = args;
     a.single_source = 0;
     for (uint32_t g = 0; g < ws.num_groups; ++g) {
