@@ -972,6 +972,9 @@ int a2a_dispatch_send(a2a_ctx *ctx, uint32_t rank, size_t num_tokens, const void
     if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && stage_send_small_fits(sa, ctx->ws)) {
         e = launch_stage_send_small(sa, ctx->ws, ctx->staging, quantize != 0, s, send_timing);
         if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send_small");
+    } else if (!(c.flags & A2A_FLAG_SEPARATE_ROUTING) && stage_send_single_fits(sa, ctx->ws, quantize != 0)) {
+        e = launch_stage_send_single(sa, ctx->ws, ctx->staging, quantize != 0, s, send_timing);
+        if (e != hipSuccess) return hip_fail(ctx, e, "launch stage_send_single");
     } else {
         RouteArgs ra;
         FinalizeArgs fa;

@@ -97,6 +97,11 @@ hipError_t launch_stage_send(const StageSendArgs &args, const Workspace &ws, con
 bool stage_send_small_fits(const StageSendArgs &args, const Workspace &ws);
 hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                                    bool quantize, hipStream_t stream, KernelTiming timing = KernelTiming());
+// One-launch send for steps of up to 8192 entries that are too large for the small-step kernel
+// (a workgroup counts once for several tokens): whether a step qualifies, and the launch.
+bool stage_send_single_fits(const StageSendArgs &args, const Workspace &ws, bool quantize);
+hipError_t launch_stage_send_single(const StageSendArgs &args, const Workspace &ws, const Staging &st,
+                                    bool quantize, hipStream_t stream, KernelTiming timing = KernelTiming());
 // The send of a large step after launch_route_accumulate(..., for_send = true).
 hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                                      bool quantize, hipStream_t stream, KernelTiming timing = KernelTiming());

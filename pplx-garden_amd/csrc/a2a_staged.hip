@@ -22,9 +22,10 @@ size_t align_up_sz(size_t n, size_t a) { return (n + a - 1) / a * a; }
 template <bool QUANT, bool PRE = false>
 __device__ __forceinline__ void stage_row(const StageSendArgs &args, const Staging &st, uint32_t g, uint32_t token,
                                           uint32_t staging_threads, u32x4 pre_a = u32x4{0, 0, 0, 0},
-                                          u32x4 pre_b = u32x4{0, 0, 0, 0}) {
-    const uint32_t tid = threadIdx.x;
-    if (tid >= staging_threads) return;
+                                          u32x4 pre_b = u32x4{0, 0, 0, 0}, uint32_t first_thread = 0) {
+    // the row is the work of threads first_thread .. first_thread + staging_threads - 1 of the workgroup
+    const uint32_t tid = threadIdx.x - first_thread;
+    if (tid >= staging_threads) return;   // (threads below first_thread wrap around to large numbers)
     const uint32_t lane = tid & (kWave - 1);
     const uint32_t wave = tid / kWave;
     const PushSrc &src = args.src;
@@ -246,6 +247,150 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
         }
     }
     stage_row<QUANT, true>(args, st, g, token, nthreads, pre_a, pre_b);
+}
+
+// The send of a step too large for stage_send_small_kernel and of at most kSendSingleMaxEntries
+// entries (448 to 1024 tokens at top-8), in ONE launch: what makes the small kernel expensive as steps
+// grow is that every token's workgroup counts every entry of the sender; here a workgroup counts once
+// for `per_group` tokens (the host picks it so that the workgroups are about as many as the compute
+// units) and stages them with teams of wavefronts, one token per team and round.  One LDS word per
+// expert holds its entries (low half) and those of the tokens before the workgroup's first (high half).
+// The rows of the first two rounds are asked for at the head and travel while the entries are counted
+// (every barrier up to their use waits for LDS only).  Dynamic LDS: 2 * E words.
+constexpr uint32_t kSendSingleMaxEntries = 8192;
+constexpr uint32_t kSendTokensPerGroup = 4;
+
+template <bool QUANT>
+__global__ __launch_bounds__(1024) void stage_send_single_kernel(const StageSendArgs args, const Workspace ws,
+                                                                 const Staging st, const uint32_t team_threads,
+                                                                 const uint32_t per_group) {
+    extern __shared__ uint32_t s_single[];
+    __shared__ uint32_t s_route_expert[kSendTokensPerGroup * A2A_MAX_EXPERTS_PER_TOKEN];
+    __shared__ uint32_t scratch[kRouteWaves];
+    __shared__ uint32_t s_carry;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nthreads = blockDim.x;
+    const uint32_t E = ws.num_experts, K = ws.topk;
+    const uint32_t g = args.rank / ws.dp_size;
+    const PushSrc &src = args.src;                     // index rows are dense (the host checks)
+    const uint32_t tokens = effective_tokens(src.bound_m, src.num_tokens);
+    const uint32_t flat_entries = tokens * K;
+    const uint32_t first_token = blockIdx.x * per_group;
+    const uint32_t my_first = first_token * K;         // flat index of my first entry
+    if (blockIdx.x != 0 && first_token >= tokens) return;   // nothing to stage; the first workgroup publishes
+
+    constexpr uint32_t kBatch = 10;   // 8192 entries over 896 threads in one batch
+    uint32_t early[kBatch];
+#pragma unroll
+    for (uint32_t j = 0; j < kBatch; ++j) {
+        const uint32_t f = j * nthreads + tid;
+        early[j] = f < flat_entries ? (uint32_t)src.indices[f] : 0xFFFFFFFFu;
+    }
+    const uint32_t my_routes = per_group * K;          // one thread each
+    uint32_t my_expert = 0xFFFFFFFFu;
+    if (tid < my_routes && my_first + tid < flat_entries) my_expert = (uint32_t)src.indices[my_first + tid];
+    const uint32_t teams = nthreads / team_threads;
+    const uint32_t team = tid / team_threads;
+    const uint32_t team_tid = tid - team * team_threads;
+    u32x4 pre_a, pre_b = {0, 0, 0, 0};
+    u32x4 next_a = {0, 0, 0, 0}, next_b = {0, 0, 0, 0};
+    {
+        const uint32_t last_token = src.num_tokens - 1;
+        const uint32_t any_token = first_token + team < src.num_tokens ? first_token + team : last_token;
+        const uint32_t second = first_token + teams + team;
+        const uint8_t *x_row = src.x + (size_t)any_token * src.x_stride;
+        const uint8_t *x_next = src.x + (size_t)(second < src.num_tokens ? second : last_token) * src.x_stride;
+        const bool two_rounds = per_group > teams;     // uniform: a branch, not a select
+        if constexpr (QUANT) {
+            const uint32_t pieces = args.hidden_dim / 16;
+            const size_t at = (size_t)(team_tid < pieces ? team_tid : 0) * 32;
+            if (two_rounds) {
+                next_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_next + at));
+                next_b = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_next + at) + 1);
+            }
+            pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row + at));
+            pre_b = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row + at) + 1);
+        } else {
+            const uint32_t pieces = args.row_bytes / 16;
+            const uint32_t at = team_tid < pieces ? team_tid : 0;
+            if (two_rounds) next_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_next) + at);
+            pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + at);
+        }
+    }
+
+    uint32_t *cnt = s_single;      // [E] low half: entries per expert, high half: those before my first token
+    uint32_t *excl = cnt + E;      // [E] exclusive scan of the entries per expert
+    for (uint32_t i = tid; i < E; i += nthreads) cnt[i] = 0;
+    lds_barrier();
+    auto count_batch = [&](const uint32_t (&expert)[kBatch], uint32_t f0) {
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t x = expert[j];
+            if (x >= E) continue;
+            atomicAdd(&cnt[x], f0 + j * nthreads + tid < my_first ? 0x10001u : 1u);
+        }
+    };
+    count_batch(early, 0);
+    for (uint32_t f0 = kBatch * nthreads; f0 < flat_entries; f0 += kBatch * nthreads) {
+        uint32_t expert[kBatch];
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t f = f0 + j * nthreads + tid;
+            expert[j] = f < flat_entries ? (uint32_t)src.indices[f] : 0xFFFFFFFFu;
+        }
+        count_batch(expert, f0);
+    }
+    if (tid < my_routes) s_route_expert[tid] = my_expert;
+    lds_barrier();
+
+    // Scan over the experts (a2a_dispatch_send.cu:236-242); the first workgroup publishes.
+    uint32_t carry = 0;
+    for (uint32_t e0 = 0; e0 < E; e0 += nthreads) {
+        const uint32_t e = e0 + tid;
+        const uint32_t c = e < E ? cnt[e] & 0xFFFFu : 0;
+        const uint32_t incl = carry + block_inclusive_scan<true>(c, scratch);
+        if (e < E) {
+            excl[e] = incl - c;
+            if (blockIdx.x == 0) {
+                ws.num_routed[g * E + e] = c;
+                ws.expert_offsets[g * E + e] = incl;
+            }
+        }
+        if (e0 + nthreads < E) {   // uniform: another round follows
+            if (tid == nthreads - 1) s_carry = incl;
+            lds_barrier();
+            carry = s_carry;
+        }
+    }
+    lds_barrier();
+
+    // One thread per route of my tokens: its rank inside its expert and the row of the sender's
+    // expert-sorted order it stands for (a2a_dispatch_send.cu:54).
+    if (tid < my_routes && my_first + tid < flat_entries) {
+        uint32_t toff = 0;
+        if (my_expert < E) {
+            uint32_t earlier = 0;
+            for (uint32_t q = 0; q < tid; ++q) earlier += s_route_expert[q] == my_expert ? 1u : 0u;
+            toff = (cnt[my_expert] >> 16) + earlier;
+            st.pos_token[(size_t)g * ws.max_tk + excl[my_expert] + toff] = first_token + tid / K;
+        } else {
+            atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
+        }
+        ws.token_offset[(size_t)g * ws.max_tk + my_first + tid] = toff;
+    }
+
+    // The teams stage one token each per round.
+    for (uint32_t first = 0; first < per_group; first += teams) {
+        const uint32_t token = first_token + first + team;
+        if (first + team >= per_group || token >= tokens) continue;   // (no barrier below: teams work alone)
+        if (first == 0) {
+            stage_row<QUANT, true>(args, st, g, token, team_threads, pre_a, pre_b, team * team_threads);
+        } else if (first == teams) {
+            stage_row<QUANT, true>(args, st, g, token, team_threads, next_a, next_b, team * team_threads);
+        } else {
+            stage_row<QUANT>(args, st, g, token, team_threads, u32x4{0, 0, 0, 0}, u32x4{0, 0, 0, 0}, team * team_threads);
+        }
+    }
 }
 
 // The send of a large step, after a routing launch that left the chunk counts,
@@ -811,34 +956,44 @@ uint32_t block_for_chunks(uint32_t chunks) {
     return threads;
 }
 
-// How the rows of a receiver are shared out.  Few rows (decode): one workgroup
-// per row, as wide as the row needs, because then the latency of a row is what
-// counts.  Many rows: teams of one wavefront, four to a workgroup, each with
-// eight pieces per lane in flight, in workgroups that stride over the rows,
-// because then memory-level parallelism is what counts (measured per receiver,
-// rows of 7 KB: 19 us against 24 us at 4096 rows, 13 against 16 us at 1024).
+// How the rows of a receiver are shared out: the wider the team of wavefronts that shares a row, the
+// shorter the life of a row (what counts when there are few rows), the narrower, the more rows are in
+// flight (what counts when there are many).  The host knows an upper bound of the rows (every copy of
+// every sender); a receiver typically gets 1/N of it, and the team is sized so that those rows give
+// about 4096 wavefronts, as many as the GPU holds at this kernel's occupancy: one wavefront per row from
+// about 4096 rows per receiver on, 2 at 2048, 4 at 1024, up to a team as wide as the row below that
+// (then one workgroup per row).  Measured per step of 8 receivers, rows of 7 KB in / 14 KB back
+// (recv / combine-send, us): 4096 tokens 122 / 198 with one wavefront per row (138 / 210 with two);
+// 2048 tokens 83 / 97 with two (93 / 137 with one, 90 / 123 with four); 1024 tokens 59 / 65 with four
+// (78 / 105 with one, 65 / 77 with two); 512 tokens 50-53 / 48-53 with four to seven (70 / 97 with one);
+// 128 tokens 34 / 31 with the full width (39 / 41 with four).
 constexpr uint32_t kMaxRowWorkgroups = 2048;
-constexpr uint32_t kManyRows = 2048;
 constexpr uint32_t kFewRowWorkgroups = 512;
+constexpr uint32_t kWavefrontsWanted = 4096;
 
 struct RowLaunch {
     uint32_t blocks, threads, team_waves;
 };
 
-RowLaunch row_launch(uint32_t max_rows, uint32_t chunks) {
-    // max_rows is the host's upper bound; a receiver typically gets 1/N of it, and
-    // workgroups without a row still pay for the layout, so the grids stay modest.
+RowLaunch row_launch(uint32_t max_rows, uint32_t chunks, uint32_t world) {
     RowLaunch l;
-    if (max_rows <= kManyRows) {
-        l.threads = block_for_chunks(chunks);
-        l.team_waves = l.threads / kWave;
+    const uint32_t width = block_for_chunks(chunks) / kWave;          // wavefronts that cover a row at one piece a lane
+    const uint32_t typical = (max_rows + world - 1) / world;
+    uint32_t want = 1;
+    while (want < width && want * typical < kWavefrontsWanted) want *= 2;
+    if (want >= width) {
+        // few rows: one workgroup per row, as wide as the row needs
+        l.threads = width * kWave;
+        l.team_waves = width;
         l.blocks = max_rows < kFewRowWorkgroups ? max_rows : kFewRowWorkgroups;
-    } else {
-        l.threads = 4 * kWave;
-        l.team_waves = 1;
-        const uint32_t blocks = (max_rows + 3) / 4;
-        l.blocks = blocks < kMaxRowWorkgroups ? blocks : kMaxRowWorkgroups;
+        return l;
     }
+    l.team_waves = want;
+    const uint32_t waves = want < 4 ? 4 : want;                       // wavefronts of a workgroup
+    l.threads = waves * kWave;
+    const uint32_t teams = waves / want;
+    const uint32_t blocks = (max_rows + teams - 1) / teams;
+    l.blocks = blocks < kMaxRowWorkgroups ? blocks : kMaxRowWorkgroups;
     return l;
 }
 
@@ -984,6 +1139,41 @@ hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &w
     return hipGetLastError();
 }
 
+uint32_t send_single_tokens_per_group(uint32_t tokens) {
+    constexpr uint32_t kComputeUnits = 256;
+    const uint32_t per_group = (tokens + kComputeUnits - 1) / kComputeUnits;
+    return per_group < 1 ? 1 : per_group > kSendTokensPerGroup ? kSendTokensPerGroup : per_group;
+}
+
+bool stage_send_single_fits(const StageSendArgs &args, const Workspace &ws, bool quantize) {
+    const uint64_t T = args.src.num_tokens;
+    const uint32_t team = block_for_chunks(quantize ? args.hidden_dim / 16 : args.row_bytes / 16);
+    const uint32_t per_group = send_single_tokens_per_group((uint32_t)T);
+    uint32_t teams = 1024 / team;
+    if (teams > per_group) teams = per_group;
+    // dense index rows (the entries are read as one flat array), one thread per route of a workgroup's tokens
+    return T != 0 && T * ws.topk <= kSendSingleMaxEntries && args.src.indices_stride == ws.topk &&
+           per_group * ws.topk <= teams * team;
+}
+
+hipError_t launch_stage_send_single(const StageSendArgs &args, const Workspace &ws, const Staging &st,
+                                    bool quantize, hipStream_t stream, KernelTiming timing) {
+    const uint32_t team = block_for_chunks(quantize ? args.hidden_dim / 16 : args.row_bytes / 16);
+    const uint32_t per_group = send_single_tokens_per_group(args.src.num_tokens);
+    uint32_t teams = 1024 / team;
+    if (teams > per_group) teams = per_group;
+    const uint32_t blocks = (args.src.num_tokens + per_group - 1) / per_group;
+    const size_t lds = 2 * (size_t)ws.num_experts * sizeof(uint32_t);
+    if (quantize) {
+        hipExtLaunchKernelGGL(stage_send_single_kernel<true>, dim3(blocks), dim3(teams * team), lds, stream,
+                              timing.start, timing.stop, 0, args, ws, st, team, per_group);
+    } else {
+        hipExtLaunchKernelGGL(stage_send_single_kernel<false>, dim3(blocks), dim3(teams * team), lds, stream,
+                              timing.start, timing.stop, 0, args, ws, st, team, per_group);
+    }
+    return hipGetLastError();
+}
+
 hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                                      bool quantize, hipStream_t stream, KernelTiming timing) {
     uint32_t threads = block_for_chunks(quantize ? args.hidden_dim / 16 : args.row_bytes / 16);
@@ -1006,7 +1196,7 @@ hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace 
 
 hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st, bool first_of_step,
                              hipStream_t stream, KernelTiming timing) {
-    RowLaunch l = row_launch(args.max_rows, args.row_bytes / 16);
+    RowLaunch l = row_launch(args.max_rows, args.row_bytes / 16, ws.world);
     if (l.blocks == 0) l.blocks = 1;    // the counts are handed over even when nothing was sent
     StageRecvArgs a = args;
     a.team_waves = l.team_waves;
@@ -1032,7 +1222,7 @@ hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, con
 hipError_t launch_combine_send(const CombineSendArgs &args, const Workspace &ws, const Staging &st,
                                hipStream_t stream, KernelTiming timing) {
     if (args.max_rows == 0) return hipSuccess;
-    const RowLaunch l = row_launch(args.max_rows, args.row_bytes / 16);
+    const RowLaunch l = row_launch(args.max_rows, args.row_bytes / 16, ws.world);
     CombineSendArgs a = args;
     a.team_waves = l.team_waves;
     hipExtLaunchKernelGGL(combine_send_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, timing.start, timing.stop,

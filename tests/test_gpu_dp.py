@@ -21,6 +21,8 @@ CONFIGS = [
     RefConfig("dp4_two_launch_fp8", 8, 4, 1300, 48, 512, 4, 8, FP8, BF16, F32, node_size=8),
     # one group of 600 tokens x 6: the one-launch dispatch of a larger single source, rows copied as bytes
     RefConfig("dp8_single_group_larger", 8, 8, 600, 24, 256, None, 6, BF16, BF16, None, expert_padding=3),
+    # no dp groups, the caller's scales, 800 tokens a rank: the one-launch send of the split calls copies scale rows
+    RefConfig("dp1_fp8_scales_800", 4, 1, 800, 32, 1024, 8, 8, FP8, BF16, F32, node_size=2),
 ]
 
 
