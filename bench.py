@@ -43,7 +43,7 @@ for _p in (REPO / "pplx-garden_amd", REPO / "pplx-garden_amd" / "benchmarks"):
         sys.path.insert(0, str(_p))
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
-TRAFFIC_PROFILE = REPO / "profiles" / "hbm_traffic_dsv3_prefill_4096_pack_and_combine.md"
+TRAFFIC_PROFILE = REPO / "profiles" / "hbm_traffic_pack_and_combine_dsv3_prefill_4096_and_kimi_1024.md"
 
 
 def algorithmic_bytes(T: int, H: int, K: int):
@@ -86,6 +86,9 @@ def measured_traffic():
     if sha is None or sha.group(1) != kernel_sources_sha256():
         return {}, "the counter summary under profiles/ was taken on other kernel sources"
     out = {m.group(1): int(m.group(2)) for m in re.finditer(r"^traffic_bytes:\s*(\w+)\s*=\s*(\d+)\s*$", text, flags=re.M)}
+    # the other shapes of the baseline: lines "traffic_bytes_<shape>: <kernel>=<bytes>"
+    for m in re.finditer(r"^traffic_bytes_(\w+):\s*(\w+)\s*=\s*(\d+)\s*$", text, flags=re.M):
+        out.setdefault(m.group(1), {})[m.group(2)] = int(m.group(3))
     return out, f"FETCH_SIZE and WRITE_SIZE passes of this build, profiles/{TRAFFIC_PROFILE.name}"
 
 
@@ -698,6 +701,10 @@ def main() -> int:
                           "of every step (each event adds about 3 us)")
         qwen = other_shape(C1, device, args.routings, side_steps, args.warmup, ctx_flags, qwen_label)
         kimi = other_shape(C4, device, args.routings, side_steps, args.warmup, ctx_flags, kimi_label, bar_us=37.0)
+        kimi_d, kimi_c = algorithmic_bytes(C4.num_tokens, C4.hidden_dim, C4.topk)
+        kimi["traffic"] = traffic.get("kimi_1024")      # HBM bytes per launch by kernel, same rule as roofline.traffic
+        kimi["traffic_source"] = traffic_note
+        kimi["algorithmic_bytes_by_kernel"] = {"dispatch_single_kernel": kimi_d, "combine_gather_kernel": kimi_c}
         # The work of the WHOLE group on this GPU: every logical rank sends its 4096 tokens (8 times the
         # bytes of the headline's step, which is one GPU's share).  Not the baseline's configuration;
         # reported beside it as the same kernels' sustained rate over a longer step.

@@ -17,6 +17,10 @@
 //              through another, a wavefront per row: rows of 7392 bytes (what a
 //              rank's split recv moves) and of 14336 bytes (its combine-send)
 //   1024       push and gather over the first 1024 tokens only
+//   launches   what a dependent launch costs by itself: empty kernels of the library's launch shapes
+//              (with 3.8 KB of arguments by value, as the library's) enqueued behind a kernel that
+//              holds the queue for 20 ms, so that the host is ahead and the pace is the GPU's; and
+//              what the events that a launch records at its own start and end read for an empty kernel
 //
 // Every kernel takes the number of its units and returns at once beyond it.
 //
@@ -31,6 +35,7 @@
 //
 // Usage: a2a_ceilings            (prints microseconds and GB/s, median of 20)
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 
 #include <algorithm>
 #include <cstdint>
@@ -170,6 +175,22 @@ __global__ __launch_bounds__(256) void write_streams(u32x4 *out, size_t n16, uin
             }
         }
     }
+}
+
+// The cost of a launch by itself.
+struct Arguments {
+    uint32_t w[960];   // 3840 bytes by value, about what the library's kernels take
+};
+
+__global__ void hold_queue(unsigned long long ticks, uint32_t *out) {   // wall_clock64 counts at 100 MHz
+    const unsigned long long t0 = wall_clock64();
+    while (wall_clock64() - t0 < ticks) {
+    }
+    if (threadIdx.x == 4096) out[0] = 1;
+}
+
+__global__ void empty(Arguments a, uint32_t *out, uint32_t never) {
+    if (threadIdx.x == never) out[0] = a.w[never % 960];
 }
 
 struct Timer {
@@ -340,5 +361,39 @@ int main() {
            (double)kFewTokens * (kInRow + kTopk * kOutRow));
     report("  gather, 1024 tokens", timer.median_us(few_push, few_gather),
            (double)kFewTokens * (kTopk + 1) * kInRow);
+
+    // What a launch costs by itself, for the launch shapes of the library's kernels.
+    std::printf("empty kernels, 3.8 KB of arguments, 1000 dependent launches behind a kernel that holds the queue:\n");
+    {
+        Arguments a = {};
+        uint32_t *flag = reinterpret_cast<uint32_t *>(combined);
+        struct Shape { const char *name; uint32_t blocks, threads; };
+        for (const Shape &sh : {Shape{"136 x 448 (128-token dispatch)", 136, 448}, Shape{"1792 x 64 (128-token gather)", 1792, 64},
+                                Shape{"256 x 896 (1024-token dispatch)", 256, 896}, Shape{"4112 x 448 (4096-token pack)", 4112, 448},
+                                Shape{"57344 x 64 (4096-token gather)", 57344, 64}}) {
+            CHECK(hipStreamSynchronize(s));
+            hipLaunchKernelGGL(hold_queue, dim3(1), dim3(64), 0, s, 2000000ull, flag);
+            CHECK(hipEventRecord(timer.start, s));
+            for (int i = 0; i < 1000; ++i) hipLaunchKernelGGL(empty, dim3(sh.blocks), dim3(sh.threads), 0, s, a, flag, 0xFFFFFu);
+            CHECK(hipEventRecord(timer.stop, s));
+            CHECK(hipEventSynchronize(timer.stop));
+            float ms = 0.0f;
+            CHECK(hipEventElapsedTime(&ms, timer.start, timer.stop));
+            std::printf("  %-50s %7.2f us per launch\n", sh.name, ms);   // ms per 1000 launches = us per launch
+        }
+        hipEvent_t own_start, own_stop;
+        CHECK(hipEventCreate(&own_start));
+        CHECK(hipEventCreate(&own_stop));
+        std::vector<float> own;
+        for (int i = 0; i < 24; ++i) {
+            hipExtLaunchKernelGGL(empty, dim3(136), dim3(448), 0, s, own_start, own_stop, 0, a, flag, 0xFFFFFu);
+            CHECK(hipStreamSynchronize(s));
+            float ms = 0.0f;
+            CHECK(hipEventElapsedTime(&ms, own_start, own_stop));
+            if (i >= 4) own.push_back(ms * 1e3f);
+        }
+        std::sort(own.begin(), own.end());
+        std::printf("  %-50s %7.2f us\n", "between an empty launch's own start and stop events", own[own.size() / 2]);
+    }
     return 0;
 }

@@ -52,3 +52,7 @@ def test_memory_ceilings_program_runs():
         for l in hits:                     # "<name>   <us> us   <GB/s> GB/s": two positive numbers
             us, gbs = float(l.split()[-4]), float(l.split()[-2])
             assert 0.5 < us < 1e4 and 100 < gbs < 8000, l
+    # what a launch costs by itself
+    launches = [l for l in done.stdout.splitlines() if "us per launch" in l]
+    assert len(launches) == 5 and all(0.3 < float(l.split()[-4]) < 100 for l in launches), launches
+    assert any("own start and stop events" in l for l in done.stdout.splitlines())
