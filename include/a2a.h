@@ -64,6 +64,8 @@ typedef enum a2a_status {
 #define A2A_DEV_BAD_EXPERT_ID   1u  /* an index was >= num_experts; that copy was dropped */
 #define A2A_DEV_RECV_OVERFLOW   2u  /* a receive buffer had too few rows; those copies were dropped */
 #define A2A_DEV_BAD_SLOT        4u  /* combine met a slot outside expert_y; it contributed 0 */
+#define A2A_DEV_INTERNAL        0x80000000u /* a kernel gave up waiting for its own wavefronts: the step's
+                                              * results are invalid (a guard against a hang; never observed) */
 
 typedef struct a2a_ctx a2a_ctx;
 

@@ -594,6 +594,341 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
     }
 }
 
+// The quick form of the one-launch dispatch of a small step: ONE source has tokens, its index rows
+// are dense, it quantises, a token has at most eight routes, and the row is one 16-element piece
+// per thread with a wavefront to spare (the host launches one more than the row has pieces for).
+// One workgroup per token, no receiver workgroups.
+//
+// In dispatch_small_kernel every wavefront walks the same chain once its data is there: count, a
+// scan of all experts' rows, its routes, quantise, K stores behind a loop's branches, scales; at
+// 128 tokens that chain was 2.9 us of a 4.1 us kernel with everything it reads already arrived,
+// and the receivers' workgroups, which start last and walk a chain of their own, ended 1.5 us
+// after the last row was out.  Here
+//  - the spare wavefront (the RESOLVER) does not count: from the token's ids it prepares what the
+//    routes need that no count decides (receiver, descriptor, copies of the token to the same
+//    expert at an earlier k), waits until every counting wavefront has said that its entries are
+//    counted (a word in LDS, not a barrier: the counting wavefronts do not wait for each other or
+//    for the resolver here), and then needs five words of the table per lane: a route's first row
+//    is the padded rows of the experts of ITS receiver before it, at most Le - 1 terms, summed by
+//    eight lanes, not a scan over all experts;
+//  - the other wavefronts count their entries, say so, and quantise their piece of the row while
+//    the resolver works; the routes and the scales meet in LDS at the one barrier that follows;
+//  - the K stores of a piece are straight-line code for K = 8;
+//  - with one source a workgroup's own table holds everything a receiver's layout needs: the
+//    resolvers of the first world + G + 1 workgroups write the step's tables, one job each, while
+//    the others store rows (done by all workgroups, a share of the experts each, the same stores
+//    were 0.3 us slower than with receiver workgroups: many wavefronts writing parts of the
+//    same lines).
+// 128 tokens, hidden 7168: 5.95 -> 5.2 us per dispatch at the GPU's own pace; hidden 2048: 5.8 -> 4.6.
+//
+// Dynamic LDS: E words.
+constexpr uint32_t kQuickSpinLimit = 1u << 22;   // (a resolver that gives up flags A2A_DEV_INTERNAL; never seen)
+
+//
+// NB: entries a counting thread asks for at the head (the host picks the smallest of 1, 2, 3, 4, 8
+// that covers the step; entries beyond NB per thread are counted by a loop).  Every one of them
+// costs each wavefront a dozen instructions whether it exists or not, and two wavefronts share a
+// SIMD here.
+template <uint32_t NB>
+__global__ __launch_bounds__(1024) void dispatch_quick_kernel(const PushArgs args, const FinalizeArgs fin,
+                                                              const Workspace ws) {
+    // everything the head of a workgroup needs from the argument block, asked for in one go
+    A2A_PIN(args.single_source);
+    A2A_PIN(args.hidden_dim);
+    A2A_PIN(args.hidden_dim_scale);
+    A2A_PIN(args.single.x);
+    A2A_PIN(args.single.indices);
+    A2A_PIN(args.single.bound_m);
+    A2A_PIN(args.single.x_stride);
+    A2A_PIN(args.single.num_tokens);
+    A2A_PIN(fin.recv_mask);
+    A2A_PIN(ws.world);
+    A2A_PIN(ws.num_groups);
+    A2A_PIN(ws.num_experts);
+    A2A_PIN(ws.topk);
+    A2A_PIN(ws.experts_per_rank);
+    A2A_PIN(ws.le_magic);
+    A2A_PIN(ws.expert_padding);
+    A2A_PIN(ws.max_tk);
+    A2A_PIN(ws.laid_before);
+    A2A_PIN(ws.route_slot);
+    A2A_PIN(ws.token_offset);
+    A2A_PIN(ws.err);
+    // the buffer for the counts and the rows of the receiver this workgroup's resolver may lay out at
+    // its end (receiver blockIdx.x; the index is kept inside the array, whether it is a receiver is
+    // decided at the use)
+    int32_t *const duty_out_tokens = fin.out_num_tokens[blockIdx.x & (kMaxWorld - 1)];
+    const uint32_t duty_out_rows = fin.out_rows[blockIdx.x & (kMaxWorld - 1)];
+    A2A_PIN(duty_out_tokens);
+    A2A_PIN(duty_out_rows);
+
+    extern __shared__ uint32_t s_cnt[];   // [E]: low half of a word the entries of the expert, high half those of
+                                          // the tokens before mine (a step of this kernel has < 2^16 entries)
+    __shared__ float s_scale[kMaxLdsScales];
+    __shared__ uint64_t s_row_ptr[8];
+    __shared__ uint64_t s_scale_ptr[8];
+    __shared__ uint32_t s_scale_stride[8];
+    __shared__ uint32_t s_counted;        // counting wavefronts whose entries are in the table
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nthreads = blockDim.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const uint32_t waves = nthreads / kWave;
+    const bool resolver = wave == waves - 1;
+    const uint32_t counters = nthreads - kWave;   // threads that count entries and move the row
+    const uint32_t G = ws.num_groups, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
+    const uint32_t pad = ws.expert_padding;
+    const PushSrc &one = args.single;
+    const uint32_t my_g = args.single_source - 1;
+    const uint32_t token = blockIdx.x;
+    const uint32_t tokens = one.num_tokens;        // the grid: one workgroup per token
+    const uint32_t entries = tokens * K;           // > 0
+    const uint32_t my_first = token * K;
+    const uint32_t num_chunks = args.hidden_dim / 16;
+
+    // What each kind of wavefront takes from memory, asked for before anything else is done: the
+    // entries, then the thread's piece of the row; the resolver its token's ids (laid out as it uses
+    // them: eight lanes per route), the receivers' descriptors (lane r: receiver r) and which sources
+    // the receiver it may lay out visits before mine.
+    constexpr uint32_t kBatch = NB;
+    uint32_t early[kBatch] = {};
+    u32x4 pre_a = {0, 0, 0, 0}, pre_b = {0, 0, 0, 0};
+    uint32_t id_route = 0xFFFFFFFFu, id_part = 0xFFFFFFFFu, duty_before = 0;
+    uint64_t my_out_x = 0, my_out_scale = 0, my_out_stride = 0;
+    uint32_t my_os_elem = 0, my_os_token = 0, my_out_rows = 0;
+    const uint32_t part = lane & 7, route = lane >> 3;
+    if (!resolver) {
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t f = j * counters + tid;
+            early[j] = (uint32_t)one.indices[f < entries ? f : entries - 1];
+        }
+        if (tid < num_chunks) {
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(one.x + (size_t)token * one.x_stride + (size_t)tid * 32);
+            pre_a = __builtin_nontemporal_load(p);
+            pre_b = __builtin_nontemporal_load(p + 1);
+        }
+    } else {
+        // (the resolver shares its SIMD with a wavefront that quantises while the routes are resolved,
+        // and the routes are what every wavefront of the workgroup waits for)
+        __builtin_amdgcn_s_setprio(3);
+        id_route = (uint32_t)one.indices[my_first + (route < K ? route : 0)];
+        id_part = (uint32_t)one.indices[my_first + (part < K ? part : 0)];
+        const PushDst &dst_of_lane = args.dst[lane < ws.world ? lane : 0];
+        my_out_x = (uint64_t)dst_of_lane.out_x;
+        my_out_scale = (uint64_t)dst_of_lane.out_scale;
+        my_out_stride = dst_of_lane.out_stride;
+        my_os_elem = dst_of_lane.os_stride_elem;
+        my_os_token = dst_of_lane.os_stride_token;
+        my_out_rows = dst_of_lane.out_rows;
+        duty_before = ws.laid_before[(blockIdx.x < ws.world ? blockIdx.x : 0) * G + my_g];
+    }
+    const uint32_t live_tokens = effective_tokens(one.bound_m, tokens);
+    const uint32_t flat_entries = live_tokens * K;
+    const bool live = token < live_tokens;   // uniform
+
+    for (uint32_t i = tid; i < E; i += nthreads) s_cnt[i] = 0;
+    if (tid == 0) s_counted = 0;
+    lds_barrier();
+
+    if (!resolver) {
+        // The first batch in straight-line code: each of its values is waited for by itself, and the
+        // row asked for after them stays in flight meanwhile.
+#pragma unroll
+        for (uint32_t j = 0; j < kBatch; ++j) {
+            const uint32_t f = j * counters + tid;
+            const uint32_t x = f < flat_entries ? early[j] : 0xFFFFFFFFu;
+            if (x < E) atomicAdd(&s_cnt[x], f < my_first ? 0x10001u : 1u);
+        }
+        for (uint32_t f0 = kBatch * counters; f0 < flat_entries; f0 += kBatch * counters) {
+            uint32_t x[kBatch];
+#pragma unroll
+            for (uint32_t j = 0; j < kBatch; ++j) {
+                const uint32_t f = f0 + j * counters + tid;
+                x[j] = f < flat_entries ? (uint32_t)one.indices[f] : 0xFFFFFFFFu;
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < kBatch; ++j) {
+                const uint32_t f = f0 + j * counters + tid;
+                if (x[j] < E) atomicAdd(&s_cnt[x[j]], f < my_first ? 0x10001u : 1u);
+            }
+        }
+        // this wavefront's entries are in the table before its arrival is counted
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (lane == 0) atomicAdd(&s_counted, 1u);
+        if (!live) return;   // nothing to send (uniform; the resolver does not wait at the barrier either)
+
+        float scale;
+        const u32x4 q = quantize16(pre_a, pre_b, &scale);
+        const bool has_piece = tid < num_chunks;
+        if (has_piece && (lane & 7) == 0) s_scale[tid / 8] = scale;
+        lds_barrier();
+        const uint64_t row_ptr = lane < K ? s_row_ptr[lane] : 0;
+        if (K == 8) {
+#pragma unroll
+            for (uint32_t k = 0; k < 8; ++k) {
+                const uint64_t row = read_lane64(row_ptr, k);
+                if (row != 0 && has_piece) store_copy(q, reinterpret_cast<u32x4 *>(row + (size_t)tid * 16));
+            }
+        } else {
+            for (uint32_t k = 0; k < K; ++k) {
+                const uint64_t row = read_lane64(row_ptr, k);
+                if (row != 0 && has_piece) store_copy(q, reinterpret_cast<u32x4 *>(row + (size_t)tid * 16));
+            }
+        }
+        // each copy's scale row goes out as one contiguous run: wavefront w takes routes w, w + waves - 1, ...
+        const uint32_t Hs = args.hidden_dim_scale;
+        for (uint32_t k = wave; k < K; k += waves - 1) {
+            const uint64_t sp = s_scale_ptr[k];
+            const uint32_t ss = s_scale_stride[k];
+            if (sp == 0) continue;
+            for (uint32_t j = lane; j < Hs; j += kWave) reinterpret_cast<float *>(sp)[(size_t)j * ss] = s_scale[j];
+        }
+        return;
+    }
+
+    // ---- the resolver ----
+    // what no count decides: the route's expert and receiver, the receiver's descriptor (from the lane
+    // that holds it), the copies of this token to the same expert at an earlier k
+    const bool in = route < K;
+    const bool route_live = in && id_route < E;
+    const uint32_t e = route_live ? id_route : 0;
+    const uint32_t r = owner_of_expert(ws, e);
+    const uint32_t le = e - r * Le;
+    const uint32_t repeats = group8_sum(part < route && id_part == id_route ? 1u : 0u);
+    PushDst dst;
+    dst.out_x = reinterpret_cast<uint8_t *>(__shfl(my_out_x, (int)r));
+    dst.out_scale = reinterpret_cast<float *>(__shfl(my_out_scale, (int)r));
+    dst.out_stride = __shfl(my_out_stride, (int)r);
+    dst.os_stride_elem = __shfl(my_os_elem, (int)r);
+    dst.os_stride_token = __shfl(my_os_token, (int)r);
+    dst.out_rows = __shfl(my_out_rows, (int)r);
+    dst.pad_ = 0;
+
+    // until the counting wavefronts have all said that their entries are in the table (at the lowest
+    // priority: the wavefront that shares this SIMD is one of those waited for)
+    __builtin_amdgcn_s_setprio(0);
+    for (uint32_t spins = 0; __hip_atomic_load(&s_counted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != waves - 1;) {
+        if (++spins == kQuickSpinLimit) {
+            if (lane == 0) atomicOr(ws.err, A2A_DEV_INTERNAL);
+            break;
+        }
+    }
+    __builtin_amdgcn_s_setprio(3);
+    asm volatile("" ::: "memory");
+
+    // The source's per-expert totals and their scan, for the caller and the combine.
+    auto publish_totals = [&]() {
+        uint32_t run = 0;
+        for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
+            const uint32_t x = e0 + lane;
+            const uint32_t v = x < E ? s_cnt[x] & 0xFFFFu : 0;
+            const uint32_t incl = run + wave_inclusive_scan(v, lane);
+            if (x < E) {
+                ws.num_routed[my_g * E + x] = v;
+                ws.expert_offsets[my_g * E + x] = incl;
+            }
+            run = __shfl(incl, kWave - 1);
+        }
+    };
+    // What the resolver does once the routes are out, while the others store rows: one of the step's
+    // world + G + 1 jobs (with fewer workgroups than jobs, several).  Every store of a job is a run of
+    // neighbouring words from neighbouring lanes.
+    auto duties = [&]() {
+        const uint32_t jobs = ws.world + G + 1;
+        for (uint32_t job = blockIdx.x; job < jobs; job += tokens) {
+            if (job < ws.world) {
+                // a receiver's layout
+                const uint32_t rr = job;
+                if (!(fin.recv_mask >> rr & 1)) continue;
+                const uint32_t before_mine = rr == blockIdx.x ? duty_before : ws.laid_before[rr * G + my_g];
+                int32_t *const out_tokens = rr == blockIdx.x ? duty_out_tokens : fin.out_num_tokens[rr];
+                const uint32_t out_rows = rr == blockIdx.x ? duty_out_rows : fin.out_rows[rr];
+                uint32_t run = 0;
+                for (uint32_t l0 = 0; l0 < Le; l0 += kWave) {
+                    const uint32_t l = l0 + lane;
+                    const uint32_t x = rr * Le + l;
+                    const bool valid = l < Le && x < E;
+                    const uint32_t tpe = valid ? s_cnt[x] & 0xFFFFu : 0;
+                    const uint32_t padded = pad > 1 ? (tpe + pad - 1) / pad * pad : tpe;
+                    const uint32_t incl = run + wave_inclusive_scan(padded, lane);
+                    const uint32_t poff = incl - padded;
+                    if (valid) {
+                        ws.tokens_per_expert[x] = tpe;
+                        ws.padded_offset[x] = poff;
+                        if (out_tokens != nullptr) out_tokens[l] = (int32_t)tpe;
+                        if (poff + tpe > out_rows) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+                        for (uint32_t g = 0; g < G; ++g) {
+                            ws.slot_base[g * E + x] = g == my_g || (before_mine >> g & 1) ? poff : poff + tpe;
+                        }
+                    }
+                    run = __shfl(incl, kWave - 1);
+                }
+            } else if (job < ws.world + G) {
+                // a source without tokens has no workgroup of its own: its tables read as zeros
+                const uint32_t g = job - ws.world;
+                if (g == my_g) continue;
+                for (uint32_t x = lane; x < E; x += kWave) {
+                    ws.num_routed[g * E + x] = 0;
+                    ws.expert_offsets[g * E + x] = 0;
+                }
+            } else {
+                publish_totals();
+            }
+        }
+    };
+    if (!live) {   // nothing to send (uniform)
+        duties();
+        return;
+    }
+
+    // padded rows of the receiver's experts before mine: four terms per lane without a branch
+    // (clamped index, masked value), the rest in a loop
+    const uint32_t mine = s_cnt[e];
+    uint32_t v_rows[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+        const uint32_t n = part + 8 * i;
+        v_rows[i] = s_cnt[r * Le + (n < le ? n : 0)] & 0xFFFFu;
+    }
+    uint32_t base = 0;
+    if (pad > 1) {   // uniform
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) base += part + 8 * i < le ? (v_rows[i] + pad - 1) / pad * pad : 0;
+        for (uint32_t n = 32 + part; n < le; n += 8) base += ((s_cnt[r * Le + n] & 0xFFFFu) + pad - 1) / pad * pad;
+    } else {
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) base += part + 8 * i < le ? v_rows[i] : 0;
+        for (uint32_t n = 32 + part; n < le; n += 8) base += s_cnt[r * Le + n] & 0xFFFFu;
+    }
+    base = group8_sum(base);
+    // copies of my source before this one: earlier tokens, then earlier k of this token
+    const uint32_t toff = route_live ? (mine >> 16) + repeats : 0;
+    uint64_t to_row, to_scale;
+    uint32_t to_stride;
+    uint32_t slot = resolve_copy(dst, ws, base + toff, part == 0 && route_live, &to_row, &to_scale, &to_stride);
+    if (!route_live) {
+        slot = kInvalidSlot;
+        to_row = 0;
+        to_scale = 0;
+        to_stride = 0;
+    }
+    if (part == 0 && in) {
+        s_row_ptr[route] = to_row;
+        s_scale_ptr[route] = to_scale;
+        s_scale_stride[route] = to_stride;
+    }
+    lds_barrier();
+    // (after the barrier: nothing of the resolver's that goes to memory stands between the others and their rows)
+    if (part == 0 && in) {
+        if (!route_live) atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
+        ws.route_slot[(size_t)my_g * ws.max_tk + my_first + route] = slot;
+        ws.token_offset[(size_t)my_g * ws.max_tk + my_first + route] = toff;
+    }
+    duties();
+}
+
 // Routing pass and dispatch pack in ONE launch for steps of ONE source with
 // dense index rows that are too large for dispatch_small_kernel (a mixed batch
 // of about a thousand tokens on one GPU's share).  What makes the one-launch
@@ -1086,6 +1421,23 @@ hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, 
         const size_t tokens_words = 4 * (size_t)ws.num_experts;
         const size_t receiver_words = (size_t)ws.num_groups * ws.experts_per_rank;
         lds = (tokens_words > receiver_words ? tokens_words : receiver_words) * sizeof(uint32_t);
+        // The quick form: a wavefront beside those that move the row, and no receiver workgroups.
+        const uint32_t pieces = args.hidden_dim / 16;
+        if (quantize && ws.topk <= 8 && pieces + kWave <= 1024) {
+            const uint32_t quick_threads = (pieces + kWave - 1) / kWave * kWave + kWave;
+            const uint32_t counters = quick_threads - kWave;
+            const uint32_t per_thread = (total_tokens * ws.topk + counters - 1) / counters;
+#define A2A_LAUNCH_QUICK(NB)                                                                                         \
+    hipExtLaunchKernelGGL(dispatch_quick_kernel<NB>, dim3(total_tokens), dim3(quick_threads),                        \
+                          (size_t)ws.num_experts * sizeof(uint32_t), stream, timing.start, timing.stop, 0, a, fin, ws)
+            if (per_thread <= 1) A2A_LAUNCH_QUICK(1);
+            else if (per_thread == 2) A2A_LAUNCH_QUICK(2);
+            else if (per_thread == 3) A2A_LAUNCH_QUICK(3);
+            else if (per_thread == 4) A2A_LAUNCH_QUICK(4);
+            else A2A_LAUNCH_QUICK(8);
+#undef A2A_LAUNCH_QUICK
+            return hipGetLastError();
+        }
     }
 #define A2A_LAUNCH_SMALL(Q, S)                                                                                       \
     hipExtLaunchKernelGGL((dispatch_small_kernel<Q, S>), dim3(blocks), dim3(threads), lds, stream, timing.start,  \

@@ -44,6 +44,7 @@ TABLE_COMBINE_SEND_OFFSET = 9
 DEV_BAD_EXPERT_ID = 1
 DEV_RECV_OVERFLOW = 2
 DEV_BAD_SLOT = 4
+DEV_INTERNAL = 0x80000000   # a kernel gave up waiting for its own wavefronts (a guard against a hang)
 
 FLAG_PREALLOC_STAGING = 1
 FLAG_SEPARATE_ROUTING = 2   # never take the one-launch paths of small steps

@@ -654,11 +654,14 @@ def test_operator_reports_the_reference_capacities():
                 op.destroy()
 
 
-def _check_single_source(case, sender, bound, strided):
+def _check_single_source(case, sender, bound, strided, repeats=False):
     """Dispatch of a step in which only `sender` has tokens, against the oracle: counts, fp8 bytes, scales,
-    untouched rows, and the sender's routing tables."""
+    untouched rows, and the sender's routing tables.  `repeats`: every third token names its first expert
+    twice (the second copy goes to the next row of that expert)."""
     N, Le, H, Hs, K = case.world_size, case.experts_per_rank, case.hidden_dim, case.hidden_dim_scale, case.topk
     world = [make_world(case, "all")[r] if r == sender else make_world(scaled(case, 0), "all")[r] for r in range(N)]
+    if repeats:
+        world[sender].indices[::3, K - 1] = world[sender].indices[::3, 0]
     rows = rows_needed(case, world)
     inputs = [oracle.RankInput(x=bf16_codes(rd.x), indices=rd.indices.numpy(), bound_m=bound if r == sender else None)
               for r, rd in enumerate(world)]
@@ -686,7 +689,9 @@ def _check_single_source(case, sender, bound, strided):
         ctx = ops[0].context
         assert ctx.status() == 0
         for r in range(N):
-            np.testing.assert_array_equal(t[r]["n"].cpu().numpy(), want[r].num_tokens)
+            n_local = max(0, min(Le, case.num_experts - r * Le))   # (a2a_dispatch_recv.cu:220-224 writes the experts that exist)
+            np.testing.assert_array_equal(t[r]["n"].cpu().numpy()[:n_local], want[r].num_tokens[:n_local])
+            assert (t[r]["n"].cpu().numpy()[n_local:] == -1).all()
             wr = want[r].written
             got_x = t[r]["ox"].view(torch.uint8).cpu().numpy()
             np.testing.assert_array_equal(got_x[wr], want[r].x[wr])
@@ -713,6 +718,22 @@ def test_one_launch_dispatch_with_a_single_source(sender, bound, strided):
     variant runs.  Either way: any rank may be the sender, `bound_m` may shorten the step on the device, and
     the result is the oracle's, bit for bit."""
     _check_single_source(C1, sender, bound, strided)   # 128 tokens, 128 experts over 8 ranks, top-8
+
+
+@pytest.mark.parametrize("tokens,sender,bound,topk,pad,experts,hidden,repeats", [
+    (1, 0, None, 8, 1, 128, 2048, False), (3, 5, None, 8, 16, 128, 2048, True), (128, 2, 100, 5, 8, 250, 7168, False),
+    (200, 7, None, 2, 1, 1024, 2048, True), (17, 1, 16, 8, 128, 64, 384, False), (64, 3, None, 1, 1, 8, 1024, False)],
+    ids=["1_token", "3_tokens_pad16_repeats", "128_top5_pad8_250_experts_bound100", "200_top2_1024_experts_repeats",
+         "17_pad128_bound16", "64_top1_one_expert_a_rank"])
+def test_quick_dispatch_of_a_small_single_source(tokens, sender, bound, topk, pad, experts, hidden, repeats):
+    """A small quantising step of one source with at most eight routes per token takes a kernel in which a
+    spare wavefront per token resolves the routes while the others quantise, and the first workgroups'
+    spare wavefronts write the step's tables.  Fewer workgroups than tables to write, a token that names
+    an expert twice, experts that do not divide among the ranks, more experts per rank than a pass of the
+    route sums covers, a bound on the device, padded receive slots: the oracle's result, bit for bit."""
+    case = replace(scaled(C1, tokens), topk=topk, expert_padding=pad, num_experts=experts, hidden_dim=hidden,
+                   name=f"quick_{tokens}")
+    _check_single_source(case, sender, bound, False, repeats)
 
 
 @pytest.mark.parametrize("tokens,sender,bound,topk,pad", [(700, 2, None, 8, 1), (1024, 0, None, 8, 16), (702, 5, 333, 8, 1),
