@@ -1202,6 +1202,327 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(7))) void 
     }
 }
 
+// The same division of labour for the larger steps of one source that dispatch_single_kernel serves
+// (448 to 1024 tokens at top-8): a workgroup counts the step's entries once for `per_group` tokens,
+// its teams of wavefronts (one token each per round, at most two rounds) quantise both rounds' pieces
+// while the spare wavefront resolves the per_group * K <= 32 routes, eight, four or two lanes per
+// route, and after the one barrier the teams only store.  The resolvers of the first workgroups
+// write the step's tables.  1024 tokens, hidden 7168, 384 experts over 16 ranks: the head of the
+// kernel (everything in front of the first store) shrinks by about a microsecond.
+//
+// Dynamic LDS: E words.
+constexpr uint32_t kTeamsMaxRoutes = 32;
+constexpr uint32_t kTeamsMaxScales = 128;   // scale groups of a row of at most (1024 - 64) pieces
+
+template <uint32_t NB, uint32_t ROUNDS>
+__global__ __launch_bounds__(1024) void dispatch_teams_kernel(const PushArgs args, const FinalizeArgs fin,
+                                                              const Workspace ws, const uint32_t team_threads,
+                                                              const uint32_t per_group) {
+    A2A_PIN(args.single_source);
+    A2A_PIN(args.hidden_dim);
+    A2A_PIN(args.hidden_dim_scale);
+    A2A_PIN(args.single.x);
+    A2A_PIN(args.single.indices);
+    A2A_PIN(args.single.bound_m);
+    A2A_PIN(args.single.x_stride);
+    A2A_PIN(args.single.num_tokens);
+    A2A_PIN(fin.recv_mask);
+    A2A_PIN(ws.world);
+    A2A_PIN(ws.num_groups);
+    A2A_PIN(ws.num_experts);
+    A2A_PIN(ws.topk);
+    A2A_PIN(ws.experts_per_rank);
+    A2A_PIN(ws.le_magic);
+    A2A_PIN(ws.expert_padding);
+    A2A_PIN(ws.max_tk);
+    A2A_PIN(ws.laid_before);
+    A2A_PIN(ws.route_slot);
+    A2A_PIN(ws.token_offset);
+    A2A_PIN(ws.err);
+    int32_t *const duty_out_tokens = fin.out_num_tokens[blockIdx.x & (kMaxWorld - 1)];
+    const uint32_t duty_out_rows = fin.out_rows[blockIdx.x & (kMaxWorld - 1)];
+    A2A_PIN(duty_out_tokens);
+    A2A_PIN(duty_out_rows);
+
+    extern __shared__ uint32_t s_cnt[];   // [E]: low half the entries of the expert, high half those before my first token
+    __shared__ float s_scale[ROUNDS][kTokensPerGroup][kTeamsMaxScales];   // [round][team]
+    __shared__ uint64_t s_row_ptr[kTeamsMaxRoutes];
+    __shared__ uint64_t s_scale_ptr[kTeamsMaxRoutes];
+    __shared__ uint32_t s_scale_stride[kTeamsMaxRoutes];
+    __shared__ uint32_t s_route_expert[kTeamsMaxRoutes];
+    __shared__ uint32_t s_counted;
+
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nthreads = blockDim.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const uint32_t waves = nthreads / kWave;
+    const bool resolver = wave == waves - 1;
+    const uint32_t counters = nthreads - kWave;          // threads that count entries and move rows
+    const uint32_t teams = counters / team_threads;
+    const uint32_t team = tid / team_threads;            // (row wavefronts)
+    const uint32_t team_tid = tid - team * team_threads;
+    const uint32_t G = ws.num_groups, E = ws.num_experts, K = ws.topk, Le = ws.experts_per_rank;
+    const uint32_t pad = ws.expert_padding;
+    const PushSrc &one = args.single;
+    const uint32_t my_g = args.single_source - 1;
+    const uint32_t tokens = one.num_tokens;
+    const uint32_t entries = tokens * K;                 // > 0
+    const uint32_t first_token = blockIdx.x * per_group;
+    const uint32_t my_first = first_token * K;           // flat index of my first entry
+    const uint32_t routes = per_group * K;               // <= kTeamsMaxRoutes
+    const uint32_t num_chunks = args.hidden_dim / 16;
+    const uint32_t token_groups = gridDim.x;
+
+    // lanes of the resolver per route: 8, 4 or 2
+    const uint32_t lpr_log = routes <= 8 ? 3 : routes <= 16 ? 2 : 1;
+    const uint32_t part = lane & ((1u << lpr_log) - 1), route = lane >> lpr_log;
+    const uint32_t lpr = 1u << lpr_log;
+
+    uint32_t early[NB] = {};
+    u32x4 pre_a[ROUNDS], pre_b[ROUNDS];
+#pragma unroll
+    for (uint32_t rd = 0; rd < ROUNDS; ++rd) {
+        pre_a[rd] = u32x4{0, 0, 0, 0};
+        pre_b[rd] = u32x4{0, 0, 0, 0};
+    }
+    uint32_t id_route = 0xFFFFFFFFu, duty_before = 0;
+    uint64_t my_out_x = 0, my_out_scale = 0, my_out_stride = 0;
+    uint32_t my_os_elem = 0, my_os_token = 0, my_out_rows = 0;
+    if (!resolver) {
+#pragma unroll
+        for (uint32_t j = 0; j < NB; ++j) {
+            const uint32_t f = j * counters + tid;
+            early[j] = (uint32_t)one.indices[f < entries ? f : entries - 1];
+        }
+        // the pieces of both rounds' rows, the later round first (it is needed later); a team without a
+        // token asks for a row that exists and ignores it
+#pragma unroll
+        for (uint32_t i = 0; i < ROUNDS; ++i) {
+            const uint32_t rd = ROUNDS - 1 - i;
+            const uint32_t t = first_token + rd * teams + team;
+            const u32x4 *p = reinterpret_cast<const u32x4 *>(one.x + (size_t)(t < tokens ? t : tokens - 1) * one.x_stride +
+                                                             (size_t)(team_tid < num_chunks ? team_tid : 0) * 32);
+            pre_a[rd] = __builtin_nontemporal_load(p);
+            pre_b[rd] = __builtin_nontemporal_load(p + 1);
+        }
+    } else {
+        __builtin_amdgcn_s_setprio(3);
+        const uint32_t f = my_first + route;
+        id_route = (uint32_t)one.indices[f < entries ? f : entries - 1];
+        const PushDst &dst_of_lane = args.dst[lane < ws.world ? lane : 0];
+        my_out_x = (uint64_t)dst_of_lane.out_x;
+        my_out_scale = (uint64_t)dst_of_lane.out_scale;
+        my_out_stride = dst_of_lane.out_stride;
+        my_os_elem = dst_of_lane.os_stride_elem;
+        my_os_token = dst_of_lane.os_stride_token;
+        my_out_rows = dst_of_lane.out_rows;
+        duty_before = ws.laid_before[(blockIdx.x < ws.world ? blockIdx.x : 0) * G + my_g];
+    }
+    const uint32_t live_tokens = effective_tokens(one.bound_m, tokens);
+    const uint32_t flat_entries = live_tokens * K;
+    const bool group_live = first_token < live_tokens;   // uniform
+
+    for (uint32_t i = tid; i < E; i += nthreads) s_cnt[i] = 0;
+    if (tid == 0) s_counted = 0;
+    lds_barrier();
+
+    if (!resolver) {
+#pragma unroll
+        for (uint32_t j = 0; j < NB; ++j) {
+            const uint32_t f = j * counters + tid;
+            const uint32_t x = f < flat_entries ? early[j] : 0xFFFFFFFFu;
+            if (x < E) atomicAdd(&s_cnt[x], f < my_first ? 0x10001u : 1u);
+        }
+        for (uint32_t f0 = NB * counters; f0 < flat_entries; f0 += counters) {
+            const uint32_t f = f0 + tid;
+            const uint32_t x = f < flat_entries ? (uint32_t)one.indices[f] : 0xFFFFFFFFu;
+            if (x < E) atomicAdd(&s_cnt[x], f < my_first ? 0x10001u : 1u);
+        }
+        // this wavefront's entries are in the table before its arrival is counted
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (lane == 0) atomicAdd(&s_counted, 1u);
+        if (!group_live) return;   // nothing to send (uniform; the resolver does not wait at the barrier either)
+
+        const bool has_piece = team_tid < num_chunks;
+        u32x4 q[ROUNDS];
+#pragma unroll
+        for (uint32_t rd = 0; rd < ROUNDS; ++rd) {
+            float scale;
+            q[rd] = quantize16(pre_a[rd], pre_b[rd], &scale);
+            if (has_piece && (lane & 7) == 0) s_scale[rd][team][team_tid / 8] = scale;
+        }
+        lds_barrier();
+        const uint32_t Hs = args.hidden_dim_scale;
+        const uint32_t team_waves = team_threads / kWave, team_wave = team_tid / kWave;
+#pragma unroll
+        for (uint32_t rd = 0; rd < ROUNDS; ++rd) {
+            const uint32_t mine = rd * teams + team;   // which of the workgroup's tokens
+            if (mine >= per_group || first_token + mine >= live_tokens) continue;   // uniform in a team
+            const uint64_t row_ptr = lane < K ? s_row_ptr[mine * K + lane] : 0;
+            if (K == 8) {
+#pragma unroll
+                for (uint32_t k = 0; k < 8; ++k) {
+                    const uint64_t row = read_lane64(row_ptr, k);
+                    if (row != 0 && has_piece) store_copy(q[rd], reinterpret_cast<u32x4 *>(row + (size_t)team_tid * 16));
+                }
+            } else {
+                for (uint32_t k = 0; k < K; ++k) {
+                    const uint64_t row = read_lane64(row_ptr, k);
+                    if (row != 0 && has_piece) store_copy(q[rd], reinterpret_cast<u32x4 *>(row + (size_t)team_tid * 16));
+                }
+            }
+            // each copy's scale row goes out as one contiguous run: wavefront w of the team takes routes w, w + team_waves, ...
+            for (uint32_t k = team_wave; k < K; k += team_waves) {
+                const uint64_t sp = s_scale_ptr[mine * K + k];
+                const uint32_t ss = s_scale_stride[mine * K + k];
+                if (sp == 0) continue;
+                for (uint32_t j = lane; j < Hs; j += kWave) {
+                    reinterpret_cast<float *>(sp)[(size_t)j * ss] = s_scale[rd][team][j];
+                }
+            }
+        }
+        return;
+    }
+
+    // ---- the resolver ----
+    auto group_sum = [&](uint32_t v) {
+        v += dpp_move_u32<0xB1>(v);                      // quad_perm [1,0,3,2]
+        if (lpr_log >= 2) v += dpp_move_u32<0x4E>(v);    // quad_perm [2,3,0,1]
+        if (lpr_log >= 3) v += dpp_move_u32<0x141>(v);   // row_half_mirror
+        return v;
+    };
+    const bool in = route < routes && my_first + route < flat_entries;
+    const bool route_live = in && id_route < E;
+    const uint32_t e = route_live ? id_route : 0;
+    const uint32_t r = owner_of_expert(ws, e);
+    const uint32_t le = e - r * Le;
+    // copies of my tokens to the same expert at an earlier route of the workgroup
+    if (part == 0 && route < kTeamsMaxRoutes) s_route_expert[route] = in ? id_route : 0xFFFFFFFFu;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    uint32_t earlier = 0;
+    for (uint32_t qd = part; qd < route && qd < kTeamsMaxRoutes; qd += lpr) earlier += s_route_expert[qd] == id_route ? 1u : 0u;
+    earlier = group_sum(earlier);
+    PushDst dst;
+    dst.out_x = reinterpret_cast<uint8_t *>(__shfl(my_out_x, (int)r));
+    dst.out_scale = reinterpret_cast<float *>(__shfl(my_out_scale, (int)r));
+    dst.out_stride = __shfl(my_out_stride, (int)r);
+    dst.os_stride_elem = __shfl(my_os_elem, (int)r);
+    dst.os_stride_token = __shfl(my_os_token, (int)r);
+    dst.out_rows = __shfl(my_out_rows, (int)r);
+    dst.pad_ = 0;
+
+    __builtin_amdgcn_s_setprio(0);
+    for (uint32_t spins = 0; __hip_atomic_load(&s_counted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != waves - 1;) {
+        if (++spins == kQuickSpinLimit) {
+            if (lane == 0) atomicOr(ws.err, A2A_DEV_INTERNAL);
+            break;
+        }
+    }
+    __builtin_amdgcn_s_setprio(3);
+    asm volatile("" ::: "memory");
+
+    auto publish_totals = [&]() {
+        uint32_t run = 0;
+        for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
+            const uint32_t x = e0 + lane;
+            const uint32_t v = x < E ? s_cnt[x] & 0xFFFFu : 0;
+            const uint32_t incl = run + wave_inclusive_scan(v, lane);
+            if (x < E) {
+                ws.num_routed[my_g * E + x] = v;
+                ws.expert_offsets[my_g * E + x] = incl;
+            }
+            run = __shfl(incl, kWave - 1);
+        }
+    };
+    auto duties = [&]() {
+        const uint32_t jobs = ws.world + G + 1;
+        for (uint32_t job = blockIdx.x; job < jobs; job += token_groups) {
+            if (job < ws.world) {
+                const uint32_t rr = job;
+                if (!(fin.recv_mask >> rr & 1)) continue;
+                const uint32_t before_mine = rr == blockIdx.x ? duty_before : ws.laid_before[rr * G + my_g];
+                int32_t *const out_tokens = rr == blockIdx.x ? duty_out_tokens : fin.out_num_tokens[rr];
+                const uint32_t out_rows = rr == blockIdx.x ? duty_out_rows : fin.out_rows[rr];
+                uint32_t run = 0;
+                for (uint32_t l0 = 0; l0 < Le; l0 += kWave) {
+                    const uint32_t l = l0 + lane;
+                    const uint32_t x = rr * Le + l;
+                    const bool valid = l < Le && x < E;
+                    const uint32_t tpe = valid ? s_cnt[x] & 0xFFFFu : 0;
+                    const uint32_t padded = pad > 1 ? (tpe + pad - 1) / pad * pad : tpe;
+                    const uint32_t incl = run + wave_inclusive_scan(padded, lane);
+                    const uint32_t poff = incl - padded;
+                    if (valid) {
+                        ws.tokens_per_expert[x] = tpe;
+                        ws.padded_offset[x] = poff;
+                        if (out_tokens != nullptr) out_tokens[l] = (int32_t)tpe;
+                        if (poff + tpe > out_rows) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+                        for (uint32_t g = 0; g < G; ++g) {
+                            ws.slot_base[g * E + x] = g == my_g || (before_mine >> g & 1) ? poff : poff + tpe;
+                        }
+                    }
+                    run = __shfl(incl, kWave - 1);
+                }
+            } else if (job < ws.world + G) {
+                const uint32_t g = job - ws.world;
+                if (g == my_g) continue;
+                for (uint32_t x = lane; x < E; x += kWave) {
+                    ws.num_routed[g * E + x] = 0;
+                    ws.expert_offsets[g * E + x] = 0;
+                }
+            } else {
+                publish_totals();
+            }
+        }
+    };
+    if (!group_live) {   // nothing to send (uniform)
+        duties();
+        return;
+    }
+
+    const uint32_t mine = s_cnt[e];
+    uint32_t v_rows[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; ++i) {
+        const uint32_t n = part + lpr * i;
+        v_rows[i] = s_cnt[r * Le + (n < le ? n : 0)] & 0xFFFFu;
+    }
+    uint32_t base = 0;
+    if (pad > 1) {   // uniform
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) base += part + lpr * i < le ? (v_rows[i] + pad - 1) / pad * pad : 0;
+        for (uint32_t n = 4 * lpr + part; n < le; n += lpr) base += ((s_cnt[r * Le + n] & 0xFFFFu) + pad - 1) / pad * pad;
+    } else {
+#pragma unroll
+        for (uint32_t i = 0; i < 4; ++i) base += part + lpr * i < le ? v_rows[i] : 0;
+        for (uint32_t n = 4 * lpr + part; n < le; n += lpr) base += s_cnt[r * Le + n] & 0xFFFFu;
+    }
+    base = group_sum(base);
+    const uint32_t toff = route_live ? (mine >> 16) + earlier : 0;
+    uint64_t to_row, to_scale;
+    uint32_t to_stride;
+    uint32_t slot = resolve_copy(dst, ws, base + toff, part == 0 && route_live, &to_row, &to_scale, &to_stride);
+    if (!route_live) {
+        slot = kInvalidSlot;
+        to_row = 0;
+        to_scale = 0;
+        to_stride = 0;
+    }
+    if (part == 0 && route < routes) {
+        s_row_ptr[route] = to_row;
+        s_scale_ptr[route] = to_scale;
+        s_scale_stride[route] = to_stride;
+    }
+    lds_barrier();
+    if (part == 0 && in) {
+        if (!route_live) atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
+        ws.route_slot[(size_t)my_g * ws.max_tk + my_first + route] = slot;
+        ws.token_offset[(size_t)my_g * ws.max_tk + my_first + route] = toff;
+    }
+    duties();
+}
+
 // Pack of a large group step, after a routing launch that left, per chunk, the
 // histogram and the rank of every entry inside its chunk, and, for the whole
 // step, the totals per (source, expert) and per expert.  No launch in between
@@ -1502,6 +1823,32 @@ hipError_t launch_dispatch_single(const PushArgs &args, const FinalizeArgs &fin,
         if (args.src[g].num_tokens != 0) a.single_source = g + 1;
     }
     a.single = args.src[a.single_source - 1];
+    // The form with a spare wavefront per workgroup that resolves the routes while the teams quantise:
+    // at most eight routes a token, 32 a workgroup, and two rounds.
+    if (quantize && ws.topk <= 8 && per_group * ws.topk <= kTeamsMaxRoutes && team + kWave <= 1024) {
+        uint32_t teams = (1024 - kWave) / team;
+        if (teams > per_group) teams = per_group;
+        const uint32_t rounds = (per_group + teams - 1) / teams;
+        const uint32_t counters = teams * team;
+        const uint32_t per_thread = (total_tokens * ws.topk + counters - 1) / counters;
+        if (rounds <= 2 && args.hidden_dim / 128 <= kTeamsMaxScales) {
+            const size_t cnt_bytes = (size_t)ws.num_experts * sizeof(uint32_t);
+#define A2A_LAUNCH_TEAMS(NB, R)                                                                                   \
+    hipExtLaunchKernelGGL((dispatch_teams_kernel<NB, R>), dim3(blocks), dim3(counters + kWave), cnt_bytes, stream, \
+                          timing.start, timing.stop, 0, a, fin, ws, team, per_group)
+            if (rounds == 1) {
+                if (per_thread <= 5) A2A_LAUNCH_TEAMS(5, 1);
+                else if (per_thread <= 10) A2A_LAUNCH_TEAMS(10, 1);
+                else A2A_LAUNCH_TEAMS(16, 1);
+            } else {
+                if (per_thread <= 5) A2A_LAUNCH_TEAMS(5, 2);
+                else if (per_thread <= 10) A2A_LAUNCH_TEAMS(10, 2);
+                else A2A_LAUNCH_TEAMS(16, 2);
+            }
+#undef A2A_LAUNCH_TEAMS
+            return hipGetLastError();
+        }
+    }
     if (quantize) {
         hipExtLaunchKernelGGL(dispatch_single_kernel<true>, dim3(blocks), dim3(threads), lds, stream, timing.start,
                               timing.stop, 0, a, fin, ws, team, per_group);

@@ -746,3 +746,13 @@ def test_one_launch_dispatch_of_a_larger_single_source(tokens, sender, bound, to
     of zero and one, odd top-k, padded receive slots: the oracle's result, bit for bit."""
     case = replace(scaled(C1, tokens), topk=topk, expert_padding=pad, name=f"single_{tokens}")
     _check_single_source(case, sender, bound, False)
+
+
+@pytest.mark.parametrize("tokens,topk,hidden", [(900, 8, 7168), (500, 3, 2048), (1024, 8, 256)],
+                         ids=["900_two_rounds", "500_top3_four_teams", "1024_small_rows"])
+def test_larger_single_source_with_experts_named_twice(tokens, topk, hidden):
+    """The same steps with tokens that name an expert twice: the second copy takes the next row of that
+    expert, also when the two routes belong to different tokens of one workgroup's share."""
+    case = replace(scaled(C1, tokens), topk=topk, hidden_dim=hidden, name=f"single_twice_{tokens}")
+    _check_single_source(case, 3, None, False, repeats=True)
+
