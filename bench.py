@@ -276,6 +276,35 @@ def time_graph_replay(wl: Workload, steps: int, warmup: int):
     return wall_s / (replays * n), replays * n
 
 
+def time_gpu_pace(wl: Workload, batches: int = 5, steps_each: int = 100):
+    """The GPU's own pace per step: `steps_each` steps are enqueued behind a kernel that holds the queue
+    for a few milliseconds, so the host is ahead of the GPU for all of them, and two events around them
+    give the time the GPU took.  For steps of about 10 us the host's share of a step (two calls through
+    ctypes and the launches behind them, 7 to 10 us on this pool's hosts) is of the same size as the
+    GPU's, and the wall time of a loop then says which host the box has.  Returns the median over
+    `batches` in microseconds, or None where torch has no such kernel."""
+    import torch
+    hold = getattr(torch.cuda, "_sleep", None)
+    if hold is None:
+        return None
+    stream = torch.cuda.current_stream(wl.device).cuda_stream
+    paces = []
+    for _ in range(batches):
+        first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        hold(20_000_000)
+        first.record()
+        for i in range(steps_each):
+            wl.step(i, stream)
+        last.record()
+        torch.cuda.synchronize(wl.device)
+        paces.append(first.elapsed_time(last) * 1e3 / steps_each)
+    flags = wl.ctx.status(stream)
+    if flags:
+        raise RuntimeError(f"device error flags {flags}")
+    paces.sort()
+    return paces[len(paces) // 2]
+
+
 def cpu_baseline(case, rd, reps: int, threads: int = 1):
     """The oracle's C restatement on the same batch; best of `reps`.  Returns seconds per step and the
     seconds of its routing part (histogram, ranks, receiver layout: what the reference does on one host
@@ -368,6 +397,7 @@ def other_shape(case, device, routings: int, steps: int, warmup: int, ctx_flags:
     _, d, c, b, p, g, _ = time_workload(wl, steps, warmup, kernel_every=4, call_every=1)
     w, _, _, _, _, _, _ = time_workload(wl, steps, warmup)
     graph_s, _ = time_graph_replay(wl, steps, warmup)
+    pace_us = time_gpu_pace(wl) if w / steps < 100e-6 else None
     wl.close()
     d_bytes, c_bytes = algorithmic_bytes(case.num_tokens * num_senders, case.hidden_dim, case.topk)
     step_us = w / steps * 1e6
@@ -375,6 +405,7 @@ def other_shape(case, device, routings: int, steps: int, warmup: int, ctx_flags:
         "workload": label,
         "step_us_wall": round(step_us, 2),
         "step_us_graph_replay": round(graph_s * 1e6, 2),
+        "step_us_gpu_pace": None if pace_us is None else round(pace_us, 2),
         "pack_kernel_us_mean": round(Statistics.create(p).mean, 2),
         "gather_kernel_us_mean": round(Statistics.create(g).mean, 2),
         "kernel_samples": len(g),
@@ -698,13 +729,16 @@ def main() -> int:
         decode["note"] = ("working set (26 MB) fits the 256 MB Infinity Cache and is not flushed between steps; "
                           "step_us_wall is wall time over steps without events, the kernel figures come from "
                           "events the launches record themselves, the p50 figures from events around the calls "
-                          "of every step (each event adds about 3 us)")
+                          "of every step (each event adds about 3 us); step_us_gpu_pace is the time per step "
+                          "between two events when the steps are enqueued behind a kernel that holds the queue, "
+                          "i.e. with the host ahead of the GPU (the host's share of such a step, two calls "
+                          "through ctypes and their launches, is 7-10 us on this pool's hosts)")
         qwen = other_shape(C1, device, args.routings, side_steps, args.warmup, ctx_flags, qwen_label)
         kimi = other_shape(C4, device, args.routings, side_steps, args.warmup, ctx_flags, kimi_label, bar_us=37.0)
         kimi_d, kimi_c = algorithmic_bytes(C4.num_tokens, C4.hidden_dim, C4.topk)
         kimi["traffic"] = traffic.get("kimi_1024")      # HBM bytes per launch by kernel, same rule as roofline.traffic
         kimi["traffic_source"] = traffic_note
-        kimi["algorithmic_bytes_by_kernel"] = {"dispatch_single_kernel": kimi_d, "combine_gather_kernel": kimi_c}
+        kimi["algorithmic_bytes_by_kernel"] = {"dispatch_teams_kernel": kimi_d, "combine_gather_kernel": kimi_c}
         # The work of the WHOLE group on this GPU: every logical rank sends its 4096 tokens (8 times the
         # bytes of the headline's step, which is one GPU's share).  Not the baseline's configuration;
         # reported beside it as the same kernels' sustained rate over a longer step.
