@@ -629,7 +629,10 @@ constexpr uint32_t kQuickSpinLimit = 1u << 22;   // (a resolver that gives up fl
 // that covers the step; entries beyond NB per thread are counted by a loop).  Every one of them
 // costs each wavefront a dozen instructions whether it exists or not, and two wavefronts share a
 // SIMD here.
-template <uint32_t NB>
+//
+// QUANT false: the rows travel as they are (the caller's fp8 bytes, or any other element type), one
+// 16-byte piece per thread, and the caller's scales, if it passed any, are copied beside them.
+template <uint32_t NB, bool QUANT>
 __global__ __launch_bounds__(1024) void dispatch_quick_kernel(const PushArgs args, const FinalizeArgs fin,
                                                               const Workspace ws) {
     // everything the head of a workgroup needs from the argument block, asked for in one go
@@ -641,6 +644,12 @@ __global__ __launch_bounds__(1024) void dispatch_quick_kernel(const PushArgs arg
     A2A_PIN(args.single.bound_m);
     A2A_PIN(args.single.x_stride);
     A2A_PIN(args.single.num_tokens);
+    if constexpr (!QUANT) {
+        A2A_PIN(args.row_bytes);
+        A2A_PIN(args.single.x_scale);
+        A2A_PIN(args.single.xs_stride_elem);
+        A2A_PIN(args.single.xs_stride_token);
+    }
     A2A_PIN(fin.recv_mask);
     A2A_PIN(ws.world);
     A2A_PIN(ws.num_groups);
@@ -685,7 +694,8 @@ __global__ __launch_bounds__(1024) void dispatch_quick_kernel(const PushArgs arg
     const uint32_t tokens = one.num_tokens;        // the grid: one workgroup per token
     const uint32_t entries = tokens * K;           // > 0
     const uint32_t my_first = token * K;
-    const uint32_t num_chunks = args.hidden_dim / 16;
+    const uint32_t num_chunks = QUANT ? args.hidden_dim / 16 : args.row_bytes / 16;   // pieces of a row, one per thread
+    const uint32_t Hs = args.hidden_dim_scale;
 
     // What each kind of wavefront takes from memory, asked for before anything else is done: the
     // entries, then the thread's piece of the row; the resolver its token's ids (laid out as it uses
@@ -705,9 +715,19 @@ __global__ __launch_bounds__(1024) void dispatch_quick_kernel(const PushArgs arg
             early[j] = (uint32_t)one.indices[f < entries ? f : entries - 1];
         }
         if (tid < num_chunks) {
-            const u32x4 *p = reinterpret_cast<const u32x4 *>(one.x + (size_t)token * one.x_stride + (size_t)tid * 32);
-            pre_a = __builtin_nontemporal_load(p);
-            pre_b = __builtin_nontemporal_load(p + 1);
+            if constexpr (QUANT) {
+                const u32x4 *p = reinterpret_cast<const u32x4 *>(one.x + (size_t)token * one.x_stride + (size_t)tid * 32);
+                pre_a = __builtin_nontemporal_load(p);
+                pre_b = __builtin_nontemporal_load(p + 1);
+            } else {
+                pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(one.x + (size_t)token * one.x_stride) + tid);
+            }
+        }
+        if constexpr (!QUANT) {
+            // the caller's scales of this token (one per thread; kept in pre_b's first word)
+            if (one.x_scale != nullptr && tid < Hs && tid < (uint32_t)kMaxLdsScales) {
+                pre_b.x = __float_as_uint(one.x_scale[(size_t)token * one.xs_stride_token + (size_t)tid * one.xs_stride_elem]);
+            }
         }
     } else {
         // (the resolver shares its SIMD with a wavefront that quantises while the routes are resolved,
@@ -759,10 +779,16 @@ __global__ __launch_bounds__(1024) void dispatch_quick_kernel(const PushArgs arg
         if (lane == 0) atomicAdd(&s_counted, 1u);
         if (!live) return;   // nothing to send (uniform; the resolver does not wait at the barrier either)
 
-        float scale;
-        const u32x4 q = quantize16(pre_a, pre_b, &scale);
         const bool has_piece = tid < num_chunks;
-        if (has_piece && (lane & 7) == 0) s_scale[tid / 8] = scale;
+        u32x4 q;
+        if constexpr (QUANT) {
+            float scale;
+            q = quantize16(pre_a, pre_b, &scale);
+            if (has_piece && (lane & 7) == 0) s_scale[tid / 8] = scale;
+        } else {
+            q = pre_a;
+            if (tid < Hs && tid < (uint32_t)kMaxLdsScales) s_scale[tid] = __uint_as_float(pre_b.x);
+        }
         lds_barrier();
         const uint64_t row_ptr = lane < K ? s_row_ptr[lane] : 0;
         if (K == 8) {
@@ -778,7 +804,7 @@ __global__ __launch_bounds__(1024) void dispatch_quick_kernel(const PushArgs arg
             }
         }
         // each copy's scale row goes out as one contiguous run: wavefront w takes routes w, w + waves - 1, ...
-        const uint32_t Hs = args.hidden_dim_scale;
+        if (!QUANT && one.x_scale == nullptr) return;   // rows without scales
         for (uint32_t k = wave; k < K; k += waves - 1) {
             const uint64_t sp = s_scale_ptr[k];
             const uint32_t ss = s_scale_stride[k];
@@ -1743,14 +1769,22 @@ hipError_t launch_dispatch_small(const PushArgs &args, const FinalizeArgs &fin, 
         const size_t receiver_words = (size_t)ws.num_groups * ws.experts_per_rank;
         lds = (tokens_words > receiver_words ? tokens_words : receiver_words) * sizeof(uint32_t);
         // The quick form: a wavefront beside those that move the row, and no receiver workgroups.
-        const uint32_t pieces = args.hidden_dim / 16;
-        if (quantize && ws.topk <= 8 && pieces + kWave <= 1024) {
+        const uint32_t pieces = quantize ? args.hidden_dim / 16 : args.row_bytes / 16;
+        if (ws.topk <= 8 && pieces + kWave <= 1024 && (quantize || args.hidden_dim_scale <= pieces)) {
             const uint32_t quick_threads = (pieces + kWave - 1) / kWave * kWave + kWave;
             const uint32_t counters = quick_threads - kWave;
             const uint32_t per_thread = (total_tokens * ws.topk + counters - 1) / counters;
 #define A2A_LAUNCH_QUICK(NB)                                                                                         \
-    hipExtLaunchKernelGGL(dispatch_quick_kernel<NB>, dim3(total_tokens), dim3(quick_threads),                        \
-                          (size_t)ws.num_experts * sizeof(uint32_t), stream, timing.start, timing.stop, 0, a, fin, ws)
+    do {                                                                                                             \
+        if (quantize)                                                                                                \
+            hipExtLaunchKernelGGL((dispatch_quick_kernel<NB, true>), dim3(total_tokens), dim3(quick_threads),        \
+                                  (size_t)ws.num_experts * sizeof(uint32_t), stream, timing.start, timing.stop, 0,   \
+                                  a, fin, ws);                                                                       \
+        else                                                                                                         \
+            hipExtLaunchKernelGGL((dispatch_quick_kernel<NB, false>), dim3(total_tokens), dim3(quick_threads),       \
+                                  (size_t)ws.num_experts * sizeof(uint32_t), stream, timing.start, timing.stop, 0,   \
+                                  a, fin, ws);                                                                       \
+    } while (0)
             if (per_thread <= 1) A2A_LAUNCH_QUICK(1);
             else if (per_thread == 2) A2A_LAUNCH_QUICK(2);
             else if (per_thread == 3) A2A_LAUNCH_QUICK(3);

@@ -64,3 +64,26 @@ def test_transposed_scale_output():
     for split in (False, True):
         got = run_gpu(cfg, world, rows, device, split, scale_layout="col")
         check(cfg, world, rows, got)
+
+
+SINGLE = [
+    (RefConfig("ONE-SENDER-FP8", 8, 1, 128, 256, 7168, 56, 8, FP8, BF16, F32), 128, 3),
+    (RefConfig("ONE-SENDER-FP8-COL", 8, 1, 128, 128, 2048, 16, 8, FP8, BF16, F32, expert_padding=16), 100, 0),
+    (RefConfig("ONE-SENDER-BF16", 4, 1, 64, 64, 7168, None, 6, BF16, BF16, None), 37, 2),
+    (RefConfig("ONE-SENDER-F32-3-TOKENS", 16, 1, 8, 48, 256, None, 3, F32, F32, None, node_size=4), 3, 9),
+]
+
+
+@pytest.mark.parametrize("cfg,tokens,sender", SINGLE, ids=lambda v: v.name if isinstance(v, RefConfig) else str(v))
+def test_one_sender_in_transport_mode(cfg, tokens, sender):
+    """One rank has tokens (one GPU's share of a decode step) and the rows travel as the caller's bytes
+    with the caller's scales: the small step of one source takes the kernel with a spare wavefront per
+    token also when it does not quantise.  fp8 rows with 56 and 16 scales a row (row-major and
+    transposed output), bf16 and float rows without scales, fewer tokens than tables to write."""
+    device = torch.device("cuda:0")
+    world = [make_ref_rank(cfg, r, tokens if r == sender else 0) for r in range(cfg.world_size)]
+    rows = rows_for(cfg, world)
+    for layout in (("row", "col") if cfg.hidden_dim_scale else ("row",)):
+        got = run_gpu(cfg, world, rows, device, False, scale_layout=layout)
+        check(cfg, world, rows, got)
+
