@@ -1236,11 +1236,13 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(7))) void 
 // write the step's tables.  1024 tokens, hidden 7168, 384 experts over 16 ranks: the head of the
 // kernel (everything in front of the first store) shrinks by about a microsecond.
 //
+// QUANT false: the rows travel as they are, with the caller's scales if it passed any.
+//
 // Dynamic LDS: E words.
 constexpr uint32_t kTeamsMaxRoutes = 32;
 constexpr uint32_t kTeamsMaxScales = 128;   // scale groups of a row of at most (1024 - 64) pieces
 
-template <uint32_t NB, uint32_t ROUNDS>
+template <uint32_t NB, uint32_t ROUNDS, bool QUANT>
 __global__ __launch_bounds__(1024) void dispatch_teams_kernel(const PushArgs args, const FinalizeArgs fin,
                                                               const Workspace ws, const uint32_t team_threads,
                                                               const uint32_t per_group) {
@@ -1252,6 +1254,12 @@ __global__ __launch_bounds__(1024) void dispatch_teams_kernel(const PushArgs arg
     A2A_PIN(args.single.bound_m);
     A2A_PIN(args.single.x_stride);
     A2A_PIN(args.single.num_tokens);
+    if constexpr (!QUANT) {
+        A2A_PIN(args.row_bytes);
+        A2A_PIN(args.single.x_scale);
+        A2A_PIN(args.single.xs_stride_elem);
+        A2A_PIN(args.single.xs_stride_token);
+    }
     A2A_PIN(fin.recv_mask);
     A2A_PIN(ws.world);
     A2A_PIN(ws.num_groups);
@@ -1297,7 +1305,8 @@ __global__ __launch_bounds__(1024) void dispatch_teams_kernel(const PushArgs arg
     const uint32_t first_token = blockIdx.x * per_group;
     const uint32_t my_first = first_token * K;           // flat index of my first entry
     const uint32_t routes = per_group * K;               // <= kTeamsMaxRoutes
-    const uint32_t num_chunks = args.hidden_dim / 16;
+    const uint32_t num_chunks = QUANT ? args.hidden_dim / 16 : args.row_bytes / 16;   // pieces of a row
+    const uint32_t Hs = args.hidden_dim_scale;
     const uint32_t token_groups = gridDim.x;
 
     // lanes of the resolver per route: 8, 4 or 2
@@ -1327,10 +1336,21 @@ __global__ __launch_bounds__(1024) void dispatch_teams_kernel(const PushArgs arg
         for (uint32_t i = 0; i < ROUNDS; ++i) {
             const uint32_t rd = ROUNDS - 1 - i;
             const uint32_t t = first_token + rd * teams + team;
-            const u32x4 *p = reinterpret_cast<const u32x4 *>(one.x + (size_t)(t < tokens ? t : tokens - 1) * one.x_stride +
-                                                             (size_t)(team_tid < num_chunks ? team_tid : 0) * 32);
-            pre_a[rd] = __builtin_nontemporal_load(p);
-            pre_b[rd] = __builtin_nontemporal_load(p + 1);
+            const uint32_t row_t = t < tokens ? t : tokens - 1;
+            if constexpr (QUANT) {
+                const u32x4 *p = reinterpret_cast<const u32x4 *>(one.x + (size_t)row_t * one.x_stride +
+                                                                 (size_t)(team_tid < num_chunks ? team_tid : 0) * 32);
+                pre_a[rd] = __builtin_nontemporal_load(p);
+                pre_b[rd] = __builtin_nontemporal_load(p + 1);
+            } else {
+                pre_a[rd] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(one.x + (size_t)row_t * one.x_stride) +
+                                                       (team_tid < num_chunks ? team_tid : 0));
+                // the caller's scales of the token (one per thread of the team; kept in pre_b's first word)
+                if (one.x_scale != nullptr && team_tid < Hs) {
+                    pre_b[rd].x = __float_as_uint(
+                        one.x_scale[(size_t)row_t * one.xs_stride_token + (size_t)team_tid * one.xs_stride_elem]);
+                }
+            }
         }
     } else {
         __builtin_amdgcn_s_setprio(3);
@@ -1374,12 +1394,16 @@ __global__ __launch_bounds__(1024) void dispatch_teams_kernel(const PushArgs arg
         u32x4 q[ROUNDS];
 #pragma unroll
         for (uint32_t rd = 0; rd < ROUNDS; ++rd) {
-            float scale;
-            q[rd] = quantize16(pre_a[rd], pre_b[rd], &scale);
-            if (has_piece && (lane & 7) == 0) s_scale[rd][team][team_tid / 8] = scale;
+            if constexpr (QUANT) {
+                float scale;
+                q[rd] = quantize16(pre_a[rd], pre_b[rd], &scale);
+                if (has_piece && (lane & 7) == 0) s_scale[rd][team][team_tid / 8] = scale;
+            } else {
+                q[rd] = pre_a[rd];
+                if (team_tid < Hs) s_scale[rd][team][team_tid] = __uint_as_float(pre_b[rd].x);
+            }
         }
         lds_barrier();
-        const uint32_t Hs = args.hidden_dim_scale;
         const uint32_t team_waves = team_threads / kWave, team_wave = team_tid / kWave;
 #pragma unroll
         for (uint32_t rd = 0; rd < ROUNDS; ++rd) {
@@ -1399,6 +1423,7 @@ __global__ __launch_bounds__(1024) void dispatch_teams_kernel(const PushArgs arg
                 }
             }
             // each copy's scale row goes out as one contiguous run: wavefront w of the team takes routes w, w + team_waves, ...
+            if (!QUANT && one.x_scale == nullptr) continue;   // rows without scales
             for (uint32_t k = team_wave; k < K; k += team_waves) {
                 const uint64_t sp = s_scale_ptr[mine * K + k];
                 const uint32_t ss = s_scale_stride[mine * K + k];
@@ -1859,17 +1884,24 @@ hipError_t launch_dispatch_single(const PushArgs &args, const FinalizeArgs &fin,
     a.single = args.src[a.single_source - 1];
     // The form with a spare wavefront per workgroup that resolves the routes while the teams quantise:
     // at most eight routes a token, 32 a workgroup, and two rounds.
-    if (quantize && ws.topk <= 8 && per_group * ws.topk <= kTeamsMaxRoutes && team + kWave <= 1024) {
+    if (ws.topk <= 8 && per_group * ws.topk <= kTeamsMaxRoutes && team + kWave <= 1024 &&
+        (quantize || args.hidden_dim_scale <= (team < kTeamsMaxScales ? team : kTeamsMaxScales))) {
         uint32_t teams = (1024 - kWave) / team;
         if (teams > per_group) teams = per_group;
         const uint32_t rounds = (per_group + teams - 1) / teams;
         const uint32_t counters = teams * team;
         const uint32_t per_thread = (total_tokens * ws.topk + counters - 1) / counters;
-        if (rounds <= 2 && args.hidden_dim / 128 <= kTeamsMaxScales) {
+        if (rounds <= 2 && (!quantize || args.hidden_dim / 128 <= kTeamsMaxScales)) {
             const size_t cnt_bytes = (size_t)ws.num_experts * sizeof(uint32_t);
 #define A2A_LAUNCH_TEAMS(NB, R)                                                                                   \
-    hipExtLaunchKernelGGL((dispatch_teams_kernel<NB, R>), dim3(blocks), dim3(counters + kWave), cnt_bytes, stream, \
-                          timing.start, timing.stop, 0, a, fin, ws, team, per_group)
+    do {                                                                                                          \
+        if (quantize)                                                                                             \
+            hipExtLaunchKernelGGL((dispatch_teams_kernel<NB, R, true>), dim3(blocks), dim3(counters + kWave),     \
+                                  cnt_bytes, stream, timing.start, timing.stop, 0, a, fin, ws, team, per_group);  \
+        else                                                                                                      \
+            hipExtLaunchKernelGGL((dispatch_teams_kernel<NB, R, false>), dim3(blocks), dim3(counters + kWave),    \
+                                  cnt_bytes, stream, timing.start, timing.stop, 0, a, fin, ws, team, per_group);  \
+    } while (0)
             if (rounds == 1) {
                 if (per_thread <= 5) A2A_LAUNCH_TEAMS(5, 1);
                 else if (per_thread <= 10) A2A_LAUNCH_TEAMS(10, 1);

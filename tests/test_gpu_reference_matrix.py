@@ -71,6 +71,9 @@ SINGLE = [
     (RefConfig("ONE-SENDER-FP8-COL", 8, 1, 128, 128, 2048, 16, 8, FP8, BF16, F32, expert_padding=16), 100, 0),
     (RefConfig("ONE-SENDER-BF16", 4, 1, 64, 64, 7168, None, 6, BF16, BF16, None), 37, 2),
     (RefConfig("ONE-SENDER-F32-3-TOKENS", 16, 1, 8, 48, 256, None, 3, F32, F32, None, node_size=4), 3, 9),
+    (RefConfig("ONE-SENDER-FP8-700", 8, 1, 700, 256, 7168, 56, 8, FP8, BF16, F32), 700, 5),
+    (RefConfig("ONE-SENDER-BF16-900", 16, 1, 900, 96, 2048, None, 8, BF16, BF16, None, expert_padding=8), 900, 1),
+    (RefConfig("ONE-SENDER-FP8-1000-TOP3", 4, 1, 1000, 64, 1024, 8, 3, FP8, F32, F32), 1000, 0),
 ]
 
 
@@ -78,8 +81,9 @@ SINGLE = [
 def test_one_sender_in_transport_mode(cfg, tokens, sender):
     """One rank has tokens (one GPU's share of a decode step) and the rows travel as the caller's bytes
     with the caller's scales: the small step of one source takes the kernel with a spare wavefront per
-    token also when it does not quantise.  fp8 rows with 56 and 16 scales a row (row-major and
-    transposed output), bf16 and float rows without scales, fewer tokens than tables to write."""
+    token (or per four tokens, from 448 tokens on) also when it does not quantise.  fp8 rows with 56, 16
+    and 8 scales a row (row-major and transposed output), bf16 and float rows without scales, fewer tokens
+    than tables to write, mid-size steps of one and of two rounds."""
     device = torch.device("cuda:0")
     world = [make_ref_rank(cfg, r, tokens if r == sender else 0) for r in range(cfg.world_size)]
     rows = rows_for(cfg, world)
