@@ -722,23 +722,26 @@ def test_one_launch_dispatch_with_a_single_source(sender, bound, strided):
 
 @pytest.mark.parametrize("tokens,sender,bound,topk,pad,experts,hidden,repeats", [
     (1, 0, None, 8, 1, 128, 2048, False), (3, 5, None, 8, 16, 128, 2048, True), (128, 2, 100, 5, 8, 250, 7168, False),
-    (200, 7, None, 2, 1, 1024, 2048, True), (17, 1, 16, 8, 128, 64, 384, False), (64, 3, None, 1, 1, 8, 1024, False)],
+    (200, 7, None, 2, 1, 1024, 2048, True), (17, 1, 16, 8, 128, 64, 384, False), (64, 3, None, 1, 1, 8, 1024, False),
+    (100, 4, None, 12, 1, 128, 2048, True)],
     ids=["1_token", "3_tokens_pad16_repeats", "128_top5_pad8_250_experts_bound100", "200_top2_1024_experts_repeats",
-         "17_pad128_bound16", "64_top1_one_expert_a_rank"])
+         "17_pad128_bound16", "64_top1_one_expert_a_rank", "100_top12_the_general_kernel"])
 def test_quick_dispatch_of_a_small_single_source(tokens, sender, bound, topk, pad, experts, hidden, repeats):
     """A small quantising step of one source with at most eight routes per token takes a kernel in which a
     spare wavefront per token resolves the routes while the others quantise, and the first workgroups'
     spare wavefronts write the step's tables.  Fewer workgroups than tables to write, a token that names
     an expert twice, experts that do not divide among the ranks, more experts per rank than a pass of the
-    route sums covers, a bound on the device, padded receive slots: the oracle's result, bit for bit."""
+    route sums covers, a bound on the device, padded receive slots: the oracle's result, bit for bit.  (More
+    than eight routes a token: the general one-launch kernel serves the step.)"""
     case = replace(scaled(C1, tokens), topk=topk, expert_padding=pad, num_experts=experts, hidden_dim=hidden,
                    name=f"quick_{tokens}")
     _check_single_source(case, sender, bound, False, repeats)
 
 
 @pytest.mark.parametrize("tokens,sender,bound,topk,pad", [(700, 2, None, 8, 1), (1024, 0, None, 8, 16), (702, 5, 333, 8, 1),
-                                                          (600, 1, 0, 8, 1), (640, 3, None, 5, 8), (1000, 7, 1, 3, 1)],
-                         ids=["700", "1024_pad16", "702_bound333", "600_bound0", "640_top5_pad8", "1000_top3_bound1"])
+                                                          (600, 1, 0, 8, 1), (640, 3, None, 5, 8), (1000, 7, 1, 3, 1), (600, 6, None, 12, 1)],
+                         ids=["700", "1024_pad16", "702_bound333", "600_bound0", "640_top5_pad8", "1000_top3_bound1",
+                              "600_top12_the_general_kernel"])
 def test_one_launch_dispatch_of_a_larger_single_source(tokens, sender, bound, topk, pad):
     """Steps of one source that are too large for the one-launch dispatch of small steps (every token's
     workgroup counting every entry) and have at most 8192 entries take a launch whose workgroups count
