@@ -24,7 +24,7 @@ namespace a2a {
 struct Staging {
     bool allocated = false;
     void *arena = nullptr;
-    uint8_t *send_buf = nullptr;         // [N][max_num_tokens][disp_stride]: payload, scales, 16 spare bytes
+    uint8_t *send_buf = nullptr;         // [N][max_num_tokens][disp_stride]: payload, scales, 16 spare bytes (+ padding to whole lines)
     uint32_t *pos_token = nullptr;       // [N][max_tk]: token behind each row of a sender's expert-sorted order
     uint8_t *comb_buf = nullptr;         // [N][max_tk][comb_stride]: combine rows at the sender's positions
     uint32_t *padded_index = nullptr;    // [N][max_recv]
