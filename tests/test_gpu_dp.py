@@ -35,6 +35,25 @@ def test_dp_groups(cfg, split):
     check_dp(cfg, groups, rows, got)
 
 
+ONE_GROUP_SENDS = [
+    (RefConfig("dp2_one_group_sends", 8, 2, 96, 64, 1024, 8, 8, FP8, BF16, F32, node_size=4), 96, 2),
+    (RefConfig("dp4_one_group_sends_bf16", 8, 4, 50, 16, 512, None, 4, BF16, BF16, None, expert_padding=4), 50, 1),
+    (RefConfig("dp2_one_group_sends_700", 4, 2, 700, 32, 1024, 8, 8, FP8, BF16, F32, node_size=2), 700, 0),
+]
+
+
+@pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
+@pytest.mark.parametrize("cfg,tokens,sender", ONE_GROUP_SENDS, ids=lambda v: v.name if isinstance(v, RefConfig) else str(v))
+def test_one_dp_group_sends(cfg, tokens, sender, split):
+    """Of several dp groups one alone has tokens (the others hold none this step): the one-launch kernels
+    of a single source serve the step, and every rank of every group still receives its experts' rows
+    and the sending group's ranks their combined tokens."""
+    print(f"cfg={cfg.name} split={split}", flush=True)
+    groups = [make_ref_rank(cfg, g, tokens if g == sender else 0) for g in range(cfg.world_size // cfg.dp_size)]
+    got, rows = run_gpu_dp(cfg, groups, torch.device("cuda:0"), split)
+    check_dp(cfg, groups, rows, got)
+
+
 def test_accumulate_is_refused_with_dp_groups():
     """python/pplx_garden/kernels/p2p_all_to_all.py:457-458"""
     from pplx_garden_amd.distributed.loopback import LoopbackWorld
