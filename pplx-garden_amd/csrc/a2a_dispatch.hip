@@ -264,7 +264,9 @@ __global__ __launch_bounds__(1024) void dispatch_push_kernel(const PushArgs args
 // token's ids are (building it costs a trip to memory before the counting can
 // start), no division of entry numbers, and no copies of other sources to
 // place before mine, so the order in which receivers lay out their sources
-// drops out too.
+// drops out too.  (With at most eight routes a token and a row that one
+// workgroup covers with a wavefront to spare, such a step takes
+// dispatch_quick_kernel instead; this variant serves the rest.)
 //
 // Dynamic LDS: (G + 3) * E words and 8 bytes per token of the step; SINGLE:
 // 4 * E words (or G * Le, if that is more: the receiver workgroups' table).
