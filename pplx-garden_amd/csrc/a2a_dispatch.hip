@@ -597,8 +597,9 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
 }
 
 // The quick form of the one-launch dispatch of a small step: ONE source has tokens, its index rows
-// are dense, it quantises, a token has at most eight routes, and the row is one 16-element piece
-// per thread with a wavefront to spare (the host launches one more than the row has pieces for).
+// are dense, a token has at most eight routes, and the row is one piece per thread (16 elements to
+// quantise, or 16 bytes to move as they are) with a wavefront to spare (the host launches one more
+// than the row has pieces for).
 // One workgroup per token, no receiver workgroups.
 //
 // In dispatch_small_kernel every wavefront walks the same chain once its data is there: count, a
@@ -621,7 +622,8 @@ __global__ __launch_bounds__(1024) void dispatch_small_kernel(const PushArgs arg
 //    the others store rows (done by all workgroups, a share of the experts each, the same stores
 //    were 0.3 us slower than with receiver workgroups: many wavefronts writing parts of the
 //    same lines).
-// 128 tokens, hidden 7168: 5.95 -> 5.2 us per dispatch at the GPU's own pace; hidden 2048: 5.8 -> 4.6.
+// 128 tokens, hidden 7168: 5.95 -> 4.5 us per dispatch at the GPU's own pace; hidden 2048: 5.8 -> 4.2.
+// (Two workgroups per token, half a row each, so that all compute units have one: 4.65 and 5.3 us.)
 //
 // Dynamic LDS: E words.
 constexpr uint32_t kQuickSpinLimit = 1u << 22;   // (a resolver that gives up flags A2A_DEV_INTERNAL; never seen)
