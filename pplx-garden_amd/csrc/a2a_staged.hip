@@ -249,6 +249,214 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
     stage_row<QUANT, true>(args, st, g, token, nthreads, pre_a, pre_b);
 }
 
+// The quick form of the one-launch send of a small step: dense index rows and a row that is one piece
+// per thread (16 elements to quantise, or 16 bytes to move as they are) with a wavefront to spare (the
+// host launches one more than the row has pieces for).  Where a row is staged does not depend on the
+// routing (one row per token, at the token's own place), so the wavefronts that move the row count
+// their entries, say so (a word in LDS, not a barrier) and then quantise and store without waiting for
+// anybody; the spare wavefront (the RESOLVER) does not count: it holds the token's ids, waits until
+// every counting wavefront has said that its entries are in the table, scans the table by itself (64
+// experts an instruction, no workgroup scan with its barriers), and writes the token's positions; the
+// resolver of token 0 publishes the counts and their scan on the way.  In stage_send_small_kernel every
+// wavefront walks count, workgroup scan, routes and row one after the other: 128 tokens of 7168,
+// 4.1 -> 3.6 us per send at the GPU's own pace; hidden 2048: 3.9 -> 3.2.
+// NB: entries a counting thread asks for at the head (the host picks the smallest of 1, 2, 3, 4, 8 that
+// covers the step; entries beyond are counted by a loop).  Dynamic LDS: E words (low half of a word:
+// the entries of the expert, high half: those of the tokens before this one; a step of this kernel
+// has fewer than 2^16 entries).
+constexpr uint32_t kSendQuickSpinLimit = 1u << 22;   // (a resolver that gives up flags A2A_DEV_INTERNAL; never seen)
+
+template <uint32_t NB, bool QUANT>
+__global__ __launch_bounds__(1024) void stage_send_quick_kernel(const StageSendArgs args, const Workspace ws,
+                                                                const Staging st) {
+    extern __shared__ uint32_t s_cnt[];
+    __shared__ uint32_t s_counted;   // counting wavefronts whose entries are in the table
+    // everything the head of a workgroup takes from the argument block, asked for in one go
+    A2A_PIN(args.src.x);
+    A2A_PIN(args.src.x_scale);
+    A2A_PIN(args.src.indices);
+    A2A_PIN(args.src.bound_m);
+    A2A_PIN(args.src.x_stride);
+    A2A_PIN(args.src.num_tokens);
+    A2A_PIN(args.rank);
+    A2A_PIN(args.hidden_dim);
+    A2A_PIN(args.row_bytes);
+    A2A_PIN(ws.num_experts);
+    A2A_PIN(ws.topk);
+    A2A_PIN(ws.dp_size);
+    A2A_PIN(ws.max_tk);
+    A2A_PIN(ws.num_routed);
+    A2A_PIN(ws.expert_offsets);
+    A2A_PIN(ws.token_offset);
+    A2A_PIN(ws.err);
+    A2A_PIN(st.send_buf);
+    A2A_PIN(st.pos_token);
+    A2A_PIN(st.disp_stride);
+    A2A_PIN(st.payload_bytes);
+    A2A_PIN(st.max_tokens);
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nthreads = blockDim.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    const uint32_t waves = nthreads / kWave;
+    const bool resolver = wave == waves - 1;
+    const uint32_t counters = nthreads - kWave;   // threads that count entries and move the row
+    const uint32_t E = ws.num_experts;
+    const uint32_t K = ws.topk;
+    const uint32_t g = args.rank / ws.dp_size;
+    const uint32_t token = blockIdx.x;
+    const PushSrc &src = args.src;
+    const uint32_t tokens = src.num_tokens;   // the grid: one workgroup per token
+    const uint32_t entries = tokens * K;      // > 0
+    const uint32_t my_first = token * K;
+    const uint32_t num_chunks = QUANT ? args.hidden_dim / 16 : args.row_bytes / 16;   // pieces of a row, one per thread
+    const bool has_piece = tid < num_chunks;
+
+    // What each kind of wavefront takes from memory, asked for before anything else is done: the
+    // entries, then the thread's piece of the row (and the first of the caller's scales it copies);
+    // the resolver its token's ids (lane k: route k).
+    uint32_t early[NB] = {};
+    u32x4 pre_a = {0, 0, 0, 0}, pre_b = {0, 0, 0, 0};
+    float first_scale = 0.0f;
+    uint32_t my_id = 0xFFFFFFFFu;
+    if (!resolver) {
+#pragma unroll
+        for (uint32_t j = 0; j < NB; ++j) {
+            const uint32_t f = j * counters + tid;
+            early[j] = (uint32_t)src.indices[f < entries ? f : entries - 1];
+        }
+        const uint8_t *x_row = src.x + (size_t)token * src.x_stride;
+        if (has_piece) {
+            if constexpr (QUANT) {
+                const u32x4 *piece = reinterpret_cast<const u32x4 *>(x_row + (size_t)tid * 32);
+                pre_a = __builtin_nontemporal_load(piece);
+                pre_b = __builtin_nontemporal_load(piece + 1);
+            } else {
+                pre_a = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x_row) + tid);
+            }
+        }
+        if constexpr (!QUANT) {
+            if (src.x_scale != nullptr && tid < args.hidden_dim_scale) {
+                first_scale = src.x_scale[(size_t)token * src.xs_stride_token + (size_t)tid * src.xs_stride_elem];
+            }
+        }
+    } else {
+        // (the resolver shares its SIMD with wavefronts that quantise while the positions are resolved)
+        __builtin_amdgcn_s_setprio(3);
+        my_id = (uint32_t)src.indices[my_first + (lane < K ? lane : 0)];
+    }
+    const uint32_t eff = effective_tokens(src.bound_m, tokens);
+    const uint32_t flat_entries = eff * K;
+    const bool live = token < eff;   // uniform
+
+    for (uint32_t i = tid; i < E; i += nthreads) s_cnt[i] = 0;
+    if (tid == 0) s_counted = 0;
+    lds_barrier();
+
+    if (!resolver) {
+        // The first batch in straight-line code: each of its values is waited for by itself, and the
+        // row asked for after them stays in flight meanwhile.
+#pragma unroll
+        for (uint32_t j = 0; j < NB; ++j) {
+            const uint32_t f = j * counters + tid;
+            const uint32_t x = f < flat_entries ? early[j] : 0xFFFFFFFFu;
+            if (x < E) atomicAdd(&s_cnt[x], f < my_first ? 0x10001u : 1u);
+        }
+        for (uint32_t f0 = NB * counters; f0 < flat_entries; f0 += NB * counters) {
+            uint32_t x[NB];
+#pragma unroll
+            for (uint32_t j = 0; j < NB; ++j) {
+                const uint32_t f = f0 + j * counters + tid;
+                x[j] = f < flat_entries ? (uint32_t)src.indices[f] : 0xFFFFFFFFu;
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < NB; ++j) {
+                const uint32_t f = f0 + j * counters + tid;
+                if (x[j] < E) atomicAdd(&s_cnt[x[j]], f < my_first ? 0x10001u : 1u);
+            }
+        }
+        // this wavefront's entries are in the table before its arrival is counted
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (lane == 0) atomicAdd(&s_counted, 1u);
+        if (!live) return;   // past bound_m: nothing to stage (uniform)
+
+        uint8_t *row = st.send_buf + ((size_t)g * st.max_tokens + token) * st.disp_stride;
+        float *row_scale = reinterpret_cast<float *>(row + st.payload_bytes);
+        if constexpr (QUANT) {
+            float scale;
+            const u32x4 q = quantize16(pre_a, pre_b, &scale);
+            if (has_piece) {
+                reinterpret_cast<u32x4 *>(row)[tid] = q;
+                if ((lane & 7) == 0) row_scale[tid / 8] = scale;
+            }
+        } else {
+            if (has_piece) reinterpret_cast<u32x4 *>(row)[tid] = pre_a;
+            if (src.x_scale != nullptr) {
+                if (tid < args.hidden_dim_scale) row_scale[tid] = first_scale;
+                const float *xs = src.x_scale + (size_t)token * src.xs_stride_token;
+                for (uint32_t j = tid + counters; j < args.hidden_dim_scale; j += counters) {
+                    row_scale[j] = xs[(size_t)j * src.xs_stride_elem];
+                }
+            }
+        }
+        return;
+    }
+
+    // ---- the resolver ----
+    // copies of this token to the same expert at an earlier k: what no count decides
+    uint32_t repeats = 0;
+    for (uint32_t k = 0; k + 1 < K; ++k) {
+        const uint32_t other = (uint32_t)__builtin_amdgcn_readlane((int)my_id, (int)k);
+        if (k < lane && other == my_id) ++repeats;
+    }
+    // until the counting wavefronts have all said that their entries are in the table (at the lowest
+    // priority: the wavefronts that share this SIMD are among those waited for)
+    __builtin_amdgcn_s_setprio(0);
+    for (uint32_t spins = 0; __hip_atomic_load(&s_counted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != waves - 1;) {
+        if (++spins == kSendQuickSpinLimit) {
+            if (lane == 0) atomicOr(ws.err, A2A_DEV_INTERNAL);
+            break;
+        }
+    }
+    __builtin_amdgcn_s_setprio(3);
+    asm volatile("" ::: "memory");
+
+    // Scan over the experts (a2a_dispatch_send.cu:236-242), 64 at a time; a route whose expert lies in
+    // the 64 at hand takes the expert's word and the entries of the experts before it from the lane
+    // that holds them.  Token 0 publishes.
+    uint32_t run = 0, my_word = 0, my_excl = 0;
+    for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
+        const uint32_t x = e0 + lane;
+        const uint32_t word = x < E ? s_cnt[x] : 0;
+        const uint32_t c = word & 0xFFFFu;
+        const uint32_t incl = run + wave_inclusive_scan(c, lane);
+        if (token == 0 && x < E) {
+            ws.num_routed[g * E + x] = c;
+            ws.expert_offsets[g * E + x] = incl;
+        }
+        const uint32_t rel = my_id - e0;   // (an id below e0 wraps around to a large number)
+        const uint32_t their_word = (uint32_t)__shfl((int)word, (int)(rel & (kWave - 1)));   // every lane takes part
+        const uint32_t their_excl = (uint32_t)__shfl((int)(incl - c), (int)(rel & (kWave - 1)));
+        if (rel < (uint32_t)kWave) {
+            my_word = their_word;
+            my_excl = their_excl;
+        }
+        run = (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
+    }
+    if (!live) return;   // past bound_m: no positions to write (uniform)
+    if (lane < K) {
+        uint32_t toff = 0;
+        if (my_id < E) {
+            toff = (my_word >> 16) + repeats;
+            // position of the copy (a2a_dispatch_send.cu:54)
+            st.pos_token[(size_t)g * ws.max_tk + my_excl + toff] = token;
+        } else {
+            atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
+        }
+        ws.token_offset[(size_t)g * ws.max_tk + my_first + lane] = toff;
+    }
+}
+
 // The send of a step too large for stage_send_small_kernel and of at most kSendSingleMaxEntries
 // entries (448 to 1024 tokens at top-8), in ONE launch: what makes the small kernel expensive as steps
 // grow is that every token's workgroup counts every entry of the sender; here a workgroup counts once
@@ -515,6 +723,25 @@ __device__ __forceinline__ void copy_row_by_team(const u32x4 *src, u32x4 *dst, u
     }
 }
 
+// Payload and scales of one received row, by a team.  The scales are asked for before the payload
+// moves: behind the payload's stores their trip would begin only when those have been acknowledged
+// (memory operations of a wavefront complete in order).
+__device__ __forceinline__ void copy_received_row(const uint8_t *src, uint32_t payload_bytes, uint32_t num_chunks,
+                                                  uint32_t num_scales, const PushDst &dst, uint32_t dst_row,
+                                                  uint32_t member, uint32_t team) {
+    const float *ss = reinterpret_cast<const float *>(src + payload_bytes);
+    float first_scale = 0.0f;
+    const bool scales = dst.out_scale != nullptr;
+    if (scales && member < num_scales) first_scale = ss[member];
+    copy_row_by_team(reinterpret_cast<const u32x4 *>(src),
+                     reinterpret_cast<u32x4 *>(dst.out_x + (size_t)dst_row * dst.out_stride), num_chunks, member, team);
+    if (scales) {
+        float *os = dst.out_scale + (size_t)dst_row * dst.os_stride_token;
+        if (member < num_scales) os[(size_t)member * dst.os_stride_elem] = first_scale;
+        for (uint32_t q = member + team; q < num_scales; q += team) os[(size_t)q * dst.os_stride_elem] = ss[q];
+    }
+}
+
 // ---------------------------------------------------------------------------
 // dispatch recv.  The receivers of a step are laid out ONCE per step, by the
 // launch of the step's first recv (the reference's host worker runs
@@ -580,15 +807,22 @@ __device__ __forceinline__ bool lay_out_receiver(uint32_t valid_mask, const Work
     // The order in which this receiver lays out its sources (one byte per source, from the table the
     // context computed once) travels with the counts and is read from LDS from then on: looked up in
     // memory where it is used, it put a dependent trip into the layout and one in front of every row.
-    if (tid < G) s_order[tid] = (uint8_t)source_order_lookup(ws.order, r, tid);
+    // All loads of a thread are asked for before the first is used (none under a condition of its own:
+    // a word that does not count is read from a valid place and dropped), or each would be waited for
+    // by itself, one trip to memory after the other.
+    const uint32_t order_word = ws.order[r * (kMaxWorld / 4) + (tid < G ? tid >> 2 : 0)];
     for (uint32_t w = tid; w < items; w += nthreads) {
         const uint32_t g = Le > 1 ? __umulhi(w, ws.le_magic) : w;
         const uint32_t le = w - g * Le;
         const uint32_t e = first + le;
         const bool live = le < n_local && (valid_mask >> g & 1);
-        tot[w] = live ? ws.num_routed[g * E + e] : 0;
-        excl[w] = live && e > 0 ? ws.expert_offsets[g * E + e - 1] : 0;
+        const uint32_t at = live ? g * E + e : 0;
+        const uint32_t count = ws.num_routed[at];
+        const uint32_t upto = ws.expert_offsets[at > 0 ? at - 1 : 0];
+        tot[w] = live ? count : 0;
+        excl[w] = live && e > 0 ? upto : 0;
     }
+    if (tid < G) s_order[tid] = (uint8_t)(order_word >> (8 * (tid & 3)));
     __syncthreads();
 
     // Rows this receiver gets from source g (lane g; there are at most kMaxWorld <= 64 sources): the
@@ -814,16 +1048,7 @@ __global__ __launch_bounds__(1024) void stage_recv_first_kernel(const StageRecvA
             continue;
         }
         const uint8_t *src = st.send_buf + ((size_t)m.g * st.max_tokens + token) * st.disp_stride;
-        copy_row_by_team(reinterpret_cast<const u32x4 *>(src),
-                         reinterpret_cast<u32x4 *>(dst.out_x + (size_t)m.dst_row * dst.out_stride), num_chunks, member,
-                         team_threads);
-        if (dst.out_scale != nullptr) {
-            const float *ss = reinterpret_cast<const float *>(src + st.payload_bytes);
-            float *os = dst.out_scale + (size_t)m.dst_row * dst.os_stride_token;
-            for (uint32_t q = member; q < args.hidden_dim_scale; q += team_threads) {
-                os[(size_t)q * dst.os_stride_elem] = ss[q];
-            }
-        }
+        copy_received_row(src, st.payload_bytes, num_chunks, args.hidden_dim_scale, dst, m.dst_row, member, team_threads);
     }
 }
 
@@ -852,13 +1077,14 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     const PushDst &dst = args.dst;
     const uint32_t num_chunks = args.row_bytes / 16;
     const uint32_t team = args.team_waves * kWave;   // threads that share a row
-    const uint32_t teams = blockDim.x / team;
-    const uint32_t member = tid % team;
+    const bool whole = team == blockDim.x;           // (uniform) the workgroup is one team: no divisions
+    const uint32_t teams = whole ? 1 : blockDim.x / team;
+    const uint32_t member = whole ? tid : tid % team;
     const uint32_t *padded_index = st.padded_index + (size_t)r * st.max_recv;
     const uint32_t *source_row = st.source_row + (size_t)r * st.max_recv;
     // The first row's two table words are asked for together with the number of rows received
     // (a row index the tables do not hold reads entry 0 and is dropped by the loop's bound).
-    uint32_t row = blockIdx.x * teams + tid / team;
+    uint32_t row = blockIdx.x * teams + (whole ? 0 : tid / team);
     const uint32_t probe = row < st.max_recv ? row : 0;
     uint32_t dst_row = padded_index[probe];
     uint32_t from = source_row[probe];
@@ -889,16 +1115,7 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
             if (member == 0) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
         } else {
             const uint8_t *src = st.send_buf + (size_t)from * st.disp_stride;
-            copy_row_by_team(reinterpret_cast<const u32x4 *>(src),
-                             reinterpret_cast<u32x4 *>(dst.out_x + (size_t)dst_row * dst.out_stride), num_chunks,
-                             member, team);
-            if (dst.out_scale != nullptr) {
-                const float *ss = reinterpret_cast<const float *>(src + st.payload_bytes);
-                float *os = dst.out_scale + (size_t)dst_row * dst.os_stride_token;
-                for (uint32_t q = member; q < args.hidden_dim_scale; q += team) {
-                    os[(size_t)q * dst.os_stride_elem] = ss[q];
-                }
-            }
+            copy_received_row(src, st.payload_bytes, num_chunks, args.hidden_dim_scale, dst, dst_row, member, team);
         }
         row = next;
         dst_row = next_dst;
@@ -928,24 +1145,44 @@ __global__ __launch_bounds__(1024) void combine_send_kernel(const CombineSendArg
     A2A_PIN(st.comb_stride);
     A2A_PIN(st.max_recv);
     const uint32_t r = args.rank;
-    uint32_t total = st.num_recv[2 * r];
-    if (total > st.max_recv) total = st.max_recv;
     const uint32_t num_chunks = args.row_bytes / 16;
     const uint32_t team = args.team_waves * kWave;   // threads that share a row
-    const uint32_t teams = blockDim.x / team;
-    const uint32_t member = threadIdx.x % team;
-    for (uint32_t i = blockIdx.x * teams + threadIdx.x / team; i < total; i += gridDim.x * teams) {
-        const uint32_t row = st.padded_index[(size_t)r * st.max_recv + i];
+    const bool whole = team == blockDim.x;           // (uniform) the workgroup is one team: no divisions
+    const uint32_t teams = whole ? 1 : blockDim.x / team;
+    const uint32_t member = whole ? threadIdx.x : threadIdx.x % team;
+    const uint32_t *padded_index = st.padded_index + (size_t)r * st.max_recv;
+    const uint32_t *source_rank = st.source_rank + (size_t)r * st.max_recv;
+    const uint32_t *source_position = st.source_position + (size_t)r * st.max_recv;
+    // The first row's three table words are asked for together with the number of rows received (a
+    // row index the tables do not hold reads entry 0 and is dropped by the loop's bound).
+    uint32_t i = blockIdx.x * teams + (whole ? 0 : threadIdx.x / team);
+    const uint32_t probe = i < st.max_recv ? i : 0;
+    uint32_t row = padded_index[probe];
+    uint32_t peer = source_rank[probe];
+    uint32_t pos = source_position[probe];
+    uint32_t total = st.num_recv[2 * r];
+    if (total > st.max_recv) total = st.max_recv;
+    const uint32_t stride = gridDim.x * teams;
+    while (i < total) {
+        // the next row's words travel while this one is copied
+        const uint32_t next = i + stride;
+        const uint32_t next_probe = next < total ? next : i;
+        const uint32_t next_row = padded_index[next_probe];
+        const uint32_t next_peer = source_rank[next_probe];
+        const uint32_t next_pos = source_position[next_probe];
         // every member of the source's dp group reads the same staging rows
-        const uint32_t g = st.source_rank[(size_t)r * st.max_recv + i] / ws.dp_size;
-        const uint32_t pos = st.source_position[(size_t)r * st.max_recv + i];
+        const uint32_t g = ws.dp_size > 1 ? peer / ws.dp_size : peer;
         if (row >= args.y_rows || pos >= ws.max_tk) {
             if (member == 0) atomicOr(ws.err, A2A_DEV_BAD_SLOT);
-            continue;
+        } else {
+            copy_row_by_team(reinterpret_cast<const u32x4 *>(args.y + (size_t)row * args.y_stride),
+                             reinterpret_cast<u32x4 *>(st.comb_buf + ((size_t)g * ws.max_tk + pos) * st.comb_stride),
+                             num_chunks, member, team);
         }
-        copy_row_by_team(reinterpret_cast<const u32x4 *>(args.y + (size_t)row * args.y_stride),
-                         reinterpret_cast<u32x4 *>(st.comb_buf + ((size_t)g * ws.max_tk + pos) * st.comb_stride),
-                         num_chunks, member, team);
+        i = next;
+        row = next_row;
+        peer = next_peer;
+        pos = next_pos;
     }
 }
 
@@ -1131,6 +1368,32 @@ bool stage_send_small_fits(const StageSendArgs &args, const Workspace &ws) {
 
 hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                                    bool quantize, hipStream_t stream, KernelTiming timing) {
+    // The quick form: dense index rows, a piece of the row per thread and a wavefront beside them.
+    const uint32_t pieces = quantize ? args.hidden_dim / 16 : args.row_bytes / 16;
+    if (args.src.indices_stride == ws.topk && pieces + kWave <= 1024) {
+        const uint32_t quick_threads = (pieces + kWave - 1) / kWave * kWave + kWave;
+        const uint32_t counters = quick_threads - kWave;
+        const uint32_t per_thread = (args.src.num_tokens * ws.topk + counters - 1) / counters;
+        const size_t quick_lds = (size_t)ws.num_experts * sizeof(uint32_t);
+#define A2A_LAUNCH_SEND_QUICK(NB)                                                                                    \
+    do {                                                                                                             \
+        if (quantize)                                                                                                \
+            hipExtLaunchKernelGGL((stage_send_quick_kernel<NB, true>), dim3(args.src.num_tokens),                    \
+                                  dim3(quick_threads), quick_lds, stream, timing.start, timing.stop, 0, args, ws,    \
+                                  st);                                                                               \
+        else                                                                                                         \
+            hipExtLaunchKernelGGL((stage_send_quick_kernel<NB, false>), dim3(args.src.num_tokens),                   \
+                                  dim3(quick_threads), quick_lds, stream, timing.start, timing.stop, 0, args, ws,    \
+                                  st);                                                                               \
+    } while (0)
+        if (per_thread <= 1) A2A_LAUNCH_SEND_QUICK(1);
+        else if (per_thread <= 2) A2A_LAUNCH_SEND_QUICK(2);
+        else if (per_thread <= 3) A2A_LAUNCH_SEND_QUICK(3);
+        else if (per_thread <= 4) A2A_LAUNCH_SEND_QUICK(4);
+        else A2A_LAUNCH_SEND_QUICK(8);
+#undef A2A_LAUNCH_SEND_QUICK
+        return hipGetLastError();
+    }
     const uint32_t threads = block_for_chunks(quantize ? args.hidden_dim / 16 : args.row_bytes / 16);
     const size_t lds = 3 * (size_t)ws.num_experts * sizeof(uint32_t);
     if (quantize) {

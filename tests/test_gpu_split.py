@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import a2a_oracle as oracle
-from a2a_cases import C0, C1, C2, C4, make_world, scaled
+from a2a_cases import C0, C1, C2, C4, Case, make_world, scaled
 from a2a_harness import (assert_combine_close, assert_dispatch_equal, make_ops, rows_needed, run_gpu,
                          run_oracle, SENTINEL)
 from pplx_garden_amd.native import p2p_all_to_all as native
@@ -35,6 +35,59 @@ def test_split_parity(case, sources, device):
     got = run_gpu(case, world, rows, device, split=True)
     assert_dispatch_equal(case, got, want)
     assert_combine_close(case, got, want)
+
+
+QUICK_SENDS = [
+    # (tokens, hidden, experts, ranks, top-k, padding, sources, experts may repeat inside a token)
+    (1, 2048, 128, 8, 8, 1, "one", False),
+    (3, 2048, 128, 8, 8, 16, "all", True),
+    (128, 7168, 250, 8, 5, 8, "ragged", False),       # experts that do not fill 64-lane passes, nor divide among the ranks
+    (200, 2048, 1024, 8, 2, 1, "all", True),          # sixteen passes of the resolver's scan
+    (100, 2048, 128, 8, 12, 1, "ragged", True),       # more than eight routes a token
+    (64, 1024, 8, 8, 1, 1, "all", False),
+    (96, 15360, 64, 4, 4, 1, "ragged", False),        # 960 pieces a row: sixteen wavefronts, the resolver is the last
+    (40, 16384, 64, 4, 4, 1, "ragged", False),        # a piece too many for a spare wavefront: the kernel without one
+    (300, 512, 96, 2, 6, 4, "all", True),             # entries beyond what the threads ask for at the head
+]
+
+
+@pytest.mark.parametrize("tokens,hidden,experts,ranks,topk,pad,sources,repeats", QUICK_SENDS,
+                         ids=[f"{t}x{h}_e{e}_n{n}_k{k}_pad{p}_{s}{'_repeats' if rep else ''}"
+                              for t, h, e, n, k, p, s, rep in QUICK_SENDS])
+def test_quick_send_of_small_steps(tokens, hidden, experts, ranks, topk, pad, sources, repeats, device):
+    """The send of a small step with dense index rows takes a kernel in which a spare wavefront per token
+    scans the counts and writes the token's positions while the others quantise and stage the row.  One
+    token, experts that do not fill the scan's passes, many passes, more routes than a wavefront's
+    eighth, rows of sixteen wavefronts, entries beyond the first batch, tokens that name an expert
+    twice: rows, scales and the routing tables are the oracle's, bit for bit."""
+    case = Case(f"quick_send_{tokens}x{hidden}", tokens, hidden, experts, ranks, topk, 4242 + tokens,
+                expert_padding=pad)
+    world = make_world(case, sources)
+    if repeats:
+        gen = torch.Generator().manual_seed(tokens)
+        for rd in world:
+            if rd.indices.shape[0] > 0:
+                rd.indices[::3, topk - 1] = rd.indices[::3, 0]      # every third token names its first expert twice
+                rd.indices.copy_(rd.indices[torch.randperm(rd.indices.shape[0], generator=gen)])
+    rows = rows_needed(case, world)
+    want = run_oracle(case, world, rows)
+    _, ops = make_ops(case, device)
+    try:
+        got = run_gpu(case, world, rows, device, split=True, ops=ops)
+        assert_dispatch_equal(case, got, want)
+        assert_combine_close(case, got, want)
+        ctx = ops[0].context
+        for g, rd in enumerate(world):
+            T = rd.indices.shape[0]
+            if T == 0:
+                continue
+            count, toff, eoff = oracle.route(rd.indices.numpy(), experts)
+            np.testing.assert_array_equal(ctx.read_table(g, native.TABLE_NUM_ROUTED, experts).numpy(), count)
+            np.testing.assert_array_equal(ctx.read_table(g, native.TABLE_EXPERT_OFFSETS, experts).numpy(), eoff)
+            np.testing.assert_array_equal(ctx.read_table(g, native.TABLE_TOKEN_OFFSET, T * topk).numpy(), toff)
+    finally:
+        for op in ops:
+            op.destroy()
 
 
 @pytest.mark.parametrize("max_private", [0, 3, 8, None], ids=lambda v: f"private_{v}")
