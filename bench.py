@@ -276,7 +276,7 @@ def time_graph_replay(wl: Workload, steps: int, warmup: int):
     return wall_s / (replays * n), replays * n
 
 
-def time_gpu_pace(wl: Workload, batches: int = 5, steps_each: int = 100):
+def time_gpu_pace(wl: Workload, batches: int = 5, steps_each: int = 100, step_fn=None):
     """The GPU's own pace per step: `steps_each` steps are enqueued behind a kernel that holds the queue
     for a few milliseconds, so the host is ahead of the GPU for all of them, and two events around them
     give the time the GPU took.  For steps of about 10 us the host's share of a step (two calls through
@@ -294,7 +294,10 @@ def time_gpu_pace(wl: Workload, batches: int = 5, steps_each: int = 100):
         hold(20_000_000)
         first.record()
         for i in range(steps_each):
-            wl.step(i, stream)
+            if step_fn is None:
+                wl.step(i, stream)
+            else:
+                step_fn(i)
         last.record()
         torch.cuda.synchronize(wl.device)
         paces.append(first.elapsed_time(last) * 1e3 / steps_each)
@@ -596,6 +599,99 @@ def split_calls(case, device, routings: int, steps: int, warmup: int, label: str
     }
 
 
+def split_calls_small(case, device, routings: int, steps: int, warmup: int, label: str):
+    """The four split calls at a step of a few microseconds (a decode shape), rank 0 holding the tokens:
+    wall time of a loop of steps and the GPU's own pace (the steps enqueued behind a kernel that holds the
+    queue), for rank 0's four calls (what a rank on a GPU of its own runs) and for the calls of the whole
+    group, and the pace of the sequences send / send + recv / send + recv + combine-send, whose
+    differences are what each call adds."""
+    import torch
+    from pplx_garden_amd.native import p2p_all_to_all as native
+
+    wl = Workload(case, device, routings, native.FLAG_PREALLOC_STAGING)
+    ctx = wl.ctx
+    N, H, Hs, K, T = case.world_size, case.hidden_dim, case.hidden_dim_scale, case.topk, case.num_tokens
+    stream = torch.cuda.current_stream(device).cuda_stream
+    R = len(wl.routings)
+
+    def send(i):
+        j = i % R
+        ctx.dispatch_send(0, T, wl.x[0].data_ptr(), 2 * H, None, 0, 0, wl.idx[j][0].data_ptr(), K,
+                          wl.w[j][0].data_ptr(), K, None, stream, quantize=True)
+
+    def empty_send(r):
+        ctx.dispatch_send(r, 0, None, 2 * H, None, 0, 0, None, K, None, K, None, stream, quantize=True)
+
+    def recv(r):
+        ctx.dispatch_recv(r, wl.out_n[r].data_ptr(), wl.out_x[r].data_ptr(), H, wl.rows, wl.out_s[r].data_ptr(), 1, Hs,
+                          stream)
+
+    def combine_send(r):
+        ctx.combine_send(r, wl.y[r].data_ptr(), 2 * H, wl.rows, stream)
+
+    def combine_recv(i):
+        j = i % R
+        ctx.combine_recv(0, T, wl.rows, torch.bfloat16, wl.out_tokens[0].data_ptr(), H, wl.idx[j][0].data_ptr(), K,
+                         wl.w[j][0].data_ptr(), K, None, False, stream)
+
+    def one_rank_step(i):
+        send(i)
+        recv(0)
+        combine_send(0)
+        combine_recv(i)
+
+    def whole_step(i):
+        send(i)
+        for r in range(1, N):
+            empty_send(r)
+        for r in range(N):
+            recv(r)
+        for r in range(N):
+            combine_send(r)
+        combine_recv(i)
+
+    def wall(step_fn, n):
+        for i in range(warmup):
+            step_fn(i)
+        torch.cuda.synchronize(device)
+        t0 = time.perf_counter()
+        for i in range(n):
+            step_fn(warmup + i)
+        torch.cuda.synchronize(device)
+        dt = time.perf_counter() - t0
+        flags = ctx.status(stream)
+        if flags:
+            raise RuntimeError(f"device error flags {flags}")
+        return dt / n * 1e6
+
+    def pace(step_fn):
+        p = time_gpu_pace(wl, step_fn=step_fn)
+        return None if p is None else round(p, 2)
+
+    for i in range(min(warmup, 20)):
+        whole_step(i)               # every rank's tables exist before rank 0's calls are timed alone
+    one_wall = wall(one_rank_step, steps)
+    whole_wall = wall(whole_step, steps)
+    out = {
+        "workload": label,
+        "one_rank_step_us_wall": round(one_wall, 2),
+        "one_rank_step_us_gpu_pace": pace(one_rank_step),
+        "all_ranks_step_us_wall": round(whole_wall, 2),
+        "gpu_pace_us_of_call_sequences": {
+            "send": pace(send),
+            "send_recv": pace(lambda i: (send(i), recv(0))),
+            "send_recv_combine_send": pace(lambda i: (send(i), recv(0), combine_send(0))),
+        },
+        "note": "rank 0 holds the tokens.  one_rank_step = rank 0's send, recv, combine-send and combine-recv: "
+                "four launches; the recv is the step's first and also lays out the other receivers.  "
+                "all_ranks_step = those plus the other ranks' (empty) sends, recvs and combine-sends: 25 calls "
+                "at 8 ranks, whose wall time is the host's.  gpu_pace: the calls enqueued behind a kernel that "
+                "holds the queue, two events around 100 steps, median of 5.",
+    }
+    wl.close()
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
@@ -724,6 +820,12 @@ def main() -> int:
         split = split_calls(C3, device, args.routings, side_steps, args.warmup,
                             "DeepSeek-V3 prefill through the four split calls (send, recv, combine-send, "
                             "combine-recv), rank 0 holds the 4096 tokens")
+    split_decode = split_qwen = None
+    if not args.no_decode and not args.no_split:
+        split_decode = split_calls_small(C2, device, args.routings, side_steps, args.warmup,
+                                         decode_label + ", through the four split calls")
+        split_qwen = split_calls_small(C1, device, args.routings, side_steps, args.warmup,
+                                       qwen_label + ", through the four split calls")
     if not args.no_decode:
         decode = other_shape(C2, device, args.routings, side_steps, args.warmup, ctx_flags, decode_label)
         decode["note"] = ("working set (26 MB) fits the 256 MB Infinity Cache and is not flushed between steps; "
@@ -836,6 +938,8 @@ def main() -> int:
             },
         },
         "split_calls_4096": split,
+        "split_calls_128": split_decode,
+        "split_calls_qwen3_128": split_qwen,
         "decode_128": decode,
         "qwen3_decode_128": qwen,
         "kimi_1024": kimi,
