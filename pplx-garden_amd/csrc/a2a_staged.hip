@@ -1077,14 +1077,13 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     const PushDst &dst = args.dst;
     const uint32_t num_chunks = args.row_bytes / 16;
     const uint32_t team = args.team_waves * kWave;   // threads that share a row
-    const bool whole = team == blockDim.x;           // (uniform) the workgroup is one team: no divisions
-    const uint32_t teams = whole ? 1 : blockDim.x / team;
-    const uint32_t member = whole ? tid : tid % team;
+    const uint32_t teams = blockDim.x / team;
+    const uint32_t member = tid % team;
     const uint32_t *padded_index = st.padded_index + (size_t)r * st.max_recv;
     const uint32_t *source_row = st.source_row + (size_t)r * st.max_recv;
     // The first row's two table words are asked for together with the number of rows received
     // (a row index the tables do not hold reads entry 0 and is dropped by the loop's bound).
-    uint32_t row = blockIdx.x * teams + (whole ? 0 : tid / team);
+    uint32_t row = blockIdx.x * teams + tid / team;
     const uint32_t probe = row < st.max_recv ? row : 0;
     uint32_t dst_row = padded_index[probe];
     uint32_t from = source_row[probe];
@@ -1123,6 +1122,70 @@ __global__ __launch_bounds__(1024) void stage_recv_kernel(const StageRecvArgs ar
     }
 }
 
+// A later recv of a step with few rows: the host gave every row a workgroup as wide as the row, so a
+// workgroup is one team and has one row, seldom two; nothing is divided and no row is asked for ahead.
+__global__ __launch_bounds__(1024) void stage_recv_few_kernel(const StageRecvArgs args, const Workspace ws,
+                                                              const Staging st) {
+    // everything a wavefront takes from the argument block, asked for in one go
+    A2A_PIN(args.dst.out_x);
+    A2A_PIN(args.dst.out_scale);
+    A2A_PIN(args.dst.out_stride);
+    A2A_PIN(args.dst.os_stride_elem);
+    A2A_PIN(args.dst.os_stride_token);
+    A2A_PIN(args.dst.out_rows);
+    A2A_PIN(args.rank);
+    A2A_PIN(args.row_bytes);
+    A2A_PIN(args.hidden_dim_scale);
+    A2A_PIN(st.send_buf);
+    A2A_PIN(st.padded_index);
+    A2A_PIN(st.source_row);
+    A2A_PIN(st.num_recv);
+    A2A_PIN(st.disp_stride);
+    A2A_PIN(st.payload_bytes);
+    A2A_PIN(st.max_recv);
+    const uint32_t r = args.rank;
+    const uint32_t tid = threadIdx.x;
+    const PushDst &dst = args.dst;
+    const uint32_t num_chunks = args.row_bytes / 16;
+    const uint32_t *padded_index = st.padded_index + (size_t)r * st.max_recv;
+    const uint32_t *source_row = st.source_row + (size_t)r * st.max_recv;
+    // The row's two table words are asked for together with the number of rows received (a row
+    // index the tables do not hold reads entry 0 and is dropped by the loop's bound).
+    uint32_t row = blockIdx.x;
+    const uint32_t probe = row < st.max_recv ? row : 0;
+    uint32_t dst_row = padded_index[probe];
+    uint32_t from = source_row[probe];
+    uint32_t total = st.num_recv[2 * r];
+    if (total > st.max_recv) total = st.max_recv;   // flagged by the layout: more rows than the region was sized for
+
+    if (blockIdx.x == 0) {
+        // the receiver's counts for the caller (a2a_dispatch_recv.cu:220-224)
+        const uint32_t E = ws.num_experts, Le = ws.experts_per_rank;
+        const uint32_t first = r * Le;
+        const uint32_t n_local = first >= E ? 0 : (E - first < Le ? E - first : Le);
+        for (uint32_t le = tid; le < n_local; le += blockDim.x) {
+            const uint32_t tpe = ws.tokens_per_expert[first + le];
+            if (args.out_num_tokens != nullptr) args.out_num_tokens[le] = (int32_t)tpe;
+            if (ws.padded_offset[first + le] + tpe > dst.out_rows) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+        }
+    }
+    if (dst.out_x == nullptr) return;
+
+    while (row < total) {
+        if (dst_row >= dst.out_rows) {
+            if (tid == 0) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+        } else {
+            const uint8_t *src = st.send_buf + (size_t)from * st.disp_stride;
+            copy_received_row(src, st.payload_bytes, num_chunks, args.hidden_dim_scale, dst, dst_row, tid, blockDim.x);
+        }
+        row += gridDim.x;
+        if (row < total) {
+            dst_row = padded_index[row];
+            from = source_row[row];
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------
 // combine send: copy expert_y[padded_index[i]] to the staging row of the copy
 // it answers, i.e. row `source_position[i]` of sender `source_rank[i]`
@@ -1145,44 +1208,75 @@ __global__ __launch_bounds__(1024) void combine_send_kernel(const CombineSendArg
     A2A_PIN(st.comb_stride);
     A2A_PIN(st.max_recv);
     const uint32_t r = args.rank;
+    uint32_t total = st.num_recv[2 * r];
+    if (total > st.max_recv) total = st.max_recv;
     const uint32_t num_chunks = args.row_bytes / 16;
     const uint32_t team = args.team_waves * kWave;   // threads that share a row
-    const bool whole = team == blockDim.x;           // (uniform) the workgroup is one team: no divisions
-    const uint32_t teams = whole ? 1 : blockDim.x / team;
-    const uint32_t member = whole ? threadIdx.x : threadIdx.x % team;
+    const uint32_t teams = blockDim.x / team;
+    const uint32_t member = threadIdx.x % team;
+    for (uint32_t i = blockIdx.x * teams + threadIdx.x / team; i < total; i += gridDim.x * teams) {
+        const uint32_t row = st.padded_index[(size_t)r * st.max_recv + i];
+        // every member of the source's dp group reads the same staging rows
+        const uint32_t g = st.source_rank[(size_t)r * st.max_recv + i] / ws.dp_size;
+        const uint32_t pos = st.source_position[(size_t)r * st.max_recv + i];
+        if (row >= args.y_rows || pos >= ws.max_tk) {
+            if (member == 0) atomicOr(ws.err, A2A_DEV_BAD_SLOT);
+            continue;
+        }
+        copy_row_by_team(reinterpret_cast<const u32x4 *>(args.y + (size_t)row * args.y_stride),
+                         reinterpret_cast<u32x4 *>(st.comb_buf + ((size_t)g * ws.max_tk + pos) * st.comb_stride),
+                         num_chunks, member, team);
+    }
+}
+
+// The combine-send of a step with few rows: the host gave every row a workgroup as wide as the row, so
+// a workgroup is one team and has one row, seldom two.  The row's three table words are asked for
+// together with the number of rows received (a row index the tables do not hold reads entry 0 and is
+// dropped by the loop's bound), and nothing is divided: 128 tokens, 3.3 -> 3.1 us per launch.  (The same
+// in the kernel of the large steps made its launches at 4096 tokens 1.5 to 4 % slower.)
+__global__ __launch_bounds__(1024) void combine_send_few_kernel(const CombineSendArgs args,
+                                                                const Workspace ws, const Staging st) {
+    // everything a wavefront takes from the argument block, asked for in one go
+    A2A_PIN(args.y);
+    A2A_PIN(args.y_stride);
+    A2A_PIN(args.y_rows);
+    A2A_PIN(args.row_bytes);
+    A2A_PIN(ws.dp_size);
+    A2A_PIN(ws.max_tk);
+    A2A_PIN(st.comb_buf);
+    A2A_PIN(st.padded_index);
+    A2A_PIN(st.source_rank);
+    A2A_PIN(st.source_position);
+    A2A_PIN(st.comb_stride);
+    A2A_PIN(st.max_recv);
+    const uint32_t r = args.rank;
+    const uint32_t num_chunks = args.row_bytes / 16;
     const uint32_t *padded_index = st.padded_index + (size_t)r * st.max_recv;
     const uint32_t *source_rank = st.source_rank + (size_t)r * st.max_recv;
     const uint32_t *source_position = st.source_position + (size_t)r * st.max_recv;
-    // The first row's three table words are asked for together with the number of rows received (a
-    // row index the tables do not hold reads entry 0 and is dropped by the loop's bound).
-    uint32_t i = blockIdx.x * teams + (whole ? 0 : threadIdx.x / team);
+    uint32_t i = blockIdx.x;
     const uint32_t probe = i < st.max_recv ? i : 0;
     uint32_t row = padded_index[probe];
     uint32_t peer = source_rank[probe];
     uint32_t pos = source_position[probe];
     uint32_t total = st.num_recv[2 * r];
     if (total > st.max_recv) total = st.max_recv;
-    const uint32_t stride = gridDim.x * teams;
     while (i < total) {
-        // the next row's words travel while this one is copied
-        const uint32_t next = i + stride;
-        const uint32_t next_probe = next < total ? next : i;
-        const uint32_t next_row = padded_index[next_probe];
-        const uint32_t next_peer = source_rank[next_probe];
-        const uint32_t next_pos = source_position[next_probe];
         // every member of the source's dp group reads the same staging rows
         const uint32_t g = ws.dp_size > 1 ? peer / ws.dp_size : peer;
         if (row >= args.y_rows || pos >= ws.max_tk) {
-            if (member == 0) atomicOr(ws.err, A2A_DEV_BAD_SLOT);
+            if (threadIdx.x == 0) atomicOr(ws.err, A2A_DEV_BAD_SLOT);
         } else {
             copy_row_by_team(reinterpret_cast<const u32x4 *>(args.y + (size_t)row * args.y_stride),
                              reinterpret_cast<u32x4 *>(st.comb_buf + ((size_t)g * ws.max_tk + pos) * st.comb_stride),
-                             num_chunks, member, team);
+                             num_chunks, threadIdx.x, blockDim.x);
         }
-        i = next;
-        row = next_row;
-        peer = next_peer;
-        pos = next_pos;
+        i += gridDim.x;
+        if (i < total) {
+            row = padded_index[i];
+            peer = source_rank[i];
+            pos = source_position[i];
+        }
     }
 }
 
@@ -1468,8 +1562,13 @@ hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, con
     StageRecvArgs a = args;
     a.team_waves = l.team_waves;
     if (!first_of_step) {
-        hipExtLaunchKernelGGL(stage_recv_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, timing.start, timing.stop,
-                              0, a, ws, st);
+        if (l.team_waves * kWave == l.threads) {   // few rows: a workgroup per row
+            hipExtLaunchKernelGGL(stage_recv_few_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, timing.start,
+                                  timing.stop, 0, a, ws, st);
+        } else {
+            hipExtLaunchKernelGGL(stage_recv_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, timing.start,
+                                  timing.stop, 0, a, ws, st);
+        }
         return hipGetLastError();
     }
     // Behind the caller's workgroups: a few per other receiver, enough threads for the rows a receiver
@@ -1492,6 +1591,11 @@ hipError_t launch_combine_send(const CombineSendArgs &args, const Workspace &ws,
     const RowLaunch l = row_launch(args.max_rows, args.row_bytes / 16, ws.world);
     CombineSendArgs a = args;
     a.team_waves = l.team_waves;
+    if (l.team_waves * kWave == l.threads) {   // few rows: a workgroup per row
+        hipExtLaunchKernelGGL(combine_send_few_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, timing.start,
+                              timing.stop, 0, a, ws, st);
+        return hipGetLastError();
+    }
     hipExtLaunchKernelGGL(combine_send_kernel, dim3(l.blocks), dim3(l.threads), 0, stream, timing.start, timing.stop,
                           0, a, ws, st);
     return hipGetLastError();
