@@ -778,6 +778,9 @@ struct ReceiverTables {   // in LDS, see lay_out_receiver
     uint32_t *grp_cnt;   // [g]      rows this receiver gets from source g
     const uint8_t *order;  // [i]    the i-th source this receiver lays out
     uint32_t rows;       // rows received
+    // only with lay_out_receiver_spread (w = i * Le + le is the run of the i-th source visited and local expert le):
+    uint32_t *pos;       // [w]      position of the run in the sender's expert-sorted order (excl, by run)
+    uint32_t own_g, own_pos, own_seg, own_row;   // run w = threadIdx.x of this thread (if there is one), in registers
 };
 
 // Lays out receiver `r` in LDS.  Whole workgroup.  `publish`: this workgroup also writes the
@@ -1049,6 +1052,322 @@ __global__ __launch_bounds__(1024) void stage_recv_first_kernel(const StageRecvA
         }
         const uint8_t *src = st.send_buf + ((size_t)m.g * st.max_tokens + token) * st.disp_stride;
         copy_received_row(src, st.payload_bytes, num_chunks, args.hidden_dim_scale, dst, m.dst_row, member, team_threads);
+    }
+}
+
+// The same layout for the steps with few rows (stage_recv_first_few_kernel), where the layout is most of
+// what a recv waits for.  In the tables run_row and seg (and pos) a run is w = i * Le + le, i the
+// source's place in the order of the layout, as in lay_out_receiver.
+//
+// The work is spread over all threads, one run (source in the order of the layout, local expert)
+// each, and what counts is the number of dependent LDS trips and barriers between the arrival of the
+// counts and the first row's load (each about 0.1 us): everything that can be asked for together is,
+// reads before writes.  One wavefront doing the layout alone, in loops over the sources with one trip
+// per step, was 1.5 us of the 2.2 us a small step's recv waited for its layout.
+// After the last barrier inside, a thread's OWN runs (w = tid, tid + blockDim.x, ...) are complete in
+// LDS and the first of them is in t.own_*; `all_visible` adds the barrier after which every thread
+// may read every run.
+__device__ __forceinline__ bool lay_out_receiver_spread(uint32_t valid_mask, const Workspace &ws, const Staging &st, uint32_t r,
+                                                 bool publish, uint32_t first_row, int32_t *out_num_tokens,
+                                                 uint32_t out_rows, uint32_t *s_recv, uint8_t *s_order,
+                                                 ReceiverTables &t, bool all_visible) {
+    const uint32_t G = ws.num_groups, E = ws.num_experts, Le = ws.experts_per_rank;
+    const uint32_t first = r * Le;
+    const uint32_t n_local = first >= E ? 0 : (E - first < Le ? E - first : Le);
+    const uint32_t items = G * Le;
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nthreads = blockDim.x;
+    const uint32_t lane = tid & (kWave - 1);
+    const uint32_t wave = tid / kWave;
+    uint32_t *tot = t.tot = s_recv;
+    uint32_t *excl = t.excl = tot + items;
+    uint32_t *pos_of = t.pos = excl + items;
+    uint32_t *run_row = t.run_row = pos_of + items;
+    uint32_t *seg = t.seg = run_row + items;
+    uint32_t *grp_dst = t.grp_dst = seg + items + 1;
+    uint32_t *grp_src = t.grp_src = grp_dst + G;
+    uint32_t *grp_cnt = t.grp_cnt = grp_src + G;
+    uint32_t *poff = grp_cnt + G;   // [le] rows of a local expert, then its padded first row
+    t.order = s_order;
+
+    // The order in which this receiver lays out its sources (one byte per source, from the table the
+    // context computed once) is asked for with the counts: every thread takes the first two words (the
+    // first eight sources) for its loops over the sources, the first eight threads copy the table's row
+    // to LDS for whoever needs the i-th source with an i of its own.  All loads of a thread are asked
+    // for before the first is used, none under a condition of its own (a word that does not count is
+    // read from a valid place and dropped): waited for one by one they are a trip to memory each.
+    const uint32_t *order_row = ws.order + r * (kMaxWorld / 4);
+    const uint32_t order_lo = order_row[0], order_hi = order_row[1];
+    const uint32_t order_mine = order_row[tid & (kMaxWorld / 4 - 1)];
+    uint32_t *order_words = reinterpret_cast<uint32_t *>(s_order);
+    for (uint32_t w = tid; w < items; w += nthreads) {
+        const uint32_t g = Le > 1 ? __umulhi(w, ws.le_magic) : w;
+        const uint32_t le = w - g * Le;
+        const uint32_t e = first + le;
+        const bool live = le < n_local && (valid_mask >> g & 1);
+        const uint32_t at = live ? g * E + e : 0;
+        const uint32_t count = ws.num_routed[at];
+        const uint32_t upto = ws.expert_offsets[at > 0 ? at - 1 : 0];
+        tot[w] = live ? count : 0;
+        excl[w] = live && e > 0 ? upto : 0;
+    }
+    if (tid < (uint32_t)kMaxWorld / 4) order_words[tid] = order_mine;
+    __syncthreads();
+    const uint32_t o0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)order_lo);
+    const uint32_t o1 = (uint32_t)__builtin_amdgcn_readfirstlane((int)order_hi);
+
+    // Rows of local expert `le` from the sources visited before the i-th, and from all of them.
+    auto sums_over_sources = [&](uint32_t i, uint32_t le, uint32_t &below, uint32_t &total) {
+        below = total = 0;
+        for (uint32_t b = 0; b < G; b += 8) {
+            // eight sources at a time: their numbers are the same for every thread (scalar), their
+            // counts are asked for together
+            const uint32_t w0 = b == 0 ? o0 : (uint32_t)__builtin_amdgcn_readfirstlane((int)order_words[b / 4]);
+            const uint32_t w1 = b == 0 ? o1 : (uint32_t)__builtin_amdgcn_readfirstlane((int)order_words[b / 4 + 1]);
+            uint32_t c[8];
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u) {
+                const uint32_t g = ((u < 4 ? w0 : w1) >> (8 * (u & 3))) & 0xFFu;   // (0 past the last source)
+                c[u] = tot[g * Le + le];
+            }
+#pragma unroll
+            for (uint32_t u = 0; u < 8; ++u) {
+                if (b + u < G) total += c[u];
+                if (b + u < i) below += c[u];
+            }
+        }
+    };
+
+    // ---- first trip: everything that needs only the counts.  Run w = tid of this thread first.
+    const uint32_t w_own = tid < items ? tid : 0;
+    const uint32_t i_own = Le > 1 ? __umulhi(w_own, ws.le_magic) : w_own;
+    const uint32_t le_own = w_own - i_own * Le;
+    const bool source_lane = lane < G && n_local != 0;
+    const uint32_t last = source_lane ? lane * Le + n_local - 1 : 0;
+    const uint32_t excl_last = excl[last], tot_last = tot[last], excl_first = excl[source_lane ? lane * Le : 0];
+    const uint32_t visited = s_order[lane < G ? lane : 0];   // lane i: the i-th source in the order of the layout
+    const uint32_t g_own = s_order[i_own];
+    uint32_t below_own, total_own;
+    sums_over_sources(i_own, le_own, below_own, total_own);
+
+    // Rows this receiver gets from source g (lane g; there are at most kMaxWorld <= 64 sources): the
+    // sender's scan over its experts gives them without a sum.  Every wavefront adds them up by itself.
+    const uint32_t from_source = source_lane ? excl_last + tot_last - excl_first : 0;
+    const uint32_t from_lower = wave_inclusive_scan(from_source, lane);   // inclusive over the sources
+    const uint32_t rows = t.rows = (uint32_t)__builtin_amdgcn_readlane((int)from_lower, kWave - 1);
+    if (!publish && first_row >= rows) return false;   // uniform
+
+    // ---- second trip: the rows of the i-th source visited (lane i), the position of the own run
+    const uint32_t theirs = (uint32_t)__shfl((int)from_source, (int)visited);   // every lane takes part
+    const uint32_t pos0_own = excl[g_own * Le];
+    const uint32_t pos_own = excl[g_own * Le + le_own];
+
+    // Padded first row of every local expert: a scan over the experts, by the first wavefront, whose
+    // thread `le` has the expert's rows already (thread le is run (0, le)).  With more than 64 local
+    // experts the counts go through LDS and a barrier.
+    const uint32_t pad = ws.expert_padding;
+    const bool wide = Le > (uint32_t)kWave;   // uniform
+    if (wide) {
+        if (tid < Le) poff[tid] = total_own;
+        for (uint32_t le = tid + nthreads; le < Le; le += nthreads) {
+            uint32_t below, total;
+            sums_over_sources(0, le, below, total);
+            poff[le] = total;
+        }
+        __syncthreads();
+    }
+    if (wave == 0) {
+        uint32_t carry = 0;
+        for (uint32_t l0 = 0; l0 < Le; l0 += kWave) {
+            const uint32_t le = l0 + lane;
+            const bool mine = le < n_local;
+            const uint32_t tpe = !mine ? 0 : (wide ? poff[le] : total_own);
+            const uint32_t padded = pad > 1 ? (tpe + pad - 1) / pad * pad : tpe;
+            const uint32_t scan = wave_inclusive_scan(padded, lane);
+            const uint32_t mine_off = carry + scan - padded;
+            if (le < Le) poff[le] = mine_off;
+            if (mine && publish) {
+                const uint32_t e = first + le;
+                ws.tokens_per_expert[e] = tpe;
+                ws.padded_offset[e] = mine_off;
+                if (out_num_tokens != nullptr) out_num_tokens[le] = (int32_t)tpe;
+                if (mine_off + tpe > out_rows) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+            }
+            carry += (uint32_t)__builtin_amdgcn_readlane((int)scan, kWave - 1);
+        }
+    }
+
+    // Arrival order: sources as the worker visits them, local experts inside a source.  Lane i of every
+    // wavefront has the rows of the i-th source visited and those that arrive before them.
+    const uint32_t arrive = lane < G ? theirs : 0;
+    const uint32_t before = wave_inclusive_scan(arrive, lane) - arrive;
+    // ---- third trip: the own run's source in that order
+    const uint32_t base_own = (uint32_t)__shfl((int)before, (int)i_own);    // every lane takes part
+    const uint32_t count_own = (uint32_t)__shfl((int)arrive, (int)i_own);
+    const uint32_t seg_own = base_own + (le_own < n_local ? pos_own - pos0_own : count_own);
+    t.own_g = g_own;
+    t.own_pos = pos_own;
+    t.own_seg = seg_own;
+
+    // ---- writes
+    if (tid < items) {
+        seg[tid] = seg_own;
+        pos_of[tid] = pos_own;
+    }
+    if (wave == 0 && lane < G) {
+        // Per source: where its rows for this receiver begin in its own send order (dst_group_offset,
+        // a2a_worker.rs:571-575) and how many rows the lower-numbered sources send here
+        // (src_group_offset, a2a_worker.rs:582-590: numeric order, not the order of arrival).
+        grp_dst[lane] = excl_first;
+        grp_cnt[lane] = from_source;
+        grp_src[lane] = from_lower - from_source;
+    }
+    if (tid == 0) {
+        seg[items] = rows;
+        if (publish) {
+            if (rows > st.max_recv) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+            st.num_recv[2 * r] = rows;
+        }
+    }
+    // the runs beyond the first of a thread (more runs than threads): the same, one at a time
+    for (uint32_t w0 = nthreads; w0 < items; w0 += nthreads) {
+        const uint32_t w = w0 + tid;
+        const bool real = w < items;
+        const uint32_t wc = real ? w : 0;
+        const uint32_t i = Le > 1 ? __umulhi(wc, ws.le_magic) : wc;
+        const uint32_t le = wc - i * Le;
+        uint32_t below, total;
+        sums_over_sources(i, le, below, total);
+        const uint32_t g = s_order[i];
+        const uint32_t p0 = excl[g * Le];
+        const uint32_t p = excl[g * Le + le];
+        const uint32_t base = (uint32_t)__shfl((int)before, (int)i);    // every lane takes part
+        const uint32_t count = (uint32_t)__shfl((int)arrive, (int)i);
+        if (real) {
+            run_row[w] = below;
+            seg[w] = base + (le < n_local ? p - p0 : count);
+            pos_of[w] = p;
+        }
+    }
+    __syncthreads();
+
+    // First row of every run: behind the rows of the expert from the sources visited earlier.
+    t.own_row = below_own + poff[le_own];
+    if (tid < items) {
+        run_row[tid] = t.own_row;
+        if (publish && le_own < n_local) ws.slot_base[g_own * E + first + le_own] = t.own_row;
+    }
+    for (uint32_t w = tid + nthreads; w < items; w += nthreads) {
+        const uint32_t i = Le > 1 ? __umulhi(w, ws.le_magic) : w;
+        const uint32_t le = w - i * Le;
+        const uint32_t row = run_row[w] + poff[le];
+        run_row[w] = row;
+        if (publish && le < n_local) ws.slot_base[(uint32_t)s_order[i] * E + first + le] = row;
+    }
+    if (publish && tid == 0) {
+        // rows that come from other nodes (num_efa_tokens, a2a_worker.rs:681-687)
+        const uint32_t remote_segs = (ws.world / ws.node_size - 1) * (ws.node_size / ws.dp_size) * Le;
+        st.num_recv[2 * r + 1] = remote_segs < items ? seg[remote_segs] : rows;
+    }
+    if (all_visible) __syncthreads();
+    return true;
+}
+
+// What the spread tables say of arrival `row` of run `s` (seg[s] <= row < seg[s + 1]): one LDS trip.
+__device__ __forceinline__ RowMeta row_of_run_spread(const ReceiverTables &t, const Workspace &ws, uint32_t s, uint32_t row) {
+    const uint32_t Le = ws.experts_per_rank;
+    const uint32_t i = Le > 1 ? __umulhi(s, ws.le_magic) : s;
+    RowMeta m;
+    m.g = t.order[i];
+    const uint32_t j = row - t.seg[s];
+    m.pos = t.pos[s] + j;
+    m.dst_row = t.run_row[s] + j;
+    return m;
+}
+
+// The step's first recv when the step has few rows (the host gave every row a workgroup as wide as the
+// row): the same work as stage_recv_first_kernel with the layout spread over the threads, and the
+// whole workgroup serves one row at a time: the thread whose run holds the row says so to the others.
+// Dynamic LDS: 5 * G * Le + 1 + 3 * G + Le words.
+__global__ __launch_bounds__(1024) void stage_recv_first_few_kernel(const StageRecvArgs args, const Workspace ws,
+                                                                    const Staging st) {
+    extern __shared__ uint32_t s_recv[];
+    __shared__ __align__(16) uint8_t s_order[kMaxWorld];
+    __shared__ uint32_t s_meta[3];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t nthreads = blockDim.x;
+    const uint32_t items = ws.num_groups * ws.experts_per_rank;
+    ReceiverTables t;
+
+    if (blockIdx.x >= args.copy_blocks) {
+        // ---- one of the other receivers: layout, then one thread per received row ----
+        const uint32_t w = blockIdx.x - args.copy_blocks;
+        uint32_t r = w / args.slices;
+        const uint32_t slice = w - r * args.slices;
+        if (r >= args.rank) ++r;   // the caller's rank is served by the first workgroups
+        if (!lay_out_receiver_spread(args.valid_mask, ws, st, r, slice == 0, slice * nthreads, nullptr, 0xFFFFFFFFu,
+                                     s_recv, s_order, t, true))
+            return;
+        const uint32_t total = t.rows < st.max_recv ? t.rows : st.max_recv;   // beyond: flagged and dropped
+        for (uint32_t row = slice * nthreads + tid; row < total; row += args.slices * nthreads) {
+            // the run this arrival belongs to: the last one with seg[s] <= row (runs without rows share
+            // their first arrival with the run after them, so the last such run is the one with rows)
+            uint32_t lo = 0, hi = items;   // seg[lo] <= row < seg[hi]
+            while (hi - lo > 1) {
+                const uint32_t mid = (lo + hi) / 2;
+                if (t.seg[mid] <= row) lo = mid; else hi = mid;
+            }
+            const RowMeta m = row_of_run_spread(t, ws, lo, row);
+            // the token behind the position: asked for first, used last
+            const uint32_t token = m.pos < ws.max_tk ? st.pos_token[(size_t)m.g * ws.max_tk + m.pos] : 0;
+            write_row_tables(t, ws, st, r, row, m, args.max_private);
+            st.source_row[(size_t)r * st.max_recv + row] = m.g * st.max_tokens + token;
+        }
+        return;
+    }
+
+    // ---- the caller's rank: layout, then the workgroup's row ----
+    const uint32_t r = args.rank;
+    const PushDst &dst = args.dst;
+    const uint32_t num_chunks = args.row_bytes / 16;
+    if (!lay_out_receiver_spread(args.valid_mask, ws, st, r, blockIdx.x == 0, blockIdx.x, args.out_num_tokens,
+                                 args.dst.out_rows, s_recv, s_order, t, false))
+        return;
+    const uint32_t own_end = t.seg[tid < items ? tid + 1 : 0];   // where the run after this thread's first begins
+    for (uint32_t row = blockIdx.x; row < t.rows; row += args.copy_blocks) {
+        if (row != blockIdx.x) __syncthreads();   // the row before this one has been taken from s_meta
+        if (tid < items && t.own_seg <= row && row < own_end) {   // in the thread's first run: all in registers
+            s_meta[0] = t.own_g;
+            s_meta[1] = t.own_pos + (row - t.own_seg);
+            s_meta[2] = t.own_row + (row - t.own_seg);
+        }
+        for (uint32_t w = tid + nthreads; w < items; w += nthreads) {
+            // (a thread's own runs are complete, and every run's first arrival is there)
+            if (t.seg[w] <= row && row < t.seg[w + 1]) {
+                const RowMeta mine = row_of_run_spread(t, ws, w, row);
+                s_meta[0] = mine.g;
+                s_meta[1] = mine.pos;
+                s_meta[2] = mine.dst_row;
+            }
+        }
+        __syncthreads();
+        RowMeta m;
+        m.g = s_meta[0];
+        m.pos = s_meta[1];
+        m.dst_row = s_meta[2];
+        if (row >= st.max_recv) continue;   // flagged by the layout: more rows than the receive region was sized for
+        const uint32_t token = st.pos_token[(size_t)m.g * ws.max_tk + m.pos];
+        if (tid == 0) {
+            write_row_tables(t, ws, st, r, row, m, args.max_private);
+            st.source_row[(size_t)r * st.max_recv + row] = m.g * st.max_tokens + token;
+        }
+        if (dst.out_x == nullptr) continue;
+        if (m.dst_row >= dst.out_rows) {
+            if (tid == 0) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+            continue;
+        }
+        const uint8_t *src = st.send_buf + ((size_t)m.g * st.max_tokens + token) * st.disp_stride;
+        copy_received_row(src, st.payload_bytes, num_chunks, args.hidden_dim_scale, dst, m.dst_row, tid, nthreads);
     }
 }
 
@@ -1579,7 +1898,14 @@ hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, con
     if (a.slices < 1) a.slices = 1;
     if (a.slices > 16) a.slices = 16;
     const uint32_t blocks = l.blocks + (ws.world - 1) * a.slices;
-    const size_t lds = (4 * (size_t)ws.num_groups * ws.experts_per_rank + 1 + 3 * (size_t)ws.num_groups) * sizeof(uint32_t);
+    const size_t items = (size_t)ws.num_groups * ws.experts_per_rank;
+    if (l.team_waves * kWave == l.threads) {   // few rows: a workgroup per row
+        const size_t lds = (5 * items + 1 + 3 * (size_t)ws.num_groups + ws.experts_per_rank) * sizeof(uint32_t);
+        hipExtLaunchKernelGGL(stage_recv_first_few_kernel, dim3(blocks), dim3(l.threads), lds, stream, timing.start,
+                              timing.stop, 0, a, ws, st);
+        return hipGetLastError();
+    }
+    const size_t lds = (4 * items + 1 + 3 * (size_t)ws.num_groups) * sizeof(uint32_t);
     hipExtLaunchKernelGGL(stage_recv_first_kernel, dim3(blocks), dim3(l.threads), lds, stream, timing.start,
                           timing.stop, 0, a, ws, st);
     return hipGetLastError();
