@@ -2,6 +2,7 @@
 #include "a2a_staged.h"
 
 #include <cstring>
+#include <type_traits>
 
 #include "a2a_device.h"
 #include "a2a_scan.h"
@@ -424,25 +425,42 @@ __global__ __launch_bounds__(1024) void stage_send_quick_kernel(const StageSendA
     // Scan over the experts (a2a_dispatch_send.cu:236-242), 64 at a time; a route whose expert lies in
     // the 64 at hand takes the expert's word and the entries of the experts before it from the lane
     // that holds them.  Token 0 publishes.
+    // Up to four passes of 64 experts at a time: their reads, scans and lane exchanges do not depend
+    // on each other, only the running total does (256 experts: 3.6 -> 3.4 us per send against one pass
+    // at a time; a step with 128 experts takes two at a time, with four it was 0.1 us slower).
     uint32_t run = 0, my_word = 0, my_excl = 0;
-    for (uint32_t e0 = 0; e0 < E; e0 += kWave) {
-        const uint32_t x = e0 + lane;
-        const uint32_t word = x < E ? s_cnt[x] : 0;
-        const uint32_t c = word & 0xFFFFu;
-        const uint32_t incl = run + wave_inclusive_scan(c, lane);
-        if (token == 0 && x < E) {
-            ws.num_routed[g * E + x] = c;
-            ws.expert_offsets[g * E + x] = incl;
+    auto passes = [&](uint32_t e0, auto width) {
+        constexpr uint32_t W = decltype(width)::value;
+        uint32_t word[W], incl[W];
+#pragma unroll
+        for (uint32_t u = 0; u < W; ++u) {
+            const uint32_t x = e0 + u * kWave + lane;
+            word[u] = s_cnt[x < E ? x : 0];
+            if (x >= E) word[u] = 0;
         }
-        const uint32_t rel = my_id - e0;   // (an id below e0 wraps around to a large number)
-        const uint32_t their_word = (uint32_t)__shfl((int)word, (int)(rel & (kWave - 1)));   // every lane takes part
-        const uint32_t their_excl = (uint32_t)__shfl((int)(incl - c), (int)(rel & (kWave - 1)));
-        if (rel < (uint32_t)kWave) {
-            my_word = their_word;
-            my_excl = their_excl;
+#pragma unroll
+        for (uint32_t u = 0; u < W; ++u) incl[u] = wave_inclusive_scan(word[u] & 0xFFFFu, lane);
+#pragma unroll
+        for (uint32_t u = 0; u < W; ++u) {
+            const uint32_t x = e0 + u * kWave + lane;
+            const uint32_t c = word[u] & 0xFFFFu;
+            const uint32_t rel = my_id - (e0 + u * kWave);   // (an id below the pass wraps around to a large number)
+            const uint32_t their_word = (uint32_t)__shfl((int)word[u], (int)(rel & (kWave - 1)));   // every lane takes part
+            const uint32_t their_excl = (uint32_t)__shfl((int)(incl[u] - c), (int)(rel & (kWave - 1)));
+            if (rel < (uint32_t)kWave) {
+                my_word = their_word;
+                my_excl = run + their_excl;
+            }
+            if (token == 0 && x < E) {
+                ws.num_routed[g * E + x] = c;
+                ws.expert_offsets[g * E + x] = run + incl[u];
+            }
+            run += (uint32_t)__builtin_amdgcn_readlane((int)incl[u], kWave - 1);
         }
-        run = (uint32_t)__builtin_amdgcn_readlane((int)incl, kWave - 1);
-    }
+    };
+    uint32_t e0 = 0;
+    for (; e0 + 2 * kWave < E; e0 += 4 * kWave) passes(e0, std::integral_constant<uint32_t, 4>{});
+    if (e0 < E) passes(e0, std::integral_constant<uint32_t, 2>{});
     if (!live) return;   // past bound_m: no positions to write (uniform)
     if (lane < K) {
         uint32_t toff = 0;
@@ -780,7 +798,7 @@ struct ReceiverTables {   // in LDS, see lay_out_receiver
     uint32_t rows;       // rows received
     // only with lay_out_receiver_spread (w = i * Le + le is the run of the i-th source visited and local expert le):
     uint32_t *pos;       // [w]      position of the run in the sender's expert-sorted order (excl, by run)
-    uint32_t own_g, own_pos, own_seg, own_row;   // run w = threadIdx.x of this thread (if there is one), in registers
+    uint32_t own_g, own_pos, own_seg, own_end, own_row;   // run w = threadIdx.x of this thread (if there is one), in registers
 };
 
 // Lays out receiver `r` in LDS.  Whole workgroup.  `publish`: this workgroup also writes the
@@ -1139,16 +1157,21 @@ __device__ __forceinline__ bool lay_out_receiver_spread(uint32_t valid_mask, con
     };
 
     // ---- first trip: everything that needs only the counts.  Run w = tid of this thread first.
+    // (A wavefront none of whose threads has a run skips what only runs need: what every wavefront
+    // of a workgroup executes costs the SIMDs they share as much time as what one executes alone.)
+    const bool has_runs = tid - lane < items;   // the same for a whole wavefront
     const uint32_t w_own = tid < items ? tid : 0;
     const uint32_t i_own = Le > 1 ? __umulhi(w_own, ws.le_magic) : w_own;
     const uint32_t le_own = w_own - i_own * Le;
     const bool source_lane = lane < G && n_local != 0;
     const uint32_t last = source_lane ? lane * Le + n_local - 1 : 0;
     const uint32_t excl_last = excl[last], tot_last = tot[last], excl_first = excl[source_lane ? lane * Le : 0];
-    const uint32_t visited = s_order[lane < G ? lane : 0];   // lane i: the i-th source in the order of the layout
-    const uint32_t g_own = s_order[i_own];
-    uint32_t below_own, total_own;
-    sums_over_sources(i_own, le_own, below_own, total_own);
+    uint32_t visited = 0, g_own = 0, below_own = 0, total_own = 0;
+    if (has_runs) {
+        visited = s_order[lane < G ? lane : 0];   // lane i: the i-th source in the order of the layout
+        g_own = s_order[i_own];
+        sums_over_sources(i_own, le_own, below_own, total_own);
+    }
 
     // Rows this receiver gets from source g (lane g; there are at most kMaxWorld <= 64 sources): the
     // sender's scan over its experts gives them without a sum.  Every wavefront adds them up by itself.
@@ -1157,10 +1180,14 @@ __device__ __forceinline__ bool lay_out_receiver_spread(uint32_t valid_mask, con
     const uint32_t rows = t.rows = (uint32_t)__builtin_amdgcn_readlane((int)from_lower, kWave - 1);
     if (!publish && first_row >= rows) return false;   // uniform
 
-    // ---- second trip: the rows of the i-th source visited (lane i), the position of the own run
-    const uint32_t theirs = (uint32_t)__shfl((int)from_source, (int)visited);   // every lane takes part
-    const uint32_t pos0_own = excl[g_own * Le];
-    const uint32_t pos_own = excl[g_own * Le + le_own];
+    // ---- second trip: the rows of the i-th source visited (lane i), the position and rows of the own run
+    uint32_t theirs = 0, pos0_own = 0, pos_own = 0, tot_own = 0;
+    if (has_runs) {
+        theirs = (uint32_t)__shfl((int)from_source, (int)visited);   // every lane of the wavefront takes part
+        pos0_own = excl[g_own * Le];
+        pos_own = excl[g_own * Le + le_own];
+        tot_own = tot[g_own * Le + le_own];
+    }
 
     // Padded first row of every local expert: a scan over the experts, by the first wavefront, whose
     // thread `le` has the expert's rows already (thread le is run (0, le)).  With more than 64 local
@@ -1199,15 +1226,19 @@ __device__ __forceinline__ bool lay_out_receiver_spread(uint32_t valid_mask, con
 
     // Arrival order: sources as the worker visits them, local experts inside a source.  Lane i of every
     // wavefront has the rows of the i-th source visited and those that arrive before them.
-    const uint32_t arrive = lane < G ? theirs : 0;
-    const uint32_t before = wave_inclusive_scan(arrive, lane) - arrive;
-    // ---- third trip: the own run's source in that order
-    const uint32_t base_own = (uint32_t)__shfl((int)before, (int)i_own);    // every lane takes part
-    const uint32_t count_own = (uint32_t)__shfl((int)arrive, (int)i_own);
-    const uint32_t seg_own = base_own + (le_own < n_local ? pos_own - pos0_own : count_own);
+    uint32_t arrive = 0, before = 0, seg_own = 0;
+    if (has_runs) {
+        arrive = lane < G ? theirs : 0;
+        before = wave_inclusive_scan(arrive, lane) - arrive;
+        // ---- third trip: the own run's source in that order
+        const uint32_t base_own = (uint32_t)__shfl((int)before, (int)i_own);    // every lane of the wavefront takes part
+        const uint32_t count_own = (uint32_t)__shfl((int)arrive, (int)i_own);
+        seg_own = base_own + (le_own < n_local ? pos_own - pos0_own : count_own);
+    }
     t.own_g = g_own;
     t.own_pos = pos_own;
     t.own_seg = seg_own;
+    t.own_end = seg_own + tot_own;   // (the run after this one begins where this one's rows end)
 
     // ---- writes
     if (tid < items) {
@@ -1299,12 +1330,16 @@ __global__ __launch_bounds__(1024) void stage_recv_first_few_kernel(const StageR
     const uint32_t items = ws.num_groups * ws.experts_per_rank;
     ReceiverTables t;
 
-    if (blockIdx.x >= args.copy_blocks) {
+    // The workgroups of the other receivers come first in the grid: their chain (layout, run and token
+    // of every row, the row's tables) is as long as the calling rank's (layout, row, copy), and started
+    // behind its workgroups they were what the kernel's end waited for (0.15 us).
+    const uint32_t other_blocks = gridDim.x - args.copy_blocks;
+    if (blockIdx.x < other_blocks) {
         // ---- one of the other receivers: layout, then one thread per received row ----
-        const uint32_t w = blockIdx.x - args.copy_blocks;
+        const uint32_t w = blockIdx.x;
         uint32_t r = w / args.slices;
         const uint32_t slice = w - r * args.slices;
-        if (r >= args.rank) ++r;   // the caller's rank is served by the first workgroups
+        if (r >= args.rank) ++r;   // the caller's rank is served by the workgroups behind these
         if (!lay_out_receiver_spread(args.valid_mask, ws, st, r, slice == 0, slice * nthreads, nullptr, 0xFFFFFFFFu,
                                      s_recv, s_order, t, true))
             return;
@@ -1330,13 +1365,13 @@ __global__ __launch_bounds__(1024) void stage_recv_first_few_kernel(const StageR
     const uint32_t r = args.rank;
     const PushDst &dst = args.dst;
     const uint32_t num_chunks = args.row_bytes / 16;
-    if (!lay_out_receiver_spread(args.valid_mask, ws, st, r, blockIdx.x == 0, blockIdx.x, args.out_num_tokens,
+    const uint32_t block = blockIdx.x - other_blocks;
+    if (!lay_out_receiver_spread(args.valid_mask, ws, st, r, block == 0, block, args.out_num_tokens,
                                  args.dst.out_rows, s_recv, s_order, t, false))
         return;
-    const uint32_t own_end = t.seg[tid < items ? tid + 1 : 0];   // where the run after this thread's first begins
-    for (uint32_t row = blockIdx.x; row < t.rows; row += args.copy_blocks) {
-        if (row != blockIdx.x) __syncthreads();   // the row before this one has been taken from s_meta
-        if (tid < items && t.own_seg <= row && row < own_end) {   // in the thread's first run: all in registers
+    for (uint32_t row = block; row < t.rows; row += args.copy_blocks) {
+        if (row != block) __syncthreads();   // the row before this one has been taken from s_meta
+        if (tid < items && t.own_seg <= row && row < t.own_end) {   // in the thread's first run: all in registers
             s_meta[0] = t.own_g;
             s_meta[1] = t.own_pos + (row - t.own_seg);
             s_meta[2] = t.own_row + (row - t.own_seg);
@@ -1361,13 +1396,14 @@ __global__ __launch_bounds__(1024) void stage_recv_first_few_kernel(const StageR
             write_row_tables(t, ws, st, r, row, m, args.max_private);
             st.source_row[(size_t)r * st.max_recv + row] = m.g * st.max_tokens + token;
         }
-        if (dst.out_x == nullptr) continue;
-        if (m.dst_row >= dst.out_rows) {
-            if (tid == 0) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
-            continue;
+        if (dst.out_x != nullptr) {
+            if (m.dst_row >= dst.out_rows) {
+                if (tid == 0) atomicOr(ws.err, A2A_DEV_RECV_OVERFLOW);
+            } else {
+                const uint8_t *src = st.send_buf + ((size_t)m.g * st.max_tokens + token) * st.disp_stride;
+                copy_received_row(src, st.payload_bytes, num_chunks, args.hidden_dim_scale, dst, m.dst_row, tid, nthreads);
+            }
         }
-        const uint8_t *src = st.send_buf + ((size_t)m.g * st.max_tokens + token) * st.disp_stride;
-        copy_received_row(src, st.payload_bytes, num_chunks, args.hidden_dim_scale, dst, m.dst_row, tid, nthreads);
     }
 }
 
