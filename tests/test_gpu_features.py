@@ -114,7 +114,7 @@ def test_quantiser_on_nan_infinity_and_the_largest_bf16_value(repeat, split):
 
 
 @pytest.mark.parametrize("split", [False, True], ids=["group", "split"])
-@pytest.mark.parametrize("case", [C0, scaled(C0, 1200)], ids=["one_launch", "two_launch"])
+@pytest.mark.parametrize("case", [C0, scaled(C0, 700), scaled(C0, 1200)], ids=["one_launch", "one_launch_mid_size", "two_launch"])
 def test_bound_m_limits_the_tokens(case, split):
     world = make_world(case, "all")
     bounds = [case.num_tokens, 0, 17, 1]

@@ -48,6 +48,13 @@ QUICK_SENDS = [
     (96, 15360, 64, 4, 4, 1, "ragged", False),        # 960 pieces a row: sixteen wavefronts, the resolver is the last
     (40, 16384, 64, 4, 4, 1, "ragged", False),        # a piece too many for a spare wavefront: the kernel without one
     (300, 512, 96, 2, 6, 4, "all", True),             # entries beyond what the threads ask for at the head
+    # steps of 448 to 1024 tokens: a workgroup per two to four tokens, teams of wavefronts and a spare one
+    (700, 7168, 384, 16, 8, 128, "one", False),       # three tokens a workgroup, two teams, two rounds
+    (1024, 2048, 128, 8, 8, 1, "all", True),          # four teams, one round
+    (600, 7168, 250, 8, 5, 8, "ragged", True),
+    (512, 15360, 64, 4, 4, 1, "ragged", False),       # one team of fifteen wavefronts, two rounds
+    (600, 512, 96, 2, 12, 4, "all", True),            # 48 routes a workgroup
+    (1000, 256, 40, 1, 3, 1, "all", False),           # one rank
 ]
 
 
@@ -56,7 +63,8 @@ QUICK_SENDS = [
                               for t, h, e, n, k, p, s, rep in QUICK_SENDS])
 def test_quick_send_of_small_steps(tokens, hidden, experts, ranks, topk, pad, sources, repeats, device):
     """The send of a small step with dense index rows takes a kernel in which a spare wavefront per token
-    scans the counts and writes the token's positions while the others quantise and stage the row.  One
+    scans the counts and writes the token's positions while the others quantise and stage the row (a
+    step of 448 to 1024 tokens: a spare wavefront per workgroup of two to four tokens).  One
     token, experts that do not fill the scan's passes, many passes, more routes than a wavefront's
     eighth, rows of sixteen wavefronts, entries beyond the first batch, tokens that name an expert
     twice: rows, scales and the routing tables are the oracle's, bit for bit."""
