@@ -236,9 +236,11 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
     if (lane < K) {
         expert = (uint32_t)dst.indices[(size_t)token * dst.indices_stride + lane];
         weight = dst.weights[(size_t)token * dst.weights_stride + lane];
-        slot = args.staged_base != nullptr
-                   ? ws.token_offset[(size_t)group * ws.max_tk + token * K + lane]
-                   : ws.route_slot[(size_t)group * ws.max_tk + token * K + lane];
+        // (after a group dispatch: the copy's row in its receiver's buffer; after the sends of the split
+        // calls: its position in the sender's expert-sorted order, a2a_combine_recv.cu:67-73 = exclusive
+        // offset of the expert + token offset, which the send wrote here so that no second, dependent
+        // look-up stands in front of the rows: 0.5 us of a 128-token combine-recv)
+        slot = ws.route_slot[(size_t)group * ws.max_tk + token * K + lane];
     }
     const bool expert_ok = expert < E;
     const uint32_t r = expert_ok ? owner_of_expert(ws, expert) : 0;
@@ -249,15 +251,9 @@ __global__ __launch_bounds__(kCombineWaves * kWave) void combine_gather_kernel(c
     if (lane < K) {
         bool ok = false;
         if (args.staged_base != nullptr) {
-            // a2a_combine_recv.cu:67-73: position = exclusive offset of the expert + token offset.
-            if (expert_ok) {
-                const uint32_t excl = expert > 0 ? ws.expert_offsets[group * E + expert - 1] : 0;
-                const uint32_t pos = excl + slot;
-                if (pos < ws.max_tk) {
-                    row_ptr = (uint64_t)(args.staged_base +
-                                         ((size_t)group * ws.max_tk + pos) * args.staged_stride);
-                    ok = true;
-                }
+            if (expert_ok && slot < ws.max_tk) {
+                row_ptr = (uint64_t)(args.staged_base + ((size_t)group * ws.max_tk + slot) * args.staged_stride);
+                ok = true;
             }
         } else if (expert_ok && r_base != 0 && slot < r_rows) {
             row_ptr = r_base + (uint64_t)slot * r_stride;

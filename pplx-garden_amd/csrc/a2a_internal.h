@@ -29,7 +29,8 @@ struct Workspace {
     uint32_t *slot_base;       // [N][E]         first receiver row of (source, expert)
     uint32_t *tokens_per_expert;  // [E]         per receiver-local expert, summed over sources
     uint32_t *padded_offset;   // [E]            first row of an expert inside its receiver
-    uint32_t *route_slot;      // [N][max_tk]    receiver row of every copy (kInvalidSlot if dropped)
+    uint32_t *route_slot;      // [N][max_tk]    receiver row of every copy (kInvalidSlot if dropped); after the sends of
+                               //                the split calls: the copy's position in its sender's expert-sorted order
     uint32_t *token_offset;    // [N][max_tk]    rank of every copy inside its (source, expert)
     uint32_t *err;             // [1]            A2A_DEV_* bits, sticky
     const uint32_t *order;     // [N][8] words   byte i of receiver r's row: the i-th source it lays out

@@ -86,15 +86,17 @@ __global__ __launch_bounds__(1024) void stage_send_kernel(const StageSendArgs ar
     if (wave == 0 && lane < K) {
         const uint32_t entry = token * K + lane;
         const uint32_t expert = (uint32_t)src.indices[(size_t)token * src.indices_stride + lane];
-        uint32_t toff = 0;
+        uint32_t toff = 0, at = kInvalidSlot;
         if (expert < E) {
             toff = ws.block_prefix[((size_t)g * ws.nb_max + entry / kRouteBlock) * E + expert] +
                    ws.local_rank[(size_t)g * ws.max_tk + entry];
             // position of the copy (a2a_dispatch_send.cu:54)
             const uint32_t excl = expert > 0 ? ws.expert_offsets[g * E + expert - 1] : 0;
-            st.pos_token[(size_t)g * ws.max_tk + excl + toff] = token;
+            at = excl + toff;
+            st.pos_token[(size_t)g * ws.max_tk + at] = token;
         }
         ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
+        ws.route_slot[(size_t)g * ws.max_tk + entry] = at;   // (the combine-recv of the step reads the position here)
     }
     stage_row<QUANT>(args, st, g, token, blockDim.x);
 }
@@ -236,15 +238,17 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
         }
         if (lane < K) {
             const uint32_t entry = token * K + lane;
-            uint32_t toff = 0;
+            uint32_t toff = 0, at = kInvalidSlot;
             if (my_expert < E) {
                 toff = prior[my_expert] + repeats;
                 // position of the copy (a2a_dispatch_send.cu:54)
-                st.pos_token[(size_t)g * ws.max_tk + excl[my_expert] + toff] = token;
+                at = excl[my_expert] + toff;
+                st.pos_token[(size_t)g * ws.max_tk + at] = token;
             } else {
                 atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
             }
             ws.token_offset[(size_t)g * ws.max_tk + entry] = toff;
+            ws.route_slot[(size_t)g * ws.max_tk + entry] = at;
         }
     }
     stage_row<QUANT, true>(args, st, g, token, nthreads, pre_a, pre_b);
@@ -463,15 +467,17 @@ __global__ __launch_bounds__(1024) void stage_send_quick_kernel(const StageSendA
     if (e0 < E) passes(e0, std::integral_constant<uint32_t, 2>{});
     if (!live) return;   // past bound_m: no positions to write (uniform)
     if (lane < K) {
-        uint32_t toff = 0;
+        uint32_t toff = 0, at = kInvalidSlot;
         if (my_id < E) {
             toff = (my_word >> 16) + repeats;
             // position of the copy (a2a_dispatch_send.cu:54)
-            st.pos_token[(size_t)g * ws.max_tk + my_excl + toff] = token;
+            at = my_excl + toff;
+            st.pos_token[(size_t)g * ws.max_tk + at] = token;
         } else {
             atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
         }
         ws.token_offset[(size_t)g * ws.max_tk + my_first + lane] = toff;
+        ws.route_slot[(size_t)g * ws.max_tk + my_first + lane] = at;
     }
 }
 
@@ -593,16 +599,18 @@ __global__ __launch_bounds__(1024) void stage_send_single_kernel(const StageSend
     // One thread per route of my tokens: its rank inside its expert and the row of the sender's
     // expert-sorted order it stands for (a2a_dispatch_send.cu:54).
     if (tid < my_routes && my_first + tid < flat_entries) {
-        uint32_t toff = 0;
+        uint32_t toff = 0, at = kInvalidSlot;
         if (my_expert < E) {
             uint32_t earlier = 0;
             for (uint32_t q = 0; q < tid; ++q) earlier += s_route_expert[q] == my_expert ? 1u : 0u;
             toff = (cnt[my_expert] >> 16) + earlier;
-            st.pos_token[(size_t)g * ws.max_tk + excl[my_expert] + toff] = first_token + tid / K;
+            at = excl[my_expert] + toff;
+            st.pos_token[(size_t)g * ws.max_tk + at] = first_token + tid / K;
         } else {
             atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
         }
         ws.token_offset[(size_t)g * ws.max_tk + my_first + tid] = toff;
+        ws.route_slot[(size_t)g * ws.max_tk + my_first + tid] = at;
     }
 
     // The teams stage one token each per round.
@@ -835,16 +843,18 @@ __global__ __launch_bounds__(1024) void stage_send_teams_kernel(const StageSendA
     if (e0 < E) passes(e0, std::integral_constant<uint32_t, 2>{});
 
     if (route_live) {
-        uint32_t toff = 0;
+        uint32_t toff = 0, at = kInvalidSlot;
         if (my_id < E) {
             toff = (my_word >> 16) + earlier;
             // position of the copy (a2a_dispatch_send.cu:54)
             const uint32_t token = first_token + (K > 1 ? __umulhi(lane, args.topk_magic) : lane);
-            st.pos_token[(size_t)g * ws.max_tk + my_excl + toff] = token;
+            at = my_excl + toff;
+            st.pos_token[(size_t)g * ws.max_tk + at] = token;
         } else {
             atomicOr(ws.err, A2A_DEV_BAD_EXPERT_ID);
         }
         ws.token_offset[(size_t)g * ws.max_tk + my_first + lane] = toff;
+        ws.route_slot[(size_t)g * ws.max_tk + my_first + lane] = at;
     }
 }
 
@@ -937,13 +947,15 @@ __global__ __launch_bounds__(1024) void stage_send_resolve_kernel(const StageSen
             earlier = group8_sum(earlier);
             excl = group8_sum(excl);
             if (part == 0 && in) {
-                uint32_t toff = 0;
+                uint32_t toff = 0, at = kInvalidSlot;
                 if (live) {
                     toff = earlier + local;
                     // position of the copy (a2a_dispatch_send.cu:54)
-                    st.pos_token[(size_t)g * ws.max_tk + excl + toff] = token;
+                    at = excl + toff;
+                    st.pos_token[(size_t)g * ws.max_tk + at] = token;
                 }
                 ws.token_offset[(size_t)g * ws.max_tk + token * K + k] = toff;
+                ws.route_slot[(size_t)g * ws.max_tk + token * K + k] = at;
             }
         }
     }
