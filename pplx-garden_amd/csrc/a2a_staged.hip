@@ -2,7 +2,6 @@
 #include "a2a_staged.h"
 
 #include <cstring>
-#include <type_traits>
 
 #include "a2a_device.h"
 #include "a2a_scan.h"
@@ -254,6 +253,59 @@ __global__ __launch_bounds__(1024) void stage_send_small_kernel(const StageSendA
     stage_row<QUANT, true>(args, st, g, token, nthreads, pre_a, pre_b);
 }
 
+// The scan over a sender's per-expert counts (a2a_dispatch_send.cu:236-242) by ONE wavefront, for the
+// sends in which a spare wavefront resolves positions.  `s_cnt[e]`: low half of a word the entries of
+// expert e.  W passes of 64 experts at a time: their reads, scans and lane exchanges do not depend on
+// each other, only the running total `run` does.  A lane whose route's expert `my_id` lies in a pass
+// takes the expert's word and the entries of the experts before it from the lane that holds them; with
+// `publish` the counts and their inclusive scan go to memory.  Whole wavefront.
+template <uint32_t W>
+__device__ __forceinline__ void scan_counts_passes(const uint32_t *s_cnt, uint32_t E, uint32_t e0, uint32_t lane,
+                                                   uint32_t my_id, bool publish, uint32_t *num_routed,
+                                                   uint32_t *expert_offsets, uint32_t &run, uint32_t &my_word,
+                                                   uint32_t &my_excl) {
+    uint32_t word[W], incl[W];
+#pragma unroll
+    for (uint32_t u = 0; u < W; ++u) {
+        const uint32_t x = e0 + u * kWave + lane;
+        word[u] = s_cnt[x < E ? x : 0];
+        if (x >= E) word[u] = 0;
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < W; ++u) incl[u] = wave_inclusive_scan(word[u] & 0xFFFFu, lane);
+#pragma unroll
+    for (uint32_t u = 0; u < W; ++u) {
+        const uint32_t x = e0 + u * kWave + lane;
+        const uint32_t c = word[u] & 0xFFFFu;
+        const uint32_t rel = my_id - (e0 + u * kWave);   // (an id below the pass wraps around to a large number)
+        const uint32_t their_word = (uint32_t)__shfl((int)word[u], (int)(rel & (kWave - 1)));   // every lane takes part
+        const uint32_t their_excl = (uint32_t)__shfl((int)(incl[u] - c), (int)(rel & (kWave - 1)));
+        if (rel < (uint32_t)kWave) {
+            my_word = their_word;
+            my_excl = run + their_excl;
+        }
+        if (publish && x < E) {
+            num_routed[x] = c;
+            expert_offsets[x] = run + incl[u];
+        }
+        run += (uint32_t)__builtin_amdgcn_readlane((int)incl[u], kWave - 1);
+    }
+}
+
+// The whole scan: four passes at a time while more than two are left, then two (256 experts: 3.6 ->
+// 3.4 us per send of 128 tokens against one pass at a time; a step with 128 experts takes two at a
+// time, with four it was 0.1 us slower).
+__device__ __forceinline__ void scan_counts_for_routes(const uint32_t *s_cnt, uint32_t E, uint32_t lane, uint32_t my_id,
+                                                       bool publish, uint32_t *num_routed, uint32_t *expert_offsets,
+                                                       uint32_t &my_word, uint32_t &my_excl) {
+    uint32_t run = 0, e0 = 0;
+    my_word = my_excl = 0;
+    for (; e0 + 2 * kWave < E; e0 += 4 * kWave) {
+        scan_counts_passes<4>(s_cnt, E, e0, lane, my_id, publish, num_routed, expert_offsets, run, my_word, my_excl);
+    }
+    if (e0 < E) scan_counts_passes<2>(s_cnt, E, e0, lane, my_id, publish, num_routed, expert_offsets, run, my_word, my_excl);
+}
+
 // The quick form of the one-launch send of a small step: dense index rows and a row that is one piece
 // per thread (16 elements to quantise, or 16 bytes to move as they are) with a wavefront to spare (the
 // host launches one more than the row has pieces for).  Where a row is staged does not depend on the
@@ -426,45 +478,11 @@ __global__ __launch_bounds__(1024) void stage_send_quick_kernel(const StageSendA
     __builtin_amdgcn_s_setprio(3);
     asm volatile("" ::: "memory");
 
-    // Scan over the experts (a2a_dispatch_send.cu:236-242), 64 at a time; a route whose expert lies in
-    // the 64 at hand takes the expert's word and the entries of the experts before it from the lane
-    // that holds them.  Token 0 publishes.
-    // Up to four passes of 64 experts at a time: their reads, scans and lane exchanges do not depend
-    // on each other, only the running total does (256 experts: 3.6 -> 3.4 us per send against one pass
-    // at a time; a step with 128 experts takes two at a time, with four it was 0.1 us slower).
-    uint32_t run = 0, my_word = 0, my_excl = 0;
-    auto passes = [&](uint32_t e0, auto width) {
-        constexpr uint32_t W = decltype(width)::value;
-        uint32_t word[W], incl[W];
-#pragma unroll
-        for (uint32_t u = 0; u < W; ++u) {
-            const uint32_t x = e0 + u * kWave + lane;
-            word[u] = s_cnt[x < E ? x : 0];
-            if (x >= E) word[u] = 0;
-        }
-#pragma unroll
-        for (uint32_t u = 0; u < W; ++u) incl[u] = wave_inclusive_scan(word[u] & 0xFFFFu, lane);
-#pragma unroll
-        for (uint32_t u = 0; u < W; ++u) {
-            const uint32_t x = e0 + u * kWave + lane;
-            const uint32_t c = word[u] & 0xFFFFu;
-            const uint32_t rel = my_id - (e0 + u * kWave);   // (an id below the pass wraps around to a large number)
-            const uint32_t their_word = (uint32_t)__shfl((int)word[u], (int)(rel & (kWave - 1)));   // every lane takes part
-            const uint32_t their_excl = (uint32_t)__shfl((int)(incl[u] - c), (int)(rel & (kWave - 1)));
-            if (rel < (uint32_t)kWave) {
-                my_word = their_word;
-                my_excl = run + their_excl;
-            }
-            if (token == 0 && x < E) {
-                ws.num_routed[g * E + x] = c;
-                ws.expert_offsets[g * E + x] = run + incl[u];
-            }
-            run += (uint32_t)__builtin_amdgcn_readlane((int)incl[u], kWave - 1);
-        }
-    };
-    uint32_t e0 = 0;
-    for (; e0 + 2 * kWave < E; e0 += 4 * kWave) passes(e0, std::integral_constant<uint32_t, 4>{});
-    if (e0 < E) passes(e0, std::integral_constant<uint32_t, 2>{});
+    // Scan over the experts; a route takes its expert's word and the entries of the experts before it.
+    // Token 0 publishes.
+    uint32_t my_word, my_excl;
+    scan_counts_for_routes(s_cnt, E, lane, my_id, token == 0, ws.num_routed + g * E, ws.expert_offsets + g * E, my_word,
+                           my_excl);
     if (!live) return;   // past bound_m: no positions to write (uniform)
     if (lane < K) {
         uint32_t toff = 0, at = kInvalidSlot;
@@ -805,42 +823,11 @@ __global__ __launch_bounds__(1024) void stage_send_teams_kernel(const StageSendA
     __builtin_amdgcn_s_setprio(3);
     asm volatile("" ::: "memory");
 
-    // Scan over the experts (a2a_dispatch_send.cu:236-242), two or four passes of 64 at a time; a
-    // route whose expert lies in a pass takes the expert's word and the entries of the experts before
-    // it from the lane that holds them.  The first workgroup publishes.
-    uint32_t run = 0, my_word = 0, my_excl = 0;
-    auto passes = [&](uint32_t e0, auto width) {
-        constexpr uint32_t W = decltype(width)::value;
-        uint32_t word[W], incl[W];
-#pragma unroll
-        for (uint32_t u = 0; u < W; ++u) {
-            const uint32_t x = e0 + u * kWave + lane;
-            word[u] = s_cnt[x < E ? x : 0];
-            if (x >= E) word[u] = 0;
-        }
-#pragma unroll
-        for (uint32_t u = 0; u < W; ++u) incl[u] = wave_inclusive_scan(word[u] & 0xFFFFu, lane);
-#pragma unroll
-        for (uint32_t u = 0; u < W; ++u) {
-            const uint32_t x = e0 + u * kWave + lane;
-            const uint32_t c = word[u] & 0xFFFFu;
-            const uint32_t rel = my_id - (e0 + u * kWave);   // (an id below the pass wraps around to a large number)
-            const uint32_t their_word = (uint32_t)__shfl((int)word[u], (int)(rel & (kWave - 1)));   // every lane takes part
-            const uint32_t their_excl = (uint32_t)__shfl((int)(incl[u] - c), (int)(rel & (kWave - 1)));
-            if (rel < (uint32_t)kWave) {
-                my_word = their_word;
-                my_excl = run + their_excl;
-            }
-            if (blockIdx.x == 0 && x < E) {
-                ws.num_routed[g * E + x] = c;
-                ws.expert_offsets[g * E + x] = run + incl[u];
-            }
-            run += (uint32_t)__builtin_amdgcn_readlane((int)incl[u], kWave - 1);
-        }
-    };
-    uint32_t e0 = 0;
-    for (; e0 + 2 * kWave < E; e0 += 4 * kWave) passes(e0, std::integral_constant<uint32_t, 4>{});
-    if (e0 < E) passes(e0, std::integral_constant<uint32_t, 2>{});
+    // Scan over the experts; a route takes its expert's word and the entries of the experts before it.
+    // The first workgroup publishes.
+    uint32_t my_word, my_excl;
+    scan_counts_for_routes(s_cnt, E, lane, my_id, blockIdx.x == 0, ws.num_routed + g * E, ws.expert_offsets + g * E,
+                           my_word, my_excl);
 
     if (route_live) {
         uint32_t toff = 0, at = kInvalidSlot;
