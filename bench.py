@@ -704,6 +704,8 @@ def main() -> int:
     ap.add_argument("--cpu-reps", type=int, default=3, help="repetitions of the CPU baseline (0 = skip)")
     ap.add_argument("--no-decode", action="store_true", help="skip the shapes other than the 4096-token one")
     ap.add_argument("--no-split", action="store_true", help="skip the pass through the four split calls")
+    ap.add_argument("--split-small-only", action="store_true",
+                    help="time only the four split calls at the two decode shapes (for a kernel trace of them alone)")
     ap.add_argument("--split-only", action="store_true",
                     help="time only the four split calls at the headline's shape (for a kernel trace of them alone)")
     ap.add_argument("--decode-only", action="store_true",
@@ -759,6 +761,13 @@ def main() -> int:
                   "receive slots padded to 128 per expert")
     others = {"decode_128": (C2, decode_label, None), "qwen3_decode_128": (C1, qwen_label, None),
               "kimi_1024": (C4, kimi_label, 37.0)}
+    if args.split_small_only:
+        print(json.dumps({
+            "split_calls_128_only": split_calls_small(C2, device, args.routings, side_steps, args.warmup,
+                                                      decode_label + ", through the four split calls"),
+            "split_calls_qwen3_128_only": split_calls_small(C1, device, args.routings, side_steps, args.warmup,
+                                                            qwen_label + ", through the four split calls")}))
+        return 0
     if args.split_only:
         print(json.dumps({"split_calls_4096_only": split_calls(
             C3, device, args.routings, side_steps, args.warmup,
