@@ -600,7 +600,8 @@ def split_calls(case, device, routings: int, steps: int, warmup: int, label: str
 
 
 def split_calls_small(case, device, routings: int, steps: int, warmup: int, label: str):
-    """The four split calls at a step of a few microseconds (a decode shape), rank 0 holding the tokens:
+    """The four split calls at a step of a few tens of microseconds at most (a decode shape, the
+    1024-token mixed batch), rank 0 holding the tokens:
     wall time of a loop of steps and the GPU's own pace (the steps enqueued behind a kernel that holds the
     queue), for rank 0's four calls (what a rank on a GPU of its own runs) and for the calls of the whole
     group, and the pace of the sequences send / send + recv / send + recv + combine-send, whose
@@ -684,8 +685,8 @@ def split_calls_small(case, device, routings: int, steps: int, warmup: int, labe
         },
         "note": "rank 0 holds the tokens.  one_rank_step = rank 0's send, recv, combine-send and combine-recv: "
                 "four launches; the recv is the step's first and also lays out the other receivers.  "
-                "all_ranks_step = those plus the other ranks' (empty) sends, recvs and combine-sends: 25 calls "
-                "at 8 ranks, whose wall time is the host's.  gpu_pace: the calls enqueued behind a kernel that "
+                "all_ranks_step = those plus the other ranks' (empty) sends, recvs and combine-sends: 3 N + 1 "
+                "calls for N ranks, whose wall time is mostly the host's.  gpu_pace: the calls enqueued behind a kernel that "
                 "holds the queue, two events around 100 steps, median of 5.",
     }
     wl.close()
@@ -766,7 +767,9 @@ def main() -> int:
             "split_calls_128_only": split_calls_small(C2, device, args.routings, side_steps, args.warmup,
                                                       decode_label + ", through the four split calls"),
             "split_calls_qwen3_128_only": split_calls_small(C1, device, args.routings, side_steps, args.warmup,
-                                                            qwen_label + ", through the four split calls")}))
+                                                            qwen_label + ", through the four split calls"),
+            "split_calls_kimi_1024_only": split_calls_small(C4, device, args.routings, side_steps, args.warmup,
+                                                            kimi_label + ", through the four split calls")}))
         return 0
     if args.split_only:
         print(json.dumps({"split_calls_4096_only": split_calls(
@@ -829,12 +832,14 @@ def main() -> int:
         split = split_calls(C3, device, args.routings, side_steps, args.warmup,
                             "DeepSeek-V3 prefill through the four split calls (send, recv, combine-send, "
                             "combine-recv), rank 0 holds the 4096 tokens")
-    split_decode = split_qwen = None
+    split_decode = split_qwen = split_kimi = None
     if not args.no_decode and not args.no_split:
         split_decode = split_calls_small(C2, device, args.routings, side_steps, args.warmup,
                                          decode_label + ", through the four split calls")
         split_qwen = split_calls_small(C1, device, args.routings, side_steps, args.warmup,
                                        qwen_label + ", through the four split calls")
+        split_kimi = split_calls_small(C4, device, args.routings, side_steps, args.warmup,
+                                       kimi_label + ", through the four split calls")
     if not args.no_decode:
         decode = other_shape(C2, device, args.routings, side_steps, args.warmup, ctx_flags, decode_label)
         decode["note"] = ("working set (26 MB) fits the 256 MB Infinity Cache and is not flushed between steps; "
@@ -949,6 +954,7 @@ def main() -> int:
         "split_calls_4096": split,
         "split_calls_128": split_decode,
         "split_calls_qwen3_128": split_qwen,
+        "split_calls_kimi_1024": split_kimi,
         "decode_128": decode,
         "qwen3_decode_128": qwen,
         "kimi_1024": kimi,
