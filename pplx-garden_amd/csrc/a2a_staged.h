@@ -26,6 +26,7 @@ struct Staging {
     void *arena = nullptr;
     uint8_t *send_buf = nullptr;         // [N][max_num_tokens][disp_stride]: payload, scales, 16 spare bytes (+ padding to whole lines)
     uint32_t *pos_token = nullptr;       // [N][max_tk]: token behind each row of a sender's expert-sorted order
+                                         // (the other way round, copy -> position, is in the workspace's route_slot)
     uint8_t *comb_buf = nullptr;         // [N][max_tk][comb_stride]: combine rows at the sender's positions
     uint32_t *padded_index = nullptr;    // [N][max_recv]
     uint32_t *source_rank = nullptr;     // [N][max_recv]
@@ -93,12 +94,15 @@ const uint32_t *staging_table(const Staging &st, const a2a_config &cfg, uint32_t
 
 hipError_t launch_stage_send(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                              bool quantize, hipStream_t stream, KernelTiming timing = KernelTiming());
-// One-launch send (routing counted inside) for small steps: whether a step qualifies, and the launch.
+// One-launch send (routing counted inside) for small steps: whether a step qualifies, and the launch
+// (dense index rows and a wavefront to spare: the kernel in which a spare wavefront resolves the
+// positions while the others stage the row; otherwise the one in which every wavefront does both).
 bool stage_send_small_fits(const StageSendArgs &args, const Workspace &ws);
 hipError_t launch_stage_send_small(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                                    bool quantize, hipStream_t stream, KernelTiming timing = KernelTiming());
 // One-launch send for steps of up to 8192 entries that are too large for the small-step kernel
-// (a workgroup counts once for several tokens): whether a step qualifies, and the launch.
+// (a workgroup counts once for several tokens): whether a step qualifies, and the launch (with a
+// wavefront to spare, again the kernel in which it resolves the positions beside the teams).
 bool stage_send_single_fits(const StageSendArgs &args, const Workspace &ws, bool quantize);
 hipError_t launch_stage_send_single(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                                     bool quantize, hipStream_t stream, KernelTiming timing = KernelTiming());
@@ -106,6 +110,7 @@ hipError_t launch_stage_send_single(const StageSendArgs &args, const Workspace &
 hipError_t launch_stage_send_resolve(const StageSendArgs &args, const Workspace &ws, const Staging &st,
                                      bool quantize, hipStream_t stream, KernelTiming timing = KernelTiming());
 // `first_of_step`: no recv has run since the step's sends; this launch also lays out the other receivers.
+// Steps with few rows (a workgroup per row) take kernels of their own, here and in the combine-send.
 hipError_t launch_stage_recv(const StageRecvArgs &args, const Workspace &ws, const Staging &st, bool first_of_step,
                              hipStream_t stream, KernelTiming timing = KernelTiming());
 hipError_t launch_combine_send(const CombineSendArgs &args, const Workspace &ws, const Staging &st,
